@@ -1,0 +1,208 @@
+/*
+ * legion_mi.h -- C ABI of the MI355X sampling-server hot path.
+ *
+ * One opaque server object per GPU.  Batch in: seed node ids.  Batch out:
+ * multi-hop sampled blocks (block CSR + the reference's COO view) plus the
+ * gathered feature rows, all resident in HBM and described by the reference's
+ * two 16-int headers.  Plain pointers and sizes only; every entry point returns
+ * 0 on success or a negative LMI_ERR_* code, with text from lmi_last_error().
+ *
+ * Each declaration names the Legion-IBP interface it stands in for (paths are
+ * relative to that tree).  The reference's own `extern "C"` functions take C++
+ * object pointers (UnifiedCache*, MemoryPool*, ...) and abort the process on
+ * error; here the objects live behind the handle and errors are returned.
+ *
+ * Threading: a server is not thread-safe; use one server per GPU from one host
+ * thread (reference: one std::thread per GPU, engine/server.cu:127-135).  Work
+ * is enqueued on the caller's stream and is asynchronous unless stated.
+ * `stream` arguments are hipStream_t values passed as void* (NULL = the default
+ * stream).  Output buffers are owned by the server and borrowed by the caller
+ * until the same pipe is used for another batch (engine/server.cu:337,377).
+ */
+#ifndef LEGION_MI_H
+#define LEGION_MI_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define LMI_ABI_VERSION 1
+#define LMI_MAX_HOPS    3   /* the 16-int headers hold 3 hops (INTRABATCH_CON, include/system_config.cuh:47-57) */
+#define LMI_MAX_FANOUT  64  /* one wavefront lane per slot; the reference asserts <= 32 (operator_impl.cu:504) */
+#define LMI_MAX_PIPES   4   /* output buffer sets; the reference uses INTERBATCH_CON = 2 */
+
+enum {
+  LMI_OK = 0,
+  LMI_ERR_ARG = -1,      /* bad argument / wrong call order */
+  LMI_ERR_HIP = -2,      /* a HIP runtime call failed */
+  LMI_ERR_STATE = -3,    /* required object (graph, features, cache) not loaded */
+  LMI_ERR_CAPACITY = -4, /* request exceeds configured capacity */
+  LMI_ERR_BAD_ID = -5    /* a seed id outside [0, n_nodes) was seen on the device */
+};
+
+enum { LMI_F32 = 0, LMI_F16 = 1 };                       /* feature element type */
+enum { LMI_LOC_HOST = 0, LMI_LOC_DEVICE = 1 };           /* where an input pointer lives */
+enum { LMI_MODE_TRAIN = 0, LMI_MODE_VALID = 1, LMI_MODE_TEST = 2 }; /* TRAINMODE.. (include/system_config.cuh) */
+enum { LMI_TABLE_HASH = 0, LMI_TABLE_DIRECT = 1 };       /* id->slot table layout */
+enum { LMI_CACHE_NONE = 0, LMI_CACHE_STATIC = 1, LMI_CACHE_LRU = 2, LMI_CACHE_INT8 = 3 };
+
+typedef struct lmi_server lmi_server;
+
+/* Replaces the positional ./meta_config line + argv of the reference
+ * (storage/storage_management.cu:33-104, main.cu:9-14). */
+typedef struct lmi_config {
+  int32_t  device_id;
+  int32_t  batch_size;              /* max seeds per batch */
+  int32_t  hops;                    /* 1..LMI_MAX_HOPS */
+  int32_t  fanout[LMI_MAX_HOPS];    /* per hop, 1..LMI_MAX_FANOUT */
+  int32_t  feat_dim;                /* elements per feature row */
+  int32_t  feat_dtype;              /* LMI_F32 | LMI_F16 */
+  int32_t  pipes;                   /* 1..LMI_MAX_PIPES output buffer sets */
+  int32_t  reserved;
+  uint64_t seed;                    /* default RNG seed (per-batch seeds may override) */
+} lmi_config;
+
+/* Device pointers of one pipe's outputs: the reference's per-pipe MemoryPool /
+ * IPC buffers (engine/memorypool.cuh:20-221, engine/ipc_service.cu:140-206) plus
+ * the block-CSR row pointers.  Row i of `features` belongs to ids[i].  Edges of
+ * hop k (1-based) are agg_*[edge_counter[12+k] .. +edge_counter[9+k]) in local
+ * ids; block k has node_counter[9+k] sources and node_counter[9+k-1]
+ * destinations (training_backend/ipc_service.cpp:61-68). */
+typedef struct lmi_batch_view {
+  int32_t *ids;                       /* [max_nodes] global ids, local-id order */
+  void    *features;                  /* [max_nodes][feat_dim] feat_dtype */
+  int32_t *labels;                    /* [batch_size] (-1 when no labels loaded) */
+  int32_t *agg_src_ids;               /* [max_edges] sampled neighbours, global ids */
+  int32_t *agg_src_off;               /* [max_edges] COO source, local ids */
+  int32_t *agg_dst_off;               /* [max_edges] COO destination, local ids */
+  int32_t *node_counter;              /* [16] */
+  int32_t *edge_counter;              /* [16] */
+  int32_t *blk_indptr[LMI_MAX_HOPS];  /* hop k: [n_{k-1}+1] row pointers into hop k's edge segment */
+  int32_t *cache_index;               /* [max_nodes] cache slot per row, -1 = miss */
+  int64_t  max_nodes, max_edges;
+} lmi_batch_view;
+
+typedef struct lmi_cache_info {
+  int32_t kind;                /* LMI_CACHE_* */
+  int32_t table_kind;          /* LMI_TABLE_* (static / int8) */
+  int64_t capacity_rows;
+  int64_t row_bytes;           /* bytes of one cached row */
+  int64_t table_bytes;         /* id->slot table footprint */
+  int64_t n_sets; int32_t ways; int32_t lru_tick;
+} lmi_cache_info;
+
+/* Per-kernel device time, measured with HIP events on the launching stream. */
+typedef struct lmi_profile {
+  double  gather_hit_ms;   int64_t gather_hit_launches;  int64_t gather_hit_rows;
+  double  gather_miss_ms;  int64_t gather_miss_launches; int64_t gather_miss_rows;
+  double  sample_ms;       int64_t sample_launches;      /* all kernels of the sampling hops */
+  double  lookup_ms;       int64_t lookup_launches;
+  double  batch_ms;        int64_t batches;              /* whole lmi_run_once */
+} lmi_profile;
+
+/* ---- lifecycle ------------------------------------------------------- */
+int         lmi_abi_version(void);
+const char *lmi_last_error(void);                               /* thread-local text */
+/* Server::Initialize + Runner::Initialize (engine/server.cu:48-92,178-301) */
+int lmi_server_create(const lmi_config *cfg, lmi_server **out);
+/* Server::Finalize / Runner::Finalize (engine/server.cu:137-170,402-451) */
+int lmi_server_destroy(lmi_server *s);
+
+/* ---- memory helpers (engine/server_imp.cuh:2-52) ---------------------- */
+int lmi_host_alloc(size_t bytes, void **host_ptr);             /* host_alloc_space: pinned + mapped */
+int lmi_host_free(void *host_ptr);
+int lmi_device_alloc(size_t bytes, void **dev_ptr);            /* d_alloc_space */
+int lmi_device_free(void *dev_ptr);                            /* d_free_space */
+int lmi_copy_to_host(void *host_dst, const void *dev_src, size_t bytes);   /* d_copy_2_h (synchronous) */
+int lmi_copy_to_device(void *dev_dst, const void *host_src, size_t bytes); /* synchronous */
+int lmi_stream_create(void **stream);
+int lmi_stream_destroy(void *stream);
+int lmi_stream_sync(void *stream);
+int lmi_device_sync(void);
+
+/* ---- storage ---------------------------------------------------------- */
+/* GraphStorage::Build (storage/graph_storage.cu:12-73): CSR with int64 row
+ * pointers and int32 neighbour ids.  LMI_LOC_HOST copies into HBM;
+ * LMI_LOC_DEVICE borrows caller-owned HBM (must outlive the server). */
+int lmi_graph_load(lmi_server *s, const int64_t *indptr, const int32_t *indices,
+                   int64_t n_nodes, int64_t n_edges, int location);
+/* FeatureStorage::Build (storage/feature_storage.cu:18-90): row-major table,
+ * row v = features of node v.  LMI_LOC_HOST must come from lmi_host_alloc and is
+ * read zero-copy by the device on cache misses; LMI_LOC_DEVICE = table in HBM. */
+int lmi_features_attach(lmi_server *s, const void *rows, int64_t n_rows, int location);
+/* Training / validation / testing id sets and labels (storage_management.cu:124-279);
+ * labels may be NULL.  Always copied into HBM. */
+int lmi_idset_load(lmi_server *s, int mode, const int32_t *ids, const int32_t *labels,
+                   int64_t n, int location);
+
+/* ---- caches (UnifiedCache::FillUp, cache/cache.cu:559-656) -------------- */
+/* Static hot-set cache: the capacity_rows nodes ranked first by (out-degree
+ * descending, id ascending). */
+int lmi_cache_build_static(lmi_server *s, int64_t capacity_rows, int table_kind);
+/* LRU dynamic cache, set-associative (comp_cache/static_cache.cu:20-113), starts empty. */
+int lmi_cache_build_lru(lmi_server *s, int64_t n_sets, int32_t ways);
+/* Compressed cache: int8 rows + per-row fp32 scale, dequantised in the gather
+ * (stands in for StaticCache::insert_features_compressed, static_cache.cu:498-612). */
+int lmi_cache_build_int8(lmi_server *s, int64_t capacity_rows, int table_kind);
+int lmi_cache_info_get(lmi_server *s, lmi_cache_info *out);
+/* Test/diagnostic read-back: slot of every node (-1 = not cached), synchronous.
+ * For the LRU cache `aux` (may be NULL) receives last_use per slot and slot_of is
+ * indexed by slot and receives the key stored there. */
+int lmi_cache_dump(lmi_server *s, int32_t *slot_of, int64_t n, int32_t *aux);
+
+/* ---- operators (engine/operator_impl.cuh:11-69, engine/operator.h:27-35) -- */
+/* BatchGenerate: stage the seeds as local ids 0..n-1.  seeds == NULL takes slice
+ * `batch_counter` of the id set `mode` (batch_generate, operator_impl.cu:28-56);
+ * otherwise `n` caller seeds at `seeds_location`.  rng_seed 0 = cfg.seed + batch_counter. */
+int lmi_op_batch_generate(lmi_server *s, int pipe, void *stream, const int32_t *seeds, int32_t n,
+                          int seeds_location, int32_t batch_counter, int mode, uint64_t rng_seed);
+/* RandomSample for hop `hop` (0-based): sample, dedup, relabel, update headers
+ * (random_sample + construct_graph + counter_update, operator_impl.cu:178-317,440-553). */
+int lmi_op_random_sample(lmi_server *s, int pipe, void *stream, int hop);
+/* FeatureCacheLookup for segment `segment`: 0 = seeds, k = nodes added by hop k
+ * (FindFeat + FeatCacheLookup, cache/cache.cu:314-338,743-803). */
+int lmi_op_cache_lookup(lmi_server *s, int pipe, void *stream, int segment);
+/* IOSubmit: empty in the reference too (operator_impl.cu:578-595). */
+int lmi_op_io_submit(lmi_server *s, int pipe, void *stream);
+/* IOComplete (operator_impl.cu:607-636): end of batch; inserts this batch's
+ * misses into the LRU cache. */
+int lmi_op_io_complete(lmi_server *s, int pipe, void *stream);
+/* Runner::RunOnce (engine/server.cu:330-400): the whole operator chain with one
+ * gather over all rows. */
+int lmi_run_once(lmi_server *s, int pipe, void *stream, const int32_t *seeds, int32_t n,
+                 int seeds_location, int32_t batch_counter, int mode, uint64_t rng_seed);
+
+/* ---- outputs ----------------------------------------------------------- */
+int lmi_batch_view_get(lmi_server *s, int pipe, lmi_batch_view *out);
+/* Synchronises `stream`, copies both headers to the host, reports a bad seed id. */
+int lmi_batch_counters(lmi_server *s, int pipe, void *stream, int32_t node_counter[16],
+                       int32_t edge_counter[16]);
+/* Steps per epoch of an id set: ceil(size / batch_size) (engine/ipc_service.cu:60-128). */
+int lmi_steps_per_epoch(lmi_server *s, int mode, int32_t *steps);
+
+/* ---- measurement ------------------------------------------------------- */
+int lmi_profile_enable(lmi_server *s, int on);   /* on: record HIP events around kernels */
+int lmi_profile_read(lmi_server *s, lmi_profile *out, int reset);  /* synchronises the device */
+/* Tuning knobs by name (e.g. "gather_lanes_per_row", "gather_unroll", "lds_dedup"). */
+int lmi_tune(lmi_server *s, const char *key, int64_t value);
+/* Plain device copy of `bytes` bytes, repeated; returns mean ms per copy
+ * (the measured HBM ceiling quoted beside the nominal peak). */
+int lmi_bench_copy(size_t bytes, int repeats, double *ms_per_copy);
+
+/* ---- synthetic inputs (stand-in for the reference's dataset tooling) ---- */
+/* Power-law graph generated in HBM: degree(v) by inverse-CDF lookup of a Philox
+ * word in `cdf` (host array of uint32 thresholds), neighbours uniform (mode 0) or
+ * degree-proportional (mode 1).  The caller owns the returned device arrays. */
+int lmi_synth_graph(uint64_t seed, const uint32_t *cdf, int32_t cdf_len, int64_t n_nodes,
+                    int32_t mode, int64_t **d_indptr, int32_t **d_indices, int64_t *n_edges);
+int lmi_synth_trainset(uint64_t seed, int64_t n_nodes, int32_t n_train, int32_t *host_ids);
+/* N(0,1) rows written straight into (pinned) host or device memory by the GPU. */
+int lmi_synth_features(uint64_t seed, void *rows, int64_t n_rows, int32_t dim, int32_t dtype);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* LEGION_MI_H */

@@ -1,0 +1,580 @@
+// C ABI of the sampling-server hot path (see include/legion_mi.h).
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+#include <new>
+
+#include "common.hpp"
+
+namespace lmi {
+
+static thread_local char g_err[512] = "";
+
+void set_error(const char *fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+}
+
+// ------------------------------------------------------------ profiling
+constexpr int kProfRing = 8192;
+
+static hipEvent_t prof_event(Server *s) {
+  if (!s->prof_free.empty()) {
+    hipEvent_t e = s->prof_free.back();
+    s->prof_free.pop_back();
+    return e;
+  }
+  hipEvent_t e = nullptr;
+  (void)hipEventCreate(&e);
+  return e;
+}
+
+int prof_begin(Server *s, hipStream_t st, int kind) {
+  if (!s->prof_on) return -1;
+  EventPair p{prof_event(s), prof_event(s), kind};
+  (void)hipEventRecord(p.a, st);
+  s->prof_events.push_back(p);
+  return (int)s->prof_events.size() - 1;
+}
+
+int prof_end(Server *s, hipStream_t st, int handle) {
+  if (handle < 0) return LMI_OK;
+  (void)hipEventRecord(s->prof_events[handle].b, st);
+  return LMI_OK;
+}
+
+static void prof_snapshot(Server *s, Pipe &p, hipStream_t st) {
+  if (!s->prof_on || s->prof_ring_n >= kProfRing) return;
+  (void)hipMemcpyAsync(&s->prof_ring[s->prof_ring_n++], p.st, sizeof(DevState), hipMemcpyDeviceToHost, st);
+}
+
+static int check_pipe(Server *s, int pipe) {
+  if (!s) LMI_FAIL(LMI_ERR_ARG, "null server");
+  if (pipe < 0 || pipe >= (int)s->pipes.size()) LMI_FAIL(LMI_ERR_ARG, "pipe %d out of range", pipe);
+  return LMI_OK;
+}
+
+template <typename T>
+static int dmalloc(T **p, int64_t count) {
+  LMI_HIP(hipMalloc((void **)p, (size_t)std::max<int64_t>(count, 1) * sizeof(T)));
+  return LMI_OK;
+}
+
+static void pipe_free(Pipe &p) {
+  void *ptrs[] = {p.ids, p.features, p.labels, p.agg_src_ids, p.agg_src_off, p.agg_dst_off, p.blk_indptr[0],
+                  p.blk_indptr[1], p.blk_indptr[2], p.cache_index, p.st, p.dedup.slots, p.eslot, p.firstv,
+                  p.cnt, p.rank, p.tile_sums, p.hit_list, p.miss_list, p.lru_fill};
+  for (void *q : ptrs)
+    if (q) (void)hipFree(q);
+  if (p.side) (void)hipStreamDestroy(p.side);
+  if (p.fork) (void)hipEventDestroy(p.fork);
+  if (p.join) (void)hipEventDestroy(p.join);
+  p = Pipe{};
+}
+
+static int pipe_alloc(Server *s, Pipe &p) {
+  LMI_TRY(dmalloc(&p.ids, s->max_nodes));
+  LMI_HIP(hipMalloc(&p.features, (size_t)s->max_nodes * s->row_bytes));
+  LMI_TRY(dmalloc(&p.labels, s->cfg.batch_size));
+  LMI_TRY(dmalloc(&p.agg_src_ids, s->max_edges));
+  LMI_TRY(dmalloc(&p.agg_src_off, s->max_edges));
+  LMI_TRY(dmalloc(&p.agg_dst_off, s->max_edges));
+  for (int k = 0; k < s->cfg.hops; ++k) LMI_TRY(dmalloc(&p.blk_indptr[k], s->node_cap[k] + 1));
+  LMI_TRY(dmalloc(&p.cache_index, s->max_nodes));
+  LMI_TRY(dmalloc(&p.st, 1));
+  LMI_HIP(hipMemset(p.st, 0, sizeof(DevState)));
+  int lg = 4;
+  while ((int64_t(1) << lg) < 2 * s->max_nodes) ++lg;
+  p.dedup.log2cap = lg;
+  LMI_HIP(hipMalloc(&p.dedup.slots, size_t(8) << lg));
+  LMI_TRY(dmalloc(&p.eslot, s->max_edges_hop));
+  LMI_TRY(dmalloc(&p.firstv, s->max_edges_hop));
+  const int64_t scan_n = std::max(s->max_nodes, s->max_edges_hop);
+  LMI_TRY(dmalloc(&p.cnt, scan_n + 1));
+  LMI_TRY(dmalloc(&p.rank, s->max_edges_hop + 1));
+  LMI_TRY(dmalloc(&p.tile_sums, ceil_div(scan_n, 2048) + 1));
+  LMI_TRY(dmalloc(&p.hit_list, s->max_nodes));
+  LMI_TRY(dmalloc(&p.miss_list, s->max_nodes));
+  LMI_TRY(dmalloc(&p.lru_fill, s->max_nodes));
+  LMI_HIP(hipStreamCreateWithFlags(&p.side, hipStreamNonBlocking));
+  LMI_HIP(hipEventCreateWithFlags(&p.fork, hipEventDisableTiming));
+  LMI_HIP(hipEventCreateWithFlags(&p.join, hipEventDisableTiming));
+  return LMI_OK;
+}
+
+static __global__ void copy_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
+    dst[i] = src[i];
+}
+
+}  // namespace lmi
+
+using namespace lmi;
+
+extern "C" {
+
+int lmi_abi_version(void) { return LMI_ABI_VERSION; }
+const char *lmi_last_error(void) { return g_err; }
+
+int lmi_server_create(const lmi_config *cfg, lmi_server **out) {
+  if (!cfg || !out) LMI_FAIL(LMI_ERR_ARG, "null argument");
+  if (cfg->hops < 1 || cfg->hops > LMI_MAX_HOPS) LMI_FAIL(LMI_ERR_ARG, "hops must be 1..%d", LMI_MAX_HOPS);
+  if (cfg->batch_size < 1) LMI_FAIL(LMI_ERR_ARG, "batch_size must be positive");
+  if (cfg->feat_dim < 1) LMI_FAIL(LMI_ERR_ARG, "feat_dim must be positive");
+  if (cfg->feat_dtype != LMI_F32 && cfg->feat_dtype != LMI_F16) LMI_FAIL(LMI_ERR_ARG, "bad feat_dtype");
+  if (cfg->pipes < 1 || cfg->pipes > LMI_MAX_PIPES) LMI_FAIL(LMI_ERR_ARG, "pipes must be 1..%d", LMI_MAX_PIPES);
+  for (int k = 0; k < cfg->hops; ++k)
+    if (cfg->fanout[k] < 1 || cfg->fanout[k] > LMI_MAX_FANOUT)
+      LMI_FAIL(LMI_ERR_ARG, "fanout[%d]=%d outside 1..%d", k, cfg->fanout[k], LMI_MAX_FANOUT);
+  int n_dev = 0;
+  LMI_HIP(hipGetDeviceCount(&n_dev));
+  if (cfg->device_id < 0 || cfg->device_id >= n_dev) LMI_FAIL(LMI_ERR_ARG, "device %d not present", cfg->device_id);
+  LMI_HIP(hipSetDevice(cfg->device_id));
+  Server *s = new (std::nothrow) Server;
+  if (!s) LMI_FAIL(LMI_ERR_HIP, "out of host memory");
+  s->cfg = *cfg;
+  s->row_bytes = (int64_t)cfg->feat_dim * (cfg->feat_dtype == LMI_F16 ? 2 : 4);
+  if (s->row_bytes % 4 != 0) {
+    delete s;
+    LMI_FAIL(LMI_ERR_ARG, "feature rows must be a multiple of 4 bytes");
+  }
+  // worst case: n_k <= n_{k-1} * (1 + f_k)   (the reference under-sizes this, engine/server.cu:204-216)
+  s->node_cap[0] = cfg->batch_size;
+  for (int k = 0; k < cfg->hops; ++k) {
+    s->edge_cap[k] = s->node_cap[k] * cfg->fanout[k];
+    s->node_cap[k + 1] = s->node_cap[k] + s->edge_cap[k];
+    s->max_edges += s->edge_cap[k];
+    s->max_edges_hop = std::max(s->max_edges_hop, s->edge_cap[k]);
+  }
+  for (int k = cfg->hops + 1; k <= LMI_MAX_HOPS; ++k) s->node_cap[k] = s->node_cap[cfg->hops];
+  s->max_nodes = s->node_cap[cfg->hops];
+  if (s->max_nodes + s->max_edges_hop >= (int64_t(1) << 30)) {
+    delete s;
+    LMI_FAIL(LMI_ERR_CAPACITY, "batch_size x fanouts too large for 32-bit local ids");
+  }
+  hipDeviceProp_t prop;
+  if (hipGetDeviceProperties(&prop, cfg->device_id) == hipSuccess) s->n_cu = prop.multiProcessorCount;
+  s->pipes.resize(cfg->pipes);
+  int rc = LMI_OK;
+  for (auto &p : s->pipes)
+    if ((rc = pipe_alloc(s, p)) != LMI_OK) break;
+  if (rc == LMI_OK && hipMalloc(&s->d_scalar, 64) != hipSuccess) rc = LMI_ERR_HIP;
+  if (rc == LMI_OK && hipHostMalloc((void **)&s->prof_ring, sizeof(DevState) * kProfRing, hipHostMallocDefault) != hipSuccess)
+    rc = LMI_ERR_HIP;
+  if (rc != LMI_OK) {
+    lmi_server_destroy(reinterpret_cast<lmi_server *>(s));
+    return rc;
+  }
+  *out = reinterpret_cast<lmi_server *>(s);
+  return LMI_OK;
+}
+
+int lmi_server_destroy(lmi_server *h) {
+  Server *s = reinterpret_cast<Server *>(h);
+  if (!s) return LMI_OK;
+  (void)hipSetDevice(s->cfg.device_id);
+  (void)hipDeviceSynchronize();
+  for (auto &p : s->pipes) pipe_free(p);
+  cache_free(s);
+  if (s->own_graph) {
+    (void)hipFree((void *)s->indptr);
+    (void)hipFree((void *)s->indices);
+  }
+  for (int m = 0; m < 3; ++m) {
+    if (s->set_ids[m]) (void)hipFree(s->set_ids[m]);
+    if (s->set_labels[m]) (void)hipFree(s->set_labels[m]);
+  }
+  for (auto &e : s->prof_events) {
+    (void)hipEventDestroy(e.a);
+    (void)hipEventDestroy(e.b);
+  }
+  for (auto &e : s->prof_free) (void)hipEventDestroy(e);
+  if (s->prof_ring) (void)hipHostFree(s->prof_ring);
+  if (s->d_scalar) (void)hipFree(s->d_scalar);
+  delete s;
+  return LMI_OK;
+}
+
+// ------------------------------------------------------------ memory helpers
+int lmi_host_alloc(size_t bytes, void **host_ptr) {
+  if (!host_ptr) LMI_FAIL(LMI_ERR_ARG, "null argument");
+  LMI_HIP(hipHostMalloc(host_ptr, bytes ? bytes : 1, hipHostMallocMapped | hipHostMallocPortable));
+  return LMI_OK;
+}
+int lmi_host_free(void *host_ptr) {
+  if (host_ptr) LMI_HIP(hipHostFree(host_ptr));
+  return LMI_OK;
+}
+int lmi_device_alloc(size_t bytes, void **dev_ptr) {
+  if (!dev_ptr) LMI_FAIL(LMI_ERR_ARG, "null argument");
+  LMI_HIP(hipMalloc(dev_ptr, bytes ? bytes : 1));
+  return LMI_OK;
+}
+int lmi_device_free(void *dev_ptr) {
+  if (dev_ptr) LMI_HIP(hipFree(dev_ptr));
+  return LMI_OK;
+}
+int lmi_copy_to_host(void *host_dst, const void *dev_src, size_t bytes) {
+  LMI_HIP(hipMemcpy(host_dst, dev_src, bytes, hipMemcpyDeviceToHost));
+  return LMI_OK;
+}
+int lmi_copy_to_device(void *dev_dst, const void *host_src, size_t bytes) {
+  LMI_HIP(hipMemcpy(dev_dst, host_src, bytes, hipMemcpyHostToDevice));
+  return LMI_OK;
+}
+int lmi_stream_create(void **stream) {
+  if (!stream) LMI_FAIL(LMI_ERR_ARG, "null argument");
+  hipStream_t st;
+  LMI_HIP(hipStreamCreateWithFlags(&st, hipStreamNonBlocking));
+  *stream = st;
+  return LMI_OK;
+}
+int lmi_stream_destroy(void *stream) {
+  if (stream) LMI_HIP(hipStreamDestroy((hipStream_t)stream));
+  return LMI_OK;
+}
+int lmi_stream_sync(void *stream) {
+  LMI_HIP(hipStreamSynchronize((hipStream_t)stream));
+  return LMI_OK;
+}
+int lmi_device_sync(void) {
+  LMI_HIP(hipDeviceSynchronize());
+  return LMI_OK;
+}
+
+// ------------------------------------------------------------------ storage
+int lmi_graph_load(lmi_server *h, const int64_t *indptr, const int32_t *indices, int64_t n_nodes, int64_t n_edges,
+                   int location) {
+  Server *s = reinterpret_cast<Server *>(h);
+  if (!s || !indptr || (!indices && n_edges > 0)) LMI_FAIL(LMI_ERR_ARG, "null argument");
+  if (n_nodes < 1 || n_nodes >= (int64_t(1) << 31) - 4096 || n_edges < 0) LMI_FAIL(LMI_ERR_ARG, "bad graph size");
+  LMI_HIP(hipSetDevice(s->cfg.device_id));
+  if (s->own_graph) {
+    (void)hipFree((void *)s->indptr);
+    (void)hipFree((void *)s->indices);
+    s->own_graph = false;
+  }
+  if (location == LMI_LOC_DEVICE) {
+    s->indptr = indptr;
+    s->indices = indices;
+  } else if (location == LMI_LOC_HOST) {
+    if (indptr[0] != 0 || indptr[n_nodes] != n_edges) LMI_FAIL(LMI_ERR_ARG, "indptr[0] must be 0 and indptr[n] == n_edges");
+    int64_t *dp = nullptr;
+    int32_t *di = nullptr;
+    LMI_HIP(hipMalloc(&dp, (size_t)(n_nodes + 1) * 8));
+    LMI_HIP(hipMalloc(&di, (size_t)std::max<int64_t>(n_edges, 1) * 4));
+    LMI_HIP(hipMemcpy(dp, indptr, (size_t)(n_nodes + 1) * 8, hipMemcpyHostToDevice));
+    if (n_edges) LMI_HIP(hipMemcpy(di, indices, (size_t)n_edges * 4, hipMemcpyHostToDevice));
+    s->indptr = dp;
+    s->indices = di;
+    s->own_graph = true;
+  } else {
+    LMI_FAIL(LMI_ERR_ARG, "bad location");
+  }
+  s->n_nodes = n_nodes;
+  s->n_edges = n_edges;
+  return LMI_OK;
+}
+
+int lmi_features_attach(lmi_server *h, const void *rows, int64_t n_rows, int location) {
+  Server *s = reinterpret_cast<Server *>(h);
+  if (!s || !rows || n_rows < 1) LMI_FAIL(LMI_ERR_ARG, "bad argument");
+  LMI_HIP(hipSetDevice(s->cfg.device_id));
+  if (location == LMI_LOC_HOST) {
+    void *d = nullptr;
+    if (hipHostGetDevicePointer(&d, const_cast<void *>(rows), 0) != hipSuccess) {
+      (void)hipGetLastError();
+      LMI_FAIL(LMI_ERR_ARG, "host feature rows must be allocated with lmi_host_alloc (pinned + mapped)");
+    }
+    s->feat = (const uint8_t *)d;
+  } else if (location == LMI_LOC_DEVICE) {
+    s->feat = (const uint8_t *)rows;
+  } else {
+    LMI_FAIL(LMI_ERR_ARG, "bad location");
+  }
+  s->feat_rows = n_rows;
+  s->feat_loc = location;
+  return LMI_OK;
+}
+
+int lmi_idset_load(lmi_server *h, int mode, const int32_t *ids, const int32_t *labels, int64_t n, int location) {
+  Server *s = reinterpret_cast<Server *>(h);
+  if (!s || !ids || n < 1 || mode < 0 || mode > 2) LMI_FAIL(LMI_ERR_ARG, "bad argument");
+  LMI_HIP(hipSetDevice(s->cfg.device_id));
+  const hipMemcpyKind kind = location == LMI_LOC_DEVICE ? hipMemcpyDeviceToDevice : hipMemcpyHostToDevice;
+  if (s->set_ids[mode]) (void)hipFree(s->set_ids[mode]);
+  if (s->set_labels[mode]) (void)hipFree(s->set_labels[mode]);
+  s->set_ids[mode] = s->set_labels[mode] = nullptr;
+  LMI_HIP(hipMalloc(&s->set_ids[mode], (size_t)n * 4));
+  LMI_HIP(hipMemcpy(s->set_ids[mode], ids, (size_t)n * 4, kind));
+  if (labels) {
+    LMI_HIP(hipMalloc(&s->set_labels[mode], (size_t)n * 4));
+    LMI_HIP(hipMemcpy(s->set_labels[mode], labels, (size_t)n * 4, kind));
+  }
+  s->set_n[mode] = n;
+  return LMI_OK;
+}
+
+// ------------------------------------------------------------------- caches
+int lmi_cache_build_static(lmi_server *h, int64_t capacity_rows, int table_kind) {
+  Server *s = reinterpret_cast<Server *>(h);
+  if (!s) LMI_FAIL(LMI_ERR_ARG, "null server");
+  LMI_HIP(hipSetDevice(s->cfg.device_id));
+  return cache_build_static(s, capacity_rows, table_kind, false);
+}
+int lmi_cache_build_int8(lmi_server *h, int64_t capacity_rows, int table_kind) {
+  Server *s = reinterpret_cast<Server *>(h);
+  if (!s) LMI_FAIL(LMI_ERR_ARG, "null server");
+  LMI_HIP(hipSetDevice(s->cfg.device_id));
+  return cache_build_static(s, capacity_rows, table_kind, true);
+}
+int lmi_cache_build_lru(lmi_server *h, int64_t n_sets, int32_t ways) {
+  Server *s = reinterpret_cast<Server *>(h);
+  if (!s) LMI_FAIL(LMI_ERR_ARG, "null server");
+  LMI_HIP(hipSetDevice(s->cfg.device_id));
+  return cache_build_lru(s, n_sets, ways);
+}
+int lmi_cache_info_get(lmi_server *h, lmi_cache_info *out) {
+  Server *s = reinterpret_cast<Server *>(h);
+  if (!s || !out) LMI_FAIL(LMI_ERR_ARG, "null argument");
+  memset(out, 0, sizeof(*out));
+  out->kind = s->cache_kind;
+  out->table_kind = s->table_kind;
+  out->capacity_rows = s->cache_rows;
+  out->row_bytes = s->cache_row_bytes;
+  out->table_bytes = s->cache_kind == LMI_CACHE_LRU ? s->cache_rows * 8
+                     : s->table_kind == LMI_TABLE_DIRECT ? (s->slot_of ? s->n_nodes * 4 : 0)
+                                                         : (int64_t)s->id_table.bytes();
+  out->n_sets = s->lru_sets;
+  out->ways = s->lru_ways;
+  out->lru_tick = s->lru_tick;
+  return LMI_OK;
+}
+int lmi_cache_dump(lmi_server *h, int32_t *slot_of, int64_t n, int32_t *aux) {
+  Server *s = reinterpret_cast<Server *>(h);
+  if (!s || !slot_of) LMI_FAIL(LMI_ERR_ARG, "null argument");
+  LMI_HIP(hipSetDevice(s->cfg.device_id));
+  return cache_dump(s, slot_of, n, aux);
+}
+
+// ---------------------------------------------------------------- operators
+static int ready(Server *s) {
+  if (!s->indptr) LMI_FAIL(LMI_ERR_STATE, "no graph loaded");
+  return LMI_OK;
+}
+
+int lmi_op_batch_generate(lmi_server *h, int pipe, void *stream, const int32_t *seeds, int32_t n, int seeds_location,
+                          int32_t batch_counter, int mode, uint64_t rng_seed) {
+  Server *s = reinterpret_cast<Server *>(h);
+  LMI_TRY(check_pipe(s, pipe));
+  LMI_TRY(ready(s));
+  Pipe &p = s->pipes[pipe];
+  hipStream_t st = (hipStream_t)stream;
+  const int32_t *d_seeds = nullptr, *d_labels = nullptr;
+  if (seeds) {
+    if (n < 0 || n > s->cfg.batch_size) LMI_FAIL(LMI_ERR_CAPACITY, "%d seeds exceed batch_size %d", n, s->cfg.batch_size);
+    if (seeds_location == LMI_LOC_DEVICE) d_seeds = seeds;
+    else {
+      // stage through the scan scratch, which the first hop only writes after the seeds are consumed
+      int32_t *stage = p.cnt;
+      LMI_HIP(hipMemcpyAsync(stage, seeds, (size_t)n * 4, hipMemcpyHostToDevice, st));
+      d_seeds = stage;
+    }
+  } else {
+    // slice `batch_counter` of the id set (batch_generate, operator_impl.cu:40-53); a short last
+    // batch is shortened rather than padded with -1
+    if (mode < 0 || mode > 2 || !s->set_ids[mode]) LMI_FAIL(LMI_ERR_STATE, "id set %d not loaded", mode);
+    const int64_t off = (int64_t)batch_counter * s->cfg.batch_size;
+    if (batch_counter < 0 || off >= s->set_n[mode]) LMI_FAIL(LMI_ERR_ARG, "batch %d is past the end of id set %d", batch_counter, mode);
+    n = (int32_t)std::min<int64_t>(s->cfg.batch_size, s->set_n[mode] - off);
+    d_seeds = s->set_ids[mode] + off;
+    if (s->set_labels[mode]) d_labels = s->set_labels[mode] + off;
+  }
+  p.rng_seed = rng_seed ? rng_seed : s->cfg.seed + (uint64_t)(uint32_t)batch_counter;
+  if (s->cache_kind == LMI_CACHE_LRU) ++s->lru_tick;
+  return launch_batch_generate(s, p, st, d_seeds, n, d_labels);
+}
+
+int lmi_op_random_sample(lmi_server *h, int pipe, void *stream, int hop) {
+  Server *s = reinterpret_cast<Server *>(h);
+  LMI_TRY(check_pipe(s, pipe));
+  LMI_TRY(ready(s));
+  Pipe &p = s->pipes[pipe];
+  if (hop != p.hops_done || hop >= s->cfg.hops) LMI_FAIL(LMI_ERR_ARG, "hop %d out of order (next is %d)", hop, p.hops_done);
+  hipStream_t st = (hipStream_t)stream;
+  int hnd = prof_begin(s, st, PROF_SAMPLE);
+  LMI_TRY(launch_hop(s, p, st, hop));
+  prof_end(s, st, hnd);
+  return LMI_OK;
+}
+
+int lmi_op_cache_lookup(lmi_server *h, int pipe, void *stream, int segment) {
+  Server *s = reinterpret_cast<Server *>(h);
+  LMI_TRY(check_pipe(s, pipe));
+  if (!s->feat) LMI_FAIL(LMI_ERR_STATE, "no features attached");
+  Pipe &p = s->pipes[pipe];
+  if (segment < 0 || segment > p.hops_done) LMI_FAIL(LMI_ERR_ARG, "segment %d not sampled yet", segment);
+  hipStream_t st = (hipStream_t)stream;
+  LMI_TRY(launch_lookup(s, p, st, segment, segment));
+  return launch_gather_seg(s, p, st, segment, segment);
+}
+
+int lmi_op_io_submit(lmi_server *h, int pipe, void *stream) {
+  (void)stream;
+  return check_pipe(reinterpret_cast<Server *>(h), pipe);
+}
+
+int lmi_op_io_complete(lmi_server *h, int pipe, void *stream) {
+  Server *s = reinterpret_cast<Server *>(h);
+  LMI_TRY(check_pipe(s, pipe));
+  Pipe &p = s->pipes[pipe];
+  hipStream_t st = (hipStream_t)stream;
+  LMI_TRY(launch_lru_insert(s, p, st, s->cfg.hops + 1));
+  prof_snapshot(s, p, st);
+  return LMI_OK;
+}
+
+int lmi_run_once(lmi_server *h, int pipe, void *stream, const int32_t *seeds, int32_t n, int seeds_location,
+                 int32_t batch_counter, int mode, uint64_t rng_seed) {
+  Server *s = reinterpret_cast<Server *>(h);
+  LMI_TRY(check_pipe(s, pipe));
+  if (!s->feat) LMI_FAIL(LMI_ERR_STATE, "no features attached");
+  Pipe &p = s->pipes[pipe];
+  hipStream_t st = (hipStream_t)stream;
+  int hb = prof_begin(s, st, PROF_BATCH);
+  LMI_TRY(lmi_op_batch_generate(h, pipe, stream, seeds, n, seeds_location, batch_counter, mode, rng_seed));
+  int hs = prof_begin(s, st, PROF_SAMPLE);
+  for (int k = 0; k < s->cfg.hops; ++k) LMI_TRY(launch_hop(s, p, st, k));
+  prof_end(s, st, hs);
+  LMI_TRY(launch_lookup(s, p, st, 0, s->cfg.hops));
+  LMI_TRY(launch_gather_seg(s, p, st, 0, s->cfg.hops));
+  LMI_TRY(launch_lru_insert(s, p, st, 1));
+  prof_end(s, st, hb);
+  prof_snapshot(s, p, st);
+  return LMI_OK;
+}
+
+// ------------------------------------------------------------------ outputs
+int lmi_batch_view_get(lmi_server *h, int pipe, lmi_batch_view *out) {
+  Server *s = reinterpret_cast<Server *>(h);
+  LMI_TRY(check_pipe(s, pipe));
+  if (!out) LMI_FAIL(LMI_ERR_ARG, "null argument");
+  Pipe &p = s->pipes[pipe];
+  memset(out, 0, sizeof(*out));
+  out->ids = p.ids;
+  out->features = p.features;
+  out->labels = p.labels;
+  out->agg_src_ids = p.agg_src_ids;
+  out->agg_src_off = p.agg_src_off;
+  out->agg_dst_off = p.agg_dst_off;
+  out->node_counter = p.st->node_counter;
+  out->edge_counter = p.st->edge_counter;
+  for (int k = 0; k < LMI_MAX_HOPS; ++k) out->blk_indptr[k] = p.blk_indptr[k];
+  out->cache_index = p.cache_index;
+  out->max_nodes = s->max_nodes;
+  out->max_edges = s->max_edges;
+  return LMI_OK;
+}
+
+int lmi_batch_counters(lmi_server *h, int pipe, void *stream, int32_t node_counter[16], int32_t edge_counter[16]) {
+  Server *s = reinterpret_cast<Server *>(h);
+  LMI_TRY(check_pipe(s, pipe));
+  DevState hs;
+  LMI_HIP(hipStreamSynchronize((hipStream_t)stream));
+  LMI_HIP(hipMemcpy(&hs, s->pipes[pipe].st, sizeof(DevState), hipMemcpyDeviceToHost));
+  if (node_counter) memcpy(node_counter, hs.node_counter, 64);
+  if (edge_counter) memcpy(edge_counter, hs.edge_counter, 64);
+  if (hs.bad_id) LMI_FAIL(LMI_ERR_BAD_ID, "a seed id outside [0, %lld) was skipped", (long long)s->n_nodes);
+  return LMI_OK;
+}
+
+int lmi_steps_per_epoch(lmi_server *h, int mode, int32_t *steps) {
+  Server *s = reinterpret_cast<Server *>(h);
+  if (!s || !steps || mode < 0 || mode > 2) LMI_FAIL(LMI_ERR_ARG, "bad argument");
+  *steps = (int32_t)ceil_div(s->set_n[mode], s->cfg.batch_size);
+  return LMI_OK;
+}
+
+// -------------------------------------------------------------- measurement
+int lmi_profile_enable(lmi_server *h, int on) {
+  Server *s = reinterpret_cast<Server *>(h);
+  if (!s) LMI_FAIL(LMI_ERR_ARG, "null server");
+  s->prof_on = on != 0;
+  return LMI_OK;
+}
+
+int lmi_profile_read(lmi_server *h, lmi_profile *out, int reset) {
+  Server *s = reinterpret_cast<Server *>(h);
+  if (!s || !out) LMI_FAIL(LMI_ERR_ARG, "null argument");
+  LMI_HIP(hipDeviceSynchronize());
+  for (auto &e : s->prof_events) {
+    float ms = 0.0f;
+    if (hipEventElapsedTime(&ms, e.a, e.b) == hipSuccess) {
+      switch (e.kind) {
+        case PROF_GATHER_HIT: s->prof.gather_hit_ms += ms; s->prof.gather_hit_launches++; break;
+        case PROF_GATHER_MISS: s->prof.gather_miss_ms += ms; s->prof.gather_miss_launches++; break;
+        case PROF_SAMPLE: s->prof.sample_ms += ms; s->prof.sample_launches++; break;
+        case PROF_LOOKUP: s->prof.lookup_ms += ms; s->prof.lookup_launches++; break;
+        case PROF_BATCH: s->prof.batch_ms += ms; s->prof.batches++; break;
+      }
+    } else {
+      (void)hipGetLastError();
+    }
+    s->prof_free.push_back(e.a);
+    s->prof_free.push_back(e.b);
+  }
+  s->prof_events.clear();
+  for (int i = 0; i < s->prof_ring_n; ++i) {
+    const DevState &d = s->prof_ring[i];
+    for (int k = 0; k <= LMI_MAX_HOPS; ++k) {
+      s->prof.gather_hit_rows += d.n_hit[k];
+      s->prof.gather_miss_rows += d.n_miss[k];
+    }
+  }
+  s->prof_ring_n = 0;
+  *out = s->prof;
+  if (reset) s->prof = lmi_profile{};
+  return LMI_OK;
+}
+
+int lmi_tune(lmi_server *h, const char *key, int64_t value) {
+  Server *s = reinterpret_cast<Server *>(h);
+  if (!s || !key) LMI_FAIL(LMI_ERR_ARG, "null argument");
+  if (!strcmp(key, "gather_lanes_per_row")) s->gather_lpr = (int)value;
+  else if (!strcmp(key, "gather_unroll")) s->gather_unroll = (int)value;
+  else if (!strcmp(key, "gather_blocks")) s->gather_blocks = (int)value;
+  else if (!strcmp(key, "gather_nontemporal")) s->gather_nt = (int)value;
+  else if (!strcmp(key, "lds_dedup")) s->lds_dedup = (int)value;
+  else if (!strcmp(key, "split_miss")) s->split_miss = (int)value;
+  else LMI_FAIL(LMI_ERR_ARG, "unknown tuning key '%s'", key);
+  return LMI_OK;
+}
+
+int lmi_bench_copy(size_t bytes, int repeats, double *ms_per_copy) {
+  if (!ms_per_copy || repeats < 1 || bytes < 16) LMI_FAIL(LMI_ERR_ARG, "bad argument");
+  void *a = nullptr, *b = nullptr;
+  LMI_HIP(hipMalloc(&a, bytes));
+  LMI_HIP(hipMalloc(&b, bytes));
+  LMI_HIP(hipMemset(a, 1, bytes));
+  hipEvent_t e0, e1;
+  LMI_HIP(hipEventCreate(&e0));
+  LMI_HIP(hipEventCreate(&e1));
+  const size_t n = bytes / 16;
+  hipLaunchKernelGGL(copy_kernel, dim3(4096), dim3(256), 0, 0, (const uint4 *)a, (uint4 *)b, n);
+  LMI_HIP(hipEventRecord(e0, 0));
+  for (int r = 0; r < repeats; ++r)
+    hipLaunchKernelGGL(copy_kernel, dim3(4096), dim3(256), 0, 0, (const uint4 *)a, (uint4 *)b, n);
+  LMI_HIP(hipEventRecord(e1, 0));
+  LMI_HIP(hipEventSynchronize(e1));
+  float ms = 0;
+  LMI_HIP(hipEventElapsedTime(&ms, e0, e1));
+  *ms_per_copy = ms / repeats;
+  (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
+  (void)hipFree(a); (void)hipFree(b);
+  return LMI_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,762 @@
+// Feature caches: static hot-set, LRU dynamic, int8-compressed; the id->slot
+// lookup; and the row gather (HBM rows on hits, zero-copy pinned host rows on
+// misses, dequantisation fused for int8 rows).
+//
+// Reference semantics (Legion-IBP, sampling_server/src):
+//   cache/cache_impl.cuh:239-303        gather: row i of the output belongs to ids[i];
+//                                       hit -> cache row, miss -> host row of the id
+//   cache/cache.cu:314-338              FindFeat: id -> slot for one frontier segment
+//   cache/cache.cu:559-656              FillUp: choose rows, copy them, build the map
+//   comp_cache/static_cache_kernel.cuh:6-29,185-266   set = id mod n_sets, ways contiguous
+// What differs on purpose: hot set = top rows by (out-degree desc, id asc) found
+// with a threshold search and two scans (no sort, no presampling); our own
+// open-addressing table (or a direct map) instead of the vendored cuckoo table;
+// a batch-synchronous LRU (the reference's LRU source is absent); int8 + per-row
+// scale instead of the un-vendored lossless codec; one lane moves 16 bytes and
+// several rows are in flight per lane instead of one float per thread.
+#include <algorithm>
+
+#include "scan.hpp"
+
+namespace lmi {
+
+// ------------------------------------------------------------------ gather
+// Generic row mover.  Row j of the work list names output row i = list[j] (or j);
+// its source row is src_index[i] (or i) and its destination row dst_index[i]
+// (or i); a negative source or destination skips the row.  LPR lanes cooperate
+// on a row, each moving sizeof(V) bytes per step, with U rows in flight.
+template <typename V, int LPR, int U, bool NT>
+static __global__ __launch_bounds__(256) void move_rows_kernel(
+    const int32_t *list, const int32_t *n_ptr, const int32_t *src_index, const int32_t *dst_index,
+    const uint8_t *src, uint8_t *dst, int chunks, int64_t src_row_bytes, int64_t dst_row_bytes) {
+  const int n = *n_ptr;
+  const int lane = threadIdx.x & (LPR - 1);
+  const int group = (blockIdx.x * blockDim.x + threadIdx.x) / LPR;
+  const int n_groups = gridDim.x * blockDim.x / LPR;
+  for (int j0 = group; j0 < n; j0 += n_groups * U) {
+    int64_t so[U], dofs[U];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int j = j0 + u * n_groups;
+      so[u] = -1;
+      dofs[u] = -1;
+      if (j < n) {
+        const int i = list ? list[j] : j;
+        const int si = src_index ? src_index[i] : i;
+        const int di = dst_index ? dst_index[i] : i;
+        if (si >= 0 && di >= 0) {
+          so[u] = (int64_t)si * src_row_bytes;
+          dofs[u] = (int64_t)di * dst_row_bytes;
+        }
+      }
+    }
+    for (int c = lane; c < chunks; c += LPR) {
+      V v[U];
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (so[u] >= 0) v[u] = *reinterpret_cast<const V *>(src + so[u] + (int64_t)c * sizeof(V));
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        if (so[u] >= 0) {
+          V *d = reinterpret_cast<V *>(dst + dofs[u] + (int64_t)c * sizeof(V));
+          if (NT) __builtin_nontemporal_store(v[u], d);
+          else *d = v[u];
+        }
+    }
+  }
+}
+
+typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+
+struct MoveArgs {
+  const int32_t *list, *n_ptr, *src_index, *dst_index;
+  const uint8_t *src;
+  uint8_t *dst;
+  int64_t src_row_bytes, dst_row_bytes, row_bytes;  // row_bytes = bytes moved per row
+  int64_t n_max;
+};
+
+template <typename V, int LPR, int U>
+static void launch_move_vlu(hipStream_t st, const MoveArgs &a, int grid, bool nt) {
+  const int chunks = (int)(a.row_bytes / sizeof(V));
+  if (nt)
+    hipLaunchKernelGGL((move_rows_kernel<V, LPR, U, true>), dim3(grid), dim3(256), 0, st, a.list, a.n_ptr,
+                       a.src_index, a.dst_index, a.src, a.dst, chunks, a.src_row_bytes, a.dst_row_bytes);
+  else
+    hipLaunchKernelGGL((move_rows_kernel<V, LPR, U, false>), dim3(grid), dim3(256), 0, st, a.list, a.n_ptr,
+                       a.src_index, a.dst_index, a.src, a.dst, chunks, a.src_row_bytes, a.dst_row_bytes);
+}
+
+template <typename V, int LPR>
+static void launch_move_vl(hipStream_t st, const MoveArgs &a, int grid, bool nt, int unroll) {
+  switch (unroll) {
+    case 1: launch_move_vlu<V, LPR, 1>(st, a, grid, nt); break;
+    case 2: launch_move_vlu<V, LPR, 2>(st, a, grid, nt); break;
+    case 8: launch_move_vlu<V, LPR, 8>(st, a, grid, nt); break;
+    default: launch_move_vlu<V, LPR, 4>(st, a, grid, nt); break;
+  }
+}
+
+template <typename V>
+static void launch_move_v(hipStream_t st, const MoveArgs &a, int grid, bool nt, int unroll, int lpr) {
+  switch (lpr) {
+    case 8: launch_move_vl<V, 8>(st, a, grid, nt, unroll); break;
+    case 16: launch_move_vl<V, 16>(st, a, grid, nt, unroll); break;
+    case 32: launch_move_vl<V, 32>(st, a, grid, nt, unroll); break;
+    default: launch_move_vl<V, 64>(st, a, grid, nt, unroll); break;
+  }
+}
+
+// Picks the widest vector that divides the row and all base addresses, and a
+// power-of-two lane group that covers one row when possible.
+static int launch_move_rows(Server *s, hipStream_t st, const MoveArgs &a, bool nt) {
+  if (a.n_max <= 0 || a.row_bytes <= 0) return LMI_OK;
+  const uintptr_t align = (uintptr_t)a.src | (uintptr_t)a.dst | (uintptr_t)a.src_row_bytes |
+                          (uintptr_t)a.dst_row_bytes | (uintptr_t)a.row_bytes;
+  int vec = (align % 16 == 0) ? 16 : (align % 8 == 0) ? 8 : 4;
+  if (align % 4 != 0) LMI_FAIL(LMI_ERR_ARG, "feature rows must be 4-byte aligned");
+  const int64_t chunks = a.row_bytes / vec;
+  int lpr = s->gather_lpr;
+  if (lpr != 8 && lpr != 16 && lpr != 32 && lpr != 64) {
+    lpr = 8;
+    while (lpr < chunks && lpr < 64) lpr <<= 1;
+  }
+  const int unroll = s->gather_unroll;
+  const int64_t groups_per_block = 256 / lpr;
+  int64_t want = ceil_div(a.n_max, groups_per_block * (unroll > 0 ? unroll : 1));
+  int64_t cap = s->gather_blocks > 0 ? s->gather_blocks : (int64_t)s->n_cu * 8;
+  const int grid = (int)std::max<int64_t>(1, std::min(want, cap));
+  if (vec == 16) launch_move_v<u32x4>(st, a, grid, nt, unroll, lpr);
+  else if (vec == 8) launch_move_v<u32x2>(st, a, grid, nt, unroll, lpr);
+  else launch_move_v<uint32_t>(st, a, grid, nt, unroll, lpr);
+  LMI_HIP(hipGetLastError());
+  return LMI_OK;
+}
+
+// ------------------------------------------------------------- int8 codec
+__device__ __forceinline__ float load_elem(const uint8_t *row, int i, int dtype) {
+  if (dtype == LMI_F16) return __half2float(reinterpret_cast<const __half *>(row)[i]);
+  return reinterpret_cast<const float *>(row)[i];
+}
+
+// One wavefront per row: absmax over the row, scale = absmax / 127,
+// q = clamp(rint(x / scale), -127, 127).  Build-time only, so the source row
+// (usually in pinned host memory) is read twice rather than staged.
+static __global__ __launch_bounds__(256) void quantize_rows_kernel(
+    const int32_t *row_ids, int64_t n_rows, const uint8_t *feat, int dim, int dtype, int64_t row_bytes,
+    int8_t *q, float *scale) {
+  const int lane = threadIdx.x & (kWave - 1);
+  const int64_t wave = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) / kWave;
+  const int64_t n_waves = (int64_t)gridDim.x * blockDim.x / kWave;
+  for (int64_t r = wave; r < n_rows; r += n_waves) {
+    const uint8_t *row = feat + (int64_t)row_ids[r] * row_bytes;
+    float a = 0.0f;
+    for (int i = lane; i < dim; i += kWave) a = fmaxf(a, fabsf(load_elem(row, i, dtype)));
+#pragma unroll
+    for (int d = kWave / 2; d > 0; d >>= 1) a = fmaxf(a, __shfl_xor(a, d, kWave));
+    const float sc = a / 127.0f;
+    if (lane == 0) scale[r] = sc;
+    for (int i = lane; i < dim; i += kWave) {
+      float v = (a == 0.0f) ? 0.0f : rintf(load_elem(row, i, dtype) / sc);
+      v = fminf(127.0f, fmaxf(-127.0f, v));
+      q[r * dim + i] = (int8_t)v;
+    }
+  }
+}
+
+// Dequantising gather for hits of the int8 cache, 16 elements per lane:
+// y = float(q) * scale, rounded to the output type (RNE for fp16).
+template <typename OUT, int LPR>
+static __global__ __launch_bounds__(256) void gather_int8_kernel(
+    const int32_t *list, const int32_t *n_ptr, const int32_t *cache_index, const int8_t *q,
+    const float *scale, OUT *out, int dim) {
+  const int n = *n_ptr;
+  const int lane = threadIdx.x & (LPR - 1);
+  const int group = (blockIdx.x * blockDim.x + threadIdx.x) / LPR;
+  const int n_groups = gridDim.x * blockDim.x / LPR;
+  const int chunks = dim / 16;
+  for (int j = group; j < n; j += n_groups) {
+    const int i = list[j];
+    const int slot = cache_index[i];
+    if (slot < 0) continue;
+    const float sc = scale[slot];
+    const int8_t *src = q + (int64_t)slot * dim;
+    OUT *dst = out + (int64_t)i * dim;
+    for (int c = lane; c < chunks; c += LPR) {
+      const u32x4 w = *reinterpret_cast<const u32x4 *>(src + c * 16);
+      union alignas(16) {
+        OUT y[16];
+        u32x4 v[sizeof(OUT)];
+      } pk;
+#pragma unroll
+      for (int k = 0; k < 16; ++k) {
+        const int8_t b = (int8_t)((w[k >> 2] >> ((k & 3) * 8)) & 0xFF);
+        const float f = __fmul_rn((float)b, sc);
+        if constexpr (sizeof(OUT) == 2) pk.y[k] = __float2half_rn(f);
+        else pk.y[k] = f;
+      }
+      u32x4 *d4 = reinterpret_cast<u32x4 *>(dst + c * 16);
+#pragma unroll
+      for (int k = 0; k < (int)sizeof(OUT); ++k) __builtin_nontemporal_store(pk.v[k], d4 + k);
+    }
+  }
+}
+
+// Element-wise fallback for row lengths that are not a multiple of 16.
+template <typename OUT>
+static __global__ __launch_bounds__(256) void gather_int8_generic_kernel(
+    const int32_t *list, const int32_t *n_ptr, const int32_t *cache_index, const int8_t *q,
+    const float *scale, OUT *out, int dim) {
+  const int n = *n_ptr;
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave = (blockIdx.x * blockDim.x + threadIdx.x) / kWave;
+  const int n_waves = gridDim.x * blockDim.x / kWave;
+  for (int j = wave; j < n; j += n_waves) {
+    const int i = list[j];
+    const int slot = cache_index[i];
+    if (slot < 0) continue;
+    const float sc = scale[slot];
+    for (int c = lane; c < dim; c += kWave) {
+      const float f = __fmul_rn((float)q[(int64_t)slot * dim + c], sc);
+      if constexpr (sizeof(OUT) == 2) out[(int64_t)i * dim + c] = __float2half_rn(f);
+      else out[(int64_t)i * dim + c] = f;
+    }
+  }
+}
+
+// ------------------------------------------------------------------ lookup
+struct LookupArgs {
+  const int32_t *ids;
+  int64_t n_nodes;
+  int kind, table_kind;
+  const HashSlot *slots;
+  int log2cap;
+  const int32_t *slot_of;
+  const int32_t *lru_keys;
+  int32_t *lru_use;
+  int64_t lru_sets;
+  int lru_ways, tick;
+  int32_t *cache_index, *hit_list, *miss_list, *lru_fill;
+  DevState *st;
+  int seg_first, seg_last, seg;
+};
+
+// id -> slot for rows [first, last) of the batch; rows are appended to the
+// segment's hit or miss list with one atomic per wavefront (ballot + prefix
+// popcount).  List order is arbitrary; it only schedules the gather.
+static __global__ __launch_bounds__(256) void lookup_kernel(LookupArgs a) {
+  const int first = (a.seg_first == 0) ? 0 : a.st->node_counter[9 + a.seg_first - 1];
+  const int last = a.st->node_counter[9 + a.seg_last];
+  const int lane = threadIdx.x & (kWave - 1);
+  const int wave0 = (blockIdx.x * blockDim.x + threadIdx.x) - lane;
+  const int stride = gridDim.x * blockDim.x;
+  for (int b = first + wave0; b < last; b += stride) {
+    const int i = b + lane;
+    bool valid = false;
+    int slot = -1;
+    if (i < last) {
+      const int32_t id = a.ids[i];
+      valid = (id >= 0 && id < a.n_nodes);
+      if (valid) {
+        if (a.kind == LMI_CACHE_LRU) {
+          const int64_t base = ((int64_t)id % a.lru_sets) * a.lru_ways;
+          for (int w = 0; w < a.lru_ways; ++w)
+            if (a.lru_keys[base + w] == id) slot = (int)(base + w);
+          if (slot >= 0) a.lru_use[slot] = a.tick;
+          a.lru_fill[i] = -1;
+        } else if (a.kind != LMI_CACHE_NONE) {
+          slot = (a.table_kind == LMI_TABLE_DIRECT) ? a.slot_of[id] : table_find(a.slots, a.log2cap, id);
+        }
+      }
+      a.cache_index[i] = slot;
+    }
+    const bool hit = valid && slot >= 0, miss = valid && slot < 0;
+    const uint64_t hm = __ballot(hit), mm = __ballot(miss);
+    int hb = 0, mb = 0;
+    if (lane == 0) {
+      if (hm) hb = atomicAdd(&a.st->n_hit[a.seg], __popcll(hm));
+      if (mm) mb = atomicAdd(&a.st->n_miss[a.seg], __popcll(mm));
+    }
+    hb = __shfl(hb, 0, kWave);
+    mb = __shfl(mb, 0, kWave);
+    const uint64_t lt = lanemask_lt();
+    if (hit) a.hit_list[hb + __popcll(hm & lt)] = i;
+    if (miss) a.miss_list[mb + __popcll(mm & lt)] = i;
+  }
+}
+
+static inline int64_t seg_list_base(const Server *s, int seg) { return seg == 0 ? 0 : s->node_cap[seg - 1]; }
+
+int launch_lookup(Server *s, Pipe &p, hipStream_t st, int seg_first, int seg_last) {
+  LookupArgs a{};
+  a.ids = p.ids;
+  a.n_nodes = s->n_nodes;
+  a.kind = s->cache_kind;
+  a.table_kind = s->table_kind;
+  a.slots = s->id_table.slots;
+  a.log2cap = s->id_table.log2cap;
+  a.slot_of = s->slot_of;
+  a.lru_keys = s->lru_keys;
+  a.lru_use = s->lru_use;
+  a.lru_sets = s->lru_sets;
+  a.lru_ways = s->lru_ways;
+  a.tick = s->lru_tick;
+  a.cache_index = p.cache_index;
+  const int64_t base = seg_list_base(s, seg_first);
+  a.hit_list = p.hit_list + base;
+  a.miss_list = p.miss_list + base;
+  a.lru_fill = p.lru_fill;
+  a.st = p.st;
+  a.seg_first = seg_first;
+  a.seg_last = seg_last;
+  a.seg = seg_first;
+  const int64_t n_max = s->node_cap[seg_last];
+  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(n_max, 256), (int64_t)s->n_cu * 8));
+  int h = prof_begin(s, st, PROF_LOOKUP);
+  hipLaunchKernelGGL(lookup_kernel, dim3(grid), dim3(256), 0, st, a);
+  LMI_HIP(hipGetLastError());
+  prof_end(s, st, h);
+  return LMI_OK;
+}
+
+// Gathers the rows of segment `seg`'s hit and miss lists into the pipe's feature
+// buffer.  Hits stream from HBM on `st`; misses stream over the host link on the
+// pipe's side stream so the two overlap; `st` waits for both.
+int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last) {
+  const int64_t base = seg_list_base(s, seg);
+  const int64_t n_max = s->node_cap[seg_last];
+  const bool split = s->split_miss && s->feat_loc == LMI_LOC_HOST && s->cache_kind != LMI_CACHE_NONE;
+  hipStream_t ms = split ? p.side : st;
+  if (split) {
+    LMI_HIP(hipEventRecord(p.fork, st));
+    LMI_HIP(hipStreamWaitEvent(p.side, p.fork, 0));
+  }
+  // misses: raw rows from the feature table
+  {
+    MoveArgs m{};
+    m.list = p.miss_list + base;
+    m.n_ptr = &p.st->n_miss[seg];
+    m.src_index = p.ids;
+    m.dst_index = nullptr;
+    m.src = s->feat;
+    m.dst = (uint8_t *)p.features;
+    m.src_row_bytes = m.dst_row_bytes = m.row_bytes = s->row_bytes;
+    m.n_max = n_max;
+    int h = prof_begin(s, ms, PROF_GATHER_MISS);
+    LMI_TRY(launch_move_rows(s, ms, m, s->gather_nt != 0));
+    prof_end(s, ms, h);
+  }
+  if (s->cache_kind != LMI_CACHE_NONE) {
+    int h = prof_begin(s, st, PROF_GATHER_HIT);
+    if (s->cache_kind == LMI_CACHE_INT8) {
+      const int dim = s->cfg.feat_dim;
+      const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(n_max, 4), (int64_t)s->n_cu * 8));
+      const int32_t *list = p.hit_list + base;
+      const int32_t *n_ptr = &p.st->n_hit[seg];
+      const int8_t *q = (const int8_t *)s->cache_data;
+      if (dim % 16 == 0) {
+        const int chunks = dim / 16;
+        if (s->cfg.feat_dtype == LMI_F16) {
+          if (chunks <= 32)
+            hipLaunchKernelGGL((gather_int8_kernel<__half, 32>), dim3(grid), dim3(256), 0, st, list, n_ptr,
+                               p.cache_index, q, s->cache_scale, (__half *)p.features, dim);
+          else
+            hipLaunchKernelGGL((gather_int8_kernel<__half, 64>), dim3(grid), dim3(256), 0, st, list, n_ptr,
+                               p.cache_index, q, s->cache_scale, (__half *)p.features, dim);
+        } else {
+          if (chunks <= 32)
+            hipLaunchKernelGGL((gather_int8_kernel<float, 32>), dim3(grid), dim3(256), 0, st, list, n_ptr,
+                               p.cache_index, q, s->cache_scale, (float *)p.features, dim);
+          else
+            hipLaunchKernelGGL((gather_int8_kernel<float, 64>), dim3(grid), dim3(256), 0, st, list, n_ptr,
+                               p.cache_index, q, s->cache_scale, (float *)p.features, dim);
+        }
+      } else {
+        if (s->cfg.feat_dtype == LMI_F16)
+          hipLaunchKernelGGL((gather_int8_generic_kernel<__half>), dim3(grid), dim3(256), 0, st, list, n_ptr,
+                             p.cache_index, q, s->cache_scale, (__half *)p.features, dim);
+        else
+          hipLaunchKernelGGL((gather_int8_generic_kernel<float>), dim3(grid), dim3(256), 0, st, list, n_ptr,
+                             p.cache_index, q, s->cache_scale, (float *)p.features, dim);
+      }
+      LMI_HIP(hipGetLastError());
+    } else {
+      MoveArgs m{};
+      m.list = p.hit_list + base;
+      m.n_ptr = &p.st->n_hit[seg];
+      m.src_index = p.cache_index;
+      m.dst_index = nullptr;
+      m.src = s->cache_data;
+      m.dst = (uint8_t *)p.features;
+      m.src_row_bytes = m.dst_row_bytes = m.row_bytes = s->row_bytes;
+      m.n_max = n_max;
+      LMI_TRY(launch_move_rows(s, st, m, s->gather_nt != 0));
+    }
+    prof_end(s, st, h);
+  }
+  if (split) {
+    LMI_HIP(hipEventRecord(p.join, p.side));
+    LMI_HIP(hipStreamWaitEvent(st, p.join, 0));
+  }
+  return LMI_OK;
+}
+
+// --------------------------------------------------------------- LRU insert
+// Round r of the batch-synchronous insertion.  claim[r&1][set] holds the
+// smallest row index among the set's still-unplaced misses; that row takes the
+// way with the smallest (last_use, way) among ways not touched in this batch.
+// Losers bid for the next round in the other claim array.  After `ways` rounds
+// every set has granted all the ways it can.
+struct LruArgs {
+  const int32_t *ids;
+  const int32_t *miss_list[LMI_MAX_HOPS + 1];
+  const DevState *st;
+  int n_lists;
+  int32_t *keys, *use, *claim_cur, *claim_next, *fill;
+  int64_t sets;
+  int ways, tick, round, last_round;
+};
+
+static __global__ __launch_bounds__(256) void lru_bid_kernel(LruArgs a) {
+  for (int l = 0; l < a.n_lists; ++l) {
+    const int n = a.st->n_miss[l];
+    for (int j = blockIdx.x * blockDim.x + threadIdx.x; j < n; j += gridDim.x * blockDim.x) {
+      const int i = a.miss_list[l][j];
+      atomicMin(&a.claim_cur[(int64_t)a.ids[i] % a.sets], i);
+    }
+  }
+}
+
+static __global__ __launch_bounds__(256) void lru_round_kernel(LruArgs a) {
+  for (int l = 0; l < a.n_lists; ++l) {
+    const int n = a.st->n_miss[l];
+    for (int j = blockIdx.x * blockDim.x + threadIdx.x; j < n; j += gridDim.x * blockDim.x) {
+      const int i = a.miss_list[l][j];
+      if (a.fill[i] != -1) continue;  // placed (>= 0) or refused (-2) earlier
+      const int32_t id = a.ids[i];
+      const int64_t set = (int64_t)id % a.sets;
+      if (a.claim_cur[set] == i) {
+        const int64_t base = set * a.ways;
+        int best = -1, best_use = kIntMax;
+        for (int w = 0; w < a.ways; ++w) {
+          const int u = a.use[base + w];
+          if (u < a.tick && u < best_use) best = w, best_use = u;
+        }
+        if (best >= 0) {
+          a.keys[base + best] = id;
+          a.use[base + best] = a.tick;
+          a.fill[i] = (int)(base + best);
+        } else {
+          a.fill[i] = -2;
+        }
+        a.claim_cur[set] = kIntMax;
+      } else if (!a.last_round) {
+        atomicMin(&a.claim_next[set], i);
+      }
+    }
+  }
+}
+
+int launch_lru_insert(Server *s, Pipe &p, hipStream_t st, int n_lists) {
+  if (s->cache_kind != LMI_CACHE_LRU) return LMI_OK;
+  LruArgs a{};
+  a.ids = p.ids;
+  for (int l = 0; l < n_lists; ++l) a.miss_list[l] = p.miss_list + seg_list_base(s, l);
+  a.st = p.st;
+  a.n_lists = n_lists;
+  a.keys = s->lru_keys;
+  a.use = s->lru_use;
+  a.fill = p.lru_fill;
+  a.sets = s->lru_sets;
+  a.ways = s->lru_ways;
+  a.tick = s->lru_tick;
+  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(s->max_nodes, 256), (int64_t)s->n_cu * 4));
+  a.claim_cur = s->lru_claim[0];
+  a.claim_next = s->lru_claim[1];
+  hipLaunchKernelGGL(lru_bid_kernel, dim3(grid), dim3(256), 0, st, a);
+  for (int r = 0; r < s->lru_ways; ++r) {
+    a.round = r;
+    a.last_round = (r == s->lru_ways - 1);
+    a.claim_cur = s->lru_claim[r & 1];
+    a.claim_next = s->lru_claim[(r + 1) & 1];
+    hipLaunchKernelGGL(lru_round_kernel, dim3(grid), dim3(256), 0, st, a);
+  }
+  LMI_HIP(hipGetLastError());
+  // copy the granted rows from the output buffer (already gathered) into the cache
+  for (int l = 0; l < n_lists; ++l) {
+    MoveArgs m{};
+    m.list = p.miss_list + seg_list_base(s, l);
+    m.n_ptr = &p.st->n_miss[l];
+    m.src_index = nullptr;
+    m.dst_index = p.lru_fill;
+    m.src = (const uint8_t *)p.features;
+    m.dst = s->cache_data;
+    m.src_row_bytes = m.dst_row_bytes = m.row_bytes = s->row_bytes;
+    m.n_max = s->node_cap[s->cfg.hops];
+    LMI_TRY(launch_move_rows(s, st, m, false));
+  }
+  return LMI_OK;
+}
+
+// -------------------------------------------------------- static cache build
+static __global__ __launch_bounds__(256) void degree_stats_kernel(const int64_t *indptr, int64_t n,
+                                                                  int64_t thr, unsigned long long *count_ge,
+                                                                  unsigned long long *max_deg) {
+  unsigned long long c = 0, m = 0;
+  for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < n; v += (int64_t)gridDim.x * blockDim.x) {
+    const unsigned long long d = (unsigned long long)(indptr[v + 1] - indptr[v]);
+    c += (d >= (unsigned long long)thr) ? 1 : 0;
+    m = d > m ? d : m;
+  }
+#pragma unroll
+  for (int d = kWave / 2; d > 0; d >>= 1) {
+    c += __shfl_down(c, d, kWave);
+    const unsigned long long o = __shfl_down(m, d, kWave);
+    m = o > m ? o : m;
+  }
+  if ((threadIdx.x & (kWave - 1)) == 0) {
+    if (c) atomicAdd(count_ge, c);
+    atomicMax(max_deg, m);
+  }
+}
+
+// mode 0: cnt[v] = (deg == thr);  mode 1: cnt[v] = member flag using tie ranks.
+static __global__ __launch_bounds__(kScanBlock) void member_flag_kernel(
+    const int64_t *indptr, const int32_t *n_ptr, int64_t thr, int mode, const int32_t *tie_rank,
+    int64_t ties_taken, int32_t *cnt, int32_t *tile_sums) {
+  __shared__ int lds[kScanBlock / kWave];
+  const int n = *n_ptr;
+  const int n_tiles = (n + kScanTile - 1) / kScanTile;
+  for (int tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+    const int base = tile * kScanTile + threadIdx.x * kScanItems;
+    int sum = 0;
+#pragma unroll
+    for (int j = 0; j < kScanItems; ++j) {
+      const int v = base + j;
+      if (v < n) {
+        const int64_t d = indptr[v + 1] - indptr[v];
+        int f;
+        if (mode == 0) f = (d == thr);
+        else f = (d > thr) || (d == thr && (int64_t)tie_rank[v] < ties_taken);
+        cnt[v] = f;
+        sum += f;
+      }
+    }
+    tile_reduce_store(sum, tile_sums, tile, lds);
+  }
+}
+
+static __global__ __launch_bounds__(256) void publish_slots_kernel(const int32_t *member, const int32_t *slot,
+                                                                   int64_t n, int table_kind, HashSlot *slots,
+                                                                   int log2cap, int32_t *slot_of,
+                                                                   int32_t *cached_ids) {
+  for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < n; v += (int64_t)gridDim.x * blockDim.x) {
+    const bool m = member[v] != 0;
+    if (table_kind == LMI_TABLE_DIRECT) slot_of[v] = m ? slot[v] : -1;
+    if (m) {
+      cached_ids[slot[v]] = (int32_t)v;
+      if (table_kind == LMI_TABLE_HASH) {
+        const uint32_t h = table_insert_min(slots, log2cap, (int32_t)v, slot[v]);
+        (void)h;
+      }
+    }
+  }
+}
+
+static __global__ void fill_i32_kernel(int32_t *p, int64_t n, int32_t v) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+    p[i] = v;
+}
+
+static __global__ void fill_slots_kernel(HashSlot *p, int64_t n) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+    p[i] = HashSlot{kEmptyKey, kIntMax};
+}
+
+int launch_table_clear(Table &t, hipStream_t st) {
+  const int64_t n = int64_t(1) << t.log2cap;
+  hipLaunchKernelGGL(fill_slots_kernel, dim3((int)std::min<int64_t>(ceil_div(n, 256), 4096)), dim3(256), 0, st,
+                     t.slots, n);
+  LMI_HIP(hipGetLastError());
+  return LMI_OK;
+}
+
+void cache_free(Server *s) {
+  if (s->cache_data) (void)hipFree(s->cache_data);
+  if (s->cache_scale) (void)hipFree(s->cache_scale);
+  if (s->id_table.slots) (void)hipFree(s->id_table.slots);
+  if (s->slot_of) (void)hipFree(s->slot_of);
+  if (s->lru_keys) (void)hipFree(s->lru_keys);
+  if (s->lru_use) (void)hipFree(s->lru_use);
+  if (s->lru_claim[0]) (void)hipFree(s->lru_claim[0]);
+  if (s->lru_claim[1]) (void)hipFree(s->lru_claim[1]);
+  s->cache_data = nullptr;
+  s->cache_scale = nullptr;
+  s->id_table = Table{};
+  s->slot_of = nullptr;
+  s->lru_keys = s->lru_use = s->lru_claim[0] = s->lru_claim[1] = nullptr;
+  s->cache_kind = LMI_CACHE_NONE;
+  s->cache_rows = 0;
+}
+
+static int count_ge(const Server *s, int64_t thr, unsigned long long *d_pair, int64_t *count, int64_t *max_deg) {
+  LMI_HIP(hipMemset(d_pair, 0, 16));
+  hipLaunchKernelGGL(degree_stats_kernel, dim3(s->n_cu * 8), dim3(256), 0, 0, s->indptr, s->n_nodes, thr, d_pair,
+                     d_pair + 1);
+  unsigned long long h[2];
+  LMI_HIP(hipMemcpy(h, d_pair, 16, hipMemcpyDeviceToHost));
+  *count = (int64_t)h[0];
+  if (max_deg) *max_deg = (int64_t)h[1];
+  return LMI_OK;
+}
+
+// Hot set = first `capacity_rows` nodes under (out-degree desc, id asc):
+// everything above the threshold degree plus the lowest-id ties at the threshold.
+// slot(v) = number of cached nodes with a smaller id.
+int cache_build_static(Server *s, int64_t capacity_rows, int table_kind, bool int8) {
+  if (!s->indptr || !s->feat) LMI_FAIL(LMI_ERR_STATE, "load the graph and attach features before building a cache");
+  if (table_kind != LMI_TABLE_HASH && table_kind != LMI_TABLE_DIRECT) LMI_FAIL(LMI_ERR_ARG, "bad table kind");
+  if (s->n_nodes >= (int64_t(1) << 31) - kScanTile) LMI_FAIL(LMI_ERR_CAPACITY, "too many nodes");
+  cache_free(s);
+  const int64_t N = s->n_nodes;
+  const int64_t cap = std::max<int64_t>(0, std::min(capacity_rows, N));
+  s->table_kind = table_kind;
+  s->cache_row_bytes = int8 ? s->cfg.feat_dim : s->row_bytes;
+  if (cap == 0) LMI_FAIL(LMI_ERR_ARG, "cache capacity must be at least one row");
+
+  unsigned long long *d_pair = nullptr;
+  int32_t *d_cnt = nullptr, *d_tie = nullptr, *d_slot = nullptr, *d_tiles = nullptr, *d_n = nullptr,
+          *d_cached = nullptr;
+  LMI_HIP(hipMalloc(&d_pair, 16));
+  LMI_HIP(hipMalloc(&d_cnt, (N + 1) * 4));
+  LMI_HIP(hipMalloc(&d_tie, (N + 1) * 4));
+  LMI_HIP(hipMalloc(&d_slot, (N + 1) * 4));
+  LMI_HIP(hipMalloc(&d_tiles, (ceil_div(N, kScanTile) + 1) * 4));
+  LMI_HIP(hipMalloc(&d_n, 8));
+  LMI_HIP(hipMalloc(&d_cached, cap * 4));
+  const int32_t n32[2] = {(int32_t)N, 0};
+  LMI_HIP(hipMemcpy(d_n, n32, 8, hipMemcpyHostToDevice));
+
+  // threshold degree: largest d with count(deg >= d) >= cap
+  int64_t cnt = 0, max_deg = 0;
+  LMI_TRY(count_ge(s, 0, d_pair, &cnt, &max_deg));
+  int64_t lo = 0, hi = max_deg + 1;
+  while (hi - lo > 1) {
+    const int64_t mid = lo + (hi - lo) / 2;
+    LMI_TRY(count_ge(s, mid, d_pair, &cnt, nullptr));
+    if (cnt >= cap) lo = mid; else hi = mid;
+  }
+  const int64_t thr = lo;
+  LMI_TRY(count_ge(s, thr + 1, d_pair, &cnt, nullptr));
+  const int64_t ties_taken = cap - cnt;
+
+  const int grid = scan_grid(N);
+  hipLaunchKernelGGL(member_flag_kernel, dim3(grid), dim3(kScanBlock), 0, 0, s->indptr, d_n, thr, 0, nullptr,
+                     (int64_t)0, d_cnt, d_tiles);
+  LMI_TRY(launch_scan_phases(0, d_cnt, d_tie, d_tiles, d_n, N, SCAN_EPI_NONE, nullptr, 0, d_n + 1));
+  hipLaunchKernelGGL(member_flag_kernel, dim3(grid), dim3(kScanBlock), 0, 0, s->indptr, d_n, thr, 1, d_tie,
+                     ties_taken, d_cnt, d_tiles);
+  LMI_TRY(launch_scan_phases(0, d_cnt, d_slot, d_tiles, d_n, N, SCAN_EPI_NONE, nullptr, 0, d_n + 1));
+  int32_t total = 0;
+  LMI_HIP(hipMemcpy(&total, d_n + 1, 4, hipMemcpyDeviceToHost));
+  if (total != cap) LMI_FAIL(LMI_ERR_HIP, "static cache selection picked %d rows, expected %lld", total, (long long)cap);
+
+  if (table_kind == LMI_TABLE_HASH) {
+    int lg = 4;
+    while ((int64_t(1) << lg) < 2 * cap) ++lg;
+    if (lg > 31) LMI_FAIL(LMI_ERR_CAPACITY, "cache too large for the hash table");
+    s->id_table.log2cap = lg;
+    LMI_HIP(hipMalloc(&s->id_table.slots, size_t(8) << lg));
+    LMI_TRY(launch_table_clear(s->id_table, 0));
+  } else {
+    LMI_HIP(hipMalloc(&s->slot_of, N * 4));
+  }
+  hipLaunchKernelGGL(publish_slots_kernel, dim3(s->n_cu * 8), dim3(256), 0, 0, d_cnt, d_slot, N, table_kind,
+                     s->id_table.slots, s->id_table.log2cap, s->slot_of, d_cached);
+  LMI_HIP(hipGetLastError());
+
+  // rows
+  LMI_HIP(hipMalloc(&s->cache_data, (size_t)cap * s->cache_row_bytes));
+  int32_t cap32[2] = {(int32_t)cap, 0};
+  LMI_HIP(hipMemcpy(d_n, cap32, 8, hipMemcpyHostToDevice));
+  if (int8) {
+    LMI_HIP(hipMalloc(&s->cache_scale, (size_t)cap * 4));
+    hipLaunchKernelGGL(quantize_rows_kernel, dim3(s->n_cu * 8), dim3(256), 0, 0, d_cached, cap, s->feat,
+                       s->cfg.feat_dim, s->cfg.feat_dtype, s->row_bytes, (int8_t *)s->cache_data, s->cache_scale);
+    LMI_HIP(hipGetLastError());
+  } else {
+    MoveArgs m{};
+    m.list = nullptr;
+    m.n_ptr = d_n;
+    m.src_index = d_cached;
+    m.dst_index = nullptr;
+    m.src = s->feat;
+    m.dst = s->cache_data;
+    m.src_row_bytes = m.dst_row_bytes = m.row_bytes = s->row_bytes;
+    m.n_max = cap;
+    LMI_TRY(launch_move_rows(s, 0, m, false));
+  }
+  LMI_HIP(hipDeviceSynchronize());
+  (void)hipFree(d_pair); (void)hipFree(d_cnt); (void)hipFree(d_tie); (void)hipFree(d_slot);
+  (void)hipFree(d_tiles); (void)hipFree(d_n); (void)hipFree(d_cached);
+  s->cache_rows = cap;
+  s->cache_kind = int8 ? LMI_CACHE_INT8 : LMI_CACHE_STATIC;
+  return LMI_OK;
+}
+
+int cache_build_lru(Server *s, int64_t n_sets, int32_t ways) {
+  if (!s->feat) LMI_FAIL(LMI_ERR_STATE, "attach features before building a cache");
+  if (n_sets < 1 || ways < 1 || ways > 64 || n_sets * ways >= (int64_t(1) << 31))
+    LMI_FAIL(LMI_ERR_ARG, "bad LRU geometry (sets=%lld ways=%d)", (long long)n_sets, ways);
+  cache_free(s);
+  const int64_t rows = n_sets * ways;
+  LMI_HIP(hipMalloc(&s->lru_keys, rows * 4));
+  LMI_HIP(hipMalloc(&s->lru_use, rows * 4));
+  LMI_HIP(hipMalloc(&s->lru_claim[0], n_sets * 4));
+  LMI_HIP(hipMalloc(&s->lru_claim[1], n_sets * 4));
+  LMI_HIP(hipMalloc(&s->cache_data, (size_t)rows * s->row_bytes));
+  const int g = 2048;
+  hipLaunchKernelGGL(fill_i32_kernel, dim3(g), dim3(256), 0, 0, s->lru_keys, rows, -1);
+  hipLaunchKernelGGL(fill_i32_kernel, dim3(g), dim3(256), 0, 0, s->lru_use, rows, 0);
+  hipLaunchKernelGGL(fill_i32_kernel, dim3(g), dim3(256), 0, 0, s->lru_claim[0], n_sets, kIntMax);
+  hipLaunchKernelGGL(fill_i32_kernel, dim3(g), dim3(256), 0, 0, s->lru_claim[1], n_sets, kIntMax);
+  LMI_HIP(hipDeviceSynchronize());
+  s->lru_sets = n_sets;
+  s->lru_ways = ways;
+  s->lru_tick = 0;
+  s->cache_rows = rows;
+  s->cache_row_bytes = s->row_bytes;
+  s->cache_kind = LMI_CACHE_LRU;
+  return LMI_OK;
+}
+
+static __global__ void dump_hash_kernel(const HashSlot *slots, int log2cap, int64_t n, int32_t *out) {
+  for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < n; v += (int64_t)gridDim.x * blockDim.x)
+    out[v] = table_find(slots, log2cap, (int32_t)v);
+}
+
+int cache_dump(Server *s, int32_t *slot_of, int64_t n, int32_t *aux) {
+  if (s->cache_kind == LMI_CACHE_NONE) LMI_FAIL(LMI_ERR_STATE, "no cache built");
+  LMI_HIP(hipDeviceSynchronize());
+  if (s->cache_kind == LMI_CACHE_LRU) {
+    if (n != s->cache_rows) LMI_FAIL(LMI_ERR_ARG, "LRU dump needs n == sets*ways");
+    LMI_HIP(hipMemcpy(slot_of, s->lru_keys, n * 4, hipMemcpyDeviceToHost));
+    if (aux) LMI_HIP(hipMemcpy(aux, s->lru_use, n * 4, hipMemcpyDeviceToHost));
+    return LMI_OK;
+  }
+  if (n != s->n_nodes) LMI_FAIL(LMI_ERR_ARG, "dump needs n == n_nodes");
+  if (s->table_kind == LMI_TABLE_DIRECT) {
+    LMI_HIP(hipMemcpy(slot_of, s->slot_of, n * 4, hipMemcpyDeviceToHost));
+  } else {
+    int32_t *d = nullptr;
+    LMI_HIP(hipMalloc(&d, n * 4));
+    hipLaunchKernelGGL(dump_hash_kernel, dim3(s->n_cu * 4), dim3(256), 0, 0, s->id_table.slots,
+                       s->id_table.log2cap, n, d);
+    LMI_HIP(hipMemcpy(slot_of, d, n * 4, hipMemcpyDeviceToHost));
+    (void)hipFree(d);
+  }
+  return LMI_OK;
+}
+
+}  // namespace lmi

@@ -1,0 +1,174 @@
+// Shared declarations of the MI355X sampling-server library (gfx950, wave64).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+#include <stdint.h>
+
+#include <string>
+#include <vector>
+
+#include "../../include/legion_mi.h"
+
+namespace lmi {
+
+constexpr int kWave = 64;
+constexpr int32_t kEmptyKey = -1;
+constexpr int32_t kIntMax = 0x7fffffff;
+
+// ---------------------------------------------------------------- errors
+void set_error(const char *fmt, ...);
+#define LMI_HIP(call)                                                                    \
+  do {                                                                                   \
+    hipError_t e_ = (call);                                                              \
+    if (e_ != hipSuccess) {                                                              \
+      lmi::set_error("%s failed: %s (%s:%d)", #call, hipGetErrorString(e_), __FILE__,    \
+                     __LINE__);                                                          \
+      return LMI_ERR_HIP;                                                                \
+    }                                                                                    \
+  } while (0)
+#define LMI_TRY(call)            \
+  do {                           \
+    int rc_ = (call);            \
+    if (rc_ != LMI_OK) return rc_; \
+  } while (0)
+#define LMI_FAIL(code, ...)        \
+  do {                             \
+    lmi::set_error(__VA_ARGS__);   \
+    return (code);                 \
+  } while (0)
+
+// ------------------------------------------------------- device-side state
+// Lives in HBM, one per pipe.  The two 16-int headers are the reference's
+// node_counter / edge_counter (engine/operator_impl.cu:58-91); the rest is
+// bookkeeping the kernels read instead of round-tripping through the host.
+struct DevState {
+  int32_t node_counter[16];
+  int32_t edge_counter[16];
+  // One hit list and one miss list per lookup segment (0 = seeds or the whole
+  // batch, k = nodes added by hop k); zeroed at batch start.
+  int32_t n_hit[LMI_MAX_HOPS + 1];
+  int32_t n_miss[LMI_MAX_HOPS + 1];
+  int32_t bad_id;      // set when a seed id is outside [0, n_nodes)
+  int32_t scan_total;  // total of the last device scan
+  int32_t pad[6];
+};
+
+struct HashSlot {  // 8-byte open-addressing slot: one 64-bit load per probe
+  int32_t key;
+  int32_t val;
+};
+
+struct Table {  // id -> value, linear probing, capacity = 2^log2cap
+  HashSlot *slots = nullptr;
+  int32_t log2cap = 0;
+  __host__ __device__ uint32_t mask() const { return (1u << log2cap) - 1u; }
+  size_t bytes() const { return slots ? (size_t(8) << log2cap) : 0; }
+};
+
+struct Pipe {
+  // outputs (reference: per-pipe MemoryPool / IPC buffers)
+  int32_t *ids = nullptr;
+  void *features = nullptr;
+  int32_t *labels = nullptr;
+  int32_t *agg_src_ids = nullptr, *agg_src_off = nullptr, *agg_dst_off = nullptr;
+  int32_t *blk_indptr[LMI_MAX_HOPS] = {nullptr, nullptr, nullptr};
+  int32_t *cache_index = nullptr;
+  DevState *st = nullptr;
+  // scratch
+  Table dedup;                 // global id -> local id (per batch)
+  int32_t *eslot = nullptr;    // [max_edges_hop] table slot of each edge's source
+  int32_t *firstv = nullptr;   // [max_edges_hop] table value seen by each edge
+  int32_t *cnt = nullptr;      // [max(max_nodes, max_edges_hop)] scan input
+  int32_t *rank = nullptr;     // [max_edges_hop + 1] scan output
+  int32_t *tile_sums = nullptr;
+  int32_t *hit_list = nullptr, *miss_list = nullptr;  // [max_nodes] row indices
+  int32_t *lru_fill = nullptr;                        // [max_nodes] slot granted to a miss
+  hipStream_t side = nullptr;  // second stream: host-link misses overlap HBM hits
+  hipEvent_t fork = nullptr, join = nullptr;
+  uint64_t rng_seed = 0;
+  int32_t n_seeds = 0;
+  int32_t hops_done = 0;
+};
+
+struct EventPair {
+  hipEvent_t a, b;
+  int kind;
+};
+
+struct Server {
+  lmi_config cfg{};
+  int64_t max_nodes = 0, max_edges = 0, max_edges_hop = 0;
+  int64_t node_cap[LMI_MAX_HOPS + 1] = {0, 0, 0, 0};  // worst-case n_k
+  int64_t edge_cap[LMI_MAX_HOPS] = {0, 0, 0};         // worst-case e_k
+  int64_t row_bytes = 0;
+  // storage
+  const int64_t *indptr = nullptr;
+  const int32_t *indices = nullptr;
+  int64_t n_nodes = 0, n_edges = 0;
+  bool own_graph = false;
+  const uint8_t *feat = nullptr;  // device-visible address of the feature table
+  int64_t feat_rows = 0;
+  int feat_loc = LMI_LOC_HOST;
+  int32_t *set_ids[3] = {nullptr, nullptr, nullptr};
+  int32_t *set_labels[3] = {nullptr, nullptr, nullptr};
+  int64_t set_n[3] = {0, 0, 0};
+  // cache
+  int cache_kind = LMI_CACHE_NONE;
+  int table_kind = LMI_TABLE_HASH;
+  int64_t cache_rows = 0;
+  int64_t cache_row_bytes = 0;
+  uint8_t *cache_data = nullptr;     // [cache_rows][cache_row_bytes]
+  float *cache_scale = nullptr;      // int8: per-row scale
+  Table id_table;                    // hash id -> slot
+  int32_t *slot_of = nullptr;        // direct id -> slot
+  int64_t lru_sets = 0;
+  int32_t lru_ways = 0;
+  int32_t lru_tick = 0;
+  int32_t *lru_keys = nullptr, *lru_use = nullptr, *lru_claim[2] = {nullptr, nullptr};
+  // pipes
+  std::vector<Pipe> pipes;
+  // tuning
+  int gather_lpr = 0;     // lanes per row (0 = auto)
+  int gather_unroll = 4;
+  int gather_blocks = 0;  // 0 = auto
+  int gather_nt = 1;      // non-temporal output stores
+  int lds_dedup = 1;
+  int split_miss = 1;     // misses on the side stream
+  // profiling
+  bool prof_on = false;
+  std::vector<EventPair> prof_events;   // recorded, not yet resolved
+  std::vector<hipEvent_t> prof_free;    // recycled events
+  DevState *prof_ring = nullptr;        // pinned host snapshots of finished batches
+  int prof_ring_n = 0;
+  lmi_profile prof{};
+  int32_t *d_scalar = nullptr;          // small device scratch (counts for build-time launches)
+  int n_cu = 256;
+};
+
+enum { PROF_GATHER_HIT = 0, PROF_GATHER_MISS = 1, PROF_SAMPLE = 2, PROF_LOOKUP = 3, PROF_BATCH = 4 };
+
+// profiling helpers (api.hip)
+int prof_begin(Server *s, hipStream_t st, int kind);
+int prof_end(Server *s, hipStream_t st, int handle);
+
+// sampler.hip
+int launch_batch_generate(Server *s, Pipe &p, hipStream_t st, const int32_t *d_seeds, int32_t n,
+                          const int32_t *d_labels);
+int launch_hop(Server *s, Pipe &p, hipStream_t st, int hop);
+int launch_table_clear(Table &t, hipStream_t st);
+
+enum { SCAN_EPI_NONE = 0, SCAN_EPI_HOP_EDGES = 1, SCAN_EPI_HOP_NODES = 2 };
+
+// cache.hip
+int cache_build_static(Server *s, int64_t capacity_rows, int table_kind, bool int8);
+int cache_build_lru(Server *s, int64_t n_sets, int32_t ways);
+void cache_free(Server *s);
+int launch_lookup(Server *s, Pipe &p, hipStream_t st, int seg_first, int seg_last);
+int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last);
+int launch_lru_insert(Server *s, Pipe &p, hipStream_t st, int n_lists);
+int cache_dump(Server *s, int32_t *slot_of, int64_t n, int32_t *aux);
+
+inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+}  // namespace lmi

@@ -1,0 +1,112 @@
+// Device-side building blocks: Philox4x32-10, open-addressing probes, wave64 /
+// block scans.  gfx950 only (64-wide wavefronts).
+#pragma once
+
+#include "common.hpp"
+
+namespace lmi {
+
+// ------------------------------------------------------------------ Philox
+// Philox4x32-10 (Salmon et al. 2011); constants as published.
+struct Philox4 {
+  uint32_t x, y, z, w;
+};
+
+__device__ __forceinline__ Philox4 philox4x32_10(uint32_t c0, uint32_t c1, uint32_t c2, uint32_t c3,
+                                                 uint32_t k0, uint32_t k1) {
+#pragma unroll
+  for (int r = 0; r < 10; ++r) {
+    const uint32_t hi0 = __umulhi(0xD2511F53u, c0), lo0 = 0xD2511F53u * c0;
+    const uint32_t hi1 = __umulhi(0xCD9E8D57u, c2), lo1 = 0xCD9E8D57u * c2;
+    c0 = hi1 ^ c1 ^ k0;
+    c1 = lo1;
+    c2 = hi0 ^ c3 ^ k1;
+    c3 = lo0;
+    k0 += 0x9E3779B9u;
+    k1 += 0xBB67AE85u;
+  }
+  return Philox4{c0, c1, c2, c3};
+}
+
+// The sampler's draw: key = 64-bit batch seed, counter = (node, hop, slot, 0).
+__device__ __forceinline__ uint32_t sample_draw(uint64_t seed, uint32_t hop, uint32_t node,
+                                                uint32_t slot) {
+  return philox4x32_10(node, hop, slot, 0u, (uint32_t)seed, (uint32_t)(seed >> 32)).x;
+}
+
+// -------------------------------------------------------------- hash table
+__device__ __forceinline__ uint32_t hash_id(int32_t key, int log2cap) {
+  return ((uint32_t)key * 0x9E3779B1u) >> (32 - log2cap);
+}
+
+// Insert `key` (if absent) and lower its value to min(value, cand); returns the
+// slot index.  Keys only ever go EMPTY -> key, so a stale non-empty read is
+// still correct and a stale EMPTY read is resolved by the CAS.
+__device__ __forceinline__ uint32_t table_insert_min(HashSlot *slots, int log2cap, int32_t key,
+                                                     int32_t cand) {
+  const uint32_t mask = (1u << log2cap) - 1u;
+  uint32_t h = hash_id(key, log2cap);
+  while (true) {
+    int32_t k = slots[h].key;
+    if (k == kEmptyKey) {
+      k = atomicCAS(&slots[h].key, kEmptyKey, key);
+      if (k == kEmptyKey) k = key;
+    }
+    if (k == key) break;
+    h = (h + 1) & mask;
+  }
+  atomicMin(&slots[h].val, cand);
+  return h;
+}
+
+// Read-only probe: value or -1.
+__device__ __forceinline__ int32_t table_find(const HashSlot *slots, int log2cap, int32_t key) {
+  const uint32_t mask = (1u << log2cap) - 1u;
+  uint32_t h = hash_id(key, log2cap);
+  while (true) {
+    const int2 kv = *reinterpret_cast<const int2 *>(&slots[h]);
+    if (kv.x == key) return kv.y;
+    if (kv.x == kEmptyKey) return -1;
+    h = (h + 1) & mask;
+  }
+}
+
+// ------------------------------------------------------------------- scans
+__device__ __forceinline__ int wave_inclusive_scan(int v) {
+  const int lane = threadIdx.x & (kWave - 1);
+#pragma unroll
+  for (int d = 1; d < kWave; d <<= 1) {
+    const int t = __shfl_up(v, d, kWave);
+    if (lane >= d) v += t;
+  }
+  return v;
+}
+
+// Exclusive scan over a block of BLOCK threads; `total` = sum over the block.
+// lds must hold BLOCK / 64 + 1 ints.  Contains __syncthreads: call uniformly.
+template <int BLOCK>
+__device__ __forceinline__ int block_exclusive_scan(int v, int *lds, int &total) {
+  constexpr int NW = BLOCK / kWave;
+  const int lane = threadIdx.x & (kWave - 1), wid = threadIdx.x / kWave;
+  const int inc = wave_inclusive_scan(v);
+  if (lane == kWave - 1) lds[wid] = inc;
+  __syncthreads();
+  if (wid == 0) {
+    int w = (lane < NW) ? lds[lane] : 0;
+    const int winc = wave_inclusive_scan(w);
+    if (lane < NW) lds[lane] = winc - w;
+    if (lane == NW - 1) lds[NW] = winc;
+  }
+  __syncthreads();
+  const int res = inc - v + lds[wid];
+  total = lds[NW];
+  __syncthreads();
+  return res;
+}
+
+__device__ __forceinline__ uint64_t lanemask_lt() {
+  const int lane = threadIdx.x & (kWave - 1);
+  return (lane == 0) ? 0ull : (~0ull >> (kWave - lane));
+}
+
+}  // namespace lmi
