@@ -56,3 +56,236 @@ def test_sample_batch_parity(lmi, oracle, fanout, n_nodes, mean_deg, batch):
     finally:
         srv.close()
         feats.free()
+
+
+def test_duplicate_seeds_and_isolated_nodes(lmi, oracle):
+    rng = np.random.default_rng(5)
+    indptr, indices = random_graph(rng, 300, 6, zero_frac=0.4)
+    feats = make_features(lmi, rng, 300, 4)
+    srv = lmi.Server(32, [4, 3], 4)
+    try:
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        seeds = rng.integers(0, 300, 32).astype(np.int32)
+        seeds[5] = seeds[1]
+        seeds[20] = seeds[1]
+        srv.run_once(seeds, rng_seed=9)
+        assert_batch_equal(srv.fetch(), oracle.sample_batch(indptr, indices, seeds, [4, 3], 9))
+        # empty batch
+        srv.run_once(np.zeros(0, np.int32), rng_seed=9)
+        g = srv.fetch()
+        assert g.n_nodes == [0, 0, 0] and g.n_edges == [0, 0]
+    finally:
+        srv.close()
+        feats.free()
+
+
+def test_bad_seed_is_reported(lmi):
+    rng = np.random.default_rng(6)
+    indptr, indices = random_graph(rng, 100, 5)
+    feats = make_features(lmi, rng, 100, 4)
+    srv = lmi.Server(8, [3], 4)
+    try:
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        srv.run_once(np.array([1, 2, 100, 3], np.int32), rng_seed=1)
+        with pytest.raises(lmi.LegionError) as ei:
+            srv.counters()
+        assert ei.value.code == -5
+        with pytest.raises(lmi.LegionError):
+            srv.run_once(np.zeros(9, np.int32))  # more seeds than batch_size
+    finally:
+        srv.close()
+        feats.free()
+
+
+@pytest.mark.parametrize("table", [0, 1])
+@pytest.mark.parametrize("dim,dtype", [(128, np.float32), (100, np.float32), (1433, np.float32), (768, np.float16),
+                                        (6, np.float16)])
+def test_static_cache_parity(lmi, oracle, table, dim, dtype):
+    rng = np.random.default_rng(dim + table)
+    n_nodes, batch, fanout = 4000, 96, [10, 5]
+    indptr, indices = random_graph(rng, n_nodes, 8, hubs=10, hub_deg=300)
+    feats = make_features(lmi, rng, n_nodes, dim, dtype)
+    srv = lmi.Server(batch, fanout, dim, feat_dtype=lmi.F16 if dtype == np.float16 else lmi.F32)
+    try:
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        for cap in (1, 1200, n_nodes):
+            srv.build_static_cache(cap, table)
+            slot_ref = oracle.static_cache_build(indptr, cap)
+            np.testing.assert_array_equal(srv.cache_dump(n_nodes), slot_ref)
+            seeds = rng.choice(n_nodes, batch, replace=False).astype(np.int32)
+            srv.run_once(seeds, rng_seed=cap)
+            g = srv.fetch()
+            o = oracle.sample_batch(indptr, indices, seeds, fanout, cap)
+            assert_batch_equal(g, o)
+            np.testing.assert_array_equal(g.cache_index, slot_ref[o.ids])
+            assert g.features.tobytes() == feats.array[o.ids].tobytes()
+    finally:
+        srv.close()
+        feats.free()
+
+
+def test_operator_chain_matches_run_once(lmi, oracle):
+    """The five reference operator slots, called one by one, give the same batch."""
+    rng = np.random.default_rng(11)
+    n_nodes, batch, fanout, dim = 3000, 50, [6, 4, 3], 32
+    indptr, indices = random_graph(rng, n_nodes, 10)
+    feats = make_features(lmi, rng, n_nodes, dim)
+    train = rng.permutation(n_nodes)[:230].astype(np.int32)
+    labels = (train % 7).astype(np.int32)
+    srv = lmi.Server(batch, fanout, dim, seed=5)
+    try:
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        srv.load_idset(lmi.MODE_TRAIN, train, labels)
+        srv.build_static_cache(1000)
+        slot_ref = oracle.static_cache_build(indptr, 1000)
+        for it in range(5):  # 230 ids / 50 -> last batch has 30 seeds
+            srv.op_batch_generate(None, batch_counter=it)
+            srv.op_cache_lookup(0)
+            srv.op_io_submit()
+            for k in range(3):
+                srv.op_random_sample(k)
+                srv.op_cache_lookup(k + 1)
+                srv.op_io_submit()
+            srv.op_io_complete()
+            g = srv.fetch()
+            seeds = train[it * batch:(it + 1) * batch]
+            o = oracle.sample_batch(indptr, indices, seeds, fanout, 5 + it)
+            assert_batch_equal(g, o)
+            np.testing.assert_array_equal(g.labels, labels[it * batch:(it + 1) * batch])
+            np.testing.assert_array_equal(g.cache_index, slot_ref[o.ids])
+            assert g.features.tobytes() == feats.array[o.ids].tobytes()
+        with pytest.raises(lmi.LegionError):
+            srv.op_batch_generate(None, batch_counter=5)  # past the end of the id set
+    finally:
+        srv.close()
+        feats.free()
+
+
+@pytest.mark.parametrize("n_sets,ways", [(64, 8), (16, 4), (1, 32), (500, 2)])
+def test_lru_cache_parity(lmi, oracle, n_sets, ways):
+    """Reference-shaped toy workload (comp_cache/tests/test_cache.cu:4-9,48-53):
+    1000 nodes, 130 hot ones, 90 % of the seeds hot -- replayed on both sides."""
+    rng = np.random.default_rng(n_sets * 100 + ways)
+    n_nodes, batch, fanout, dim = 1000, 128, [3, 2], 32
+    indptr, indices = random_graph(rng, n_nodes, 6)
+    feats = make_features(lmi, rng, n_nodes, dim)
+    hot = rng.choice(n_nodes, 130, replace=False)
+    srv = lmi.Server(batch, fanout, dim)
+    lru = oracle.Lru(n_sets, ways, dim * 4)
+    host_rows = feats.array.view(np.uint8).reshape(n_nodes, dim * 4)
+    try:
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        srv.build_lru_cache(n_sets, ways)
+        for it in range(12):
+            k_hot = int(batch * 0.9)
+            seeds = np.concatenate([rng.choice(hot, k_hot, replace=False),
+                                    rng.choice(n_nodes, batch - k_hot, replace=False)]).astype(np.int32)
+            seeds = np.array(list(dict.fromkeys(seeds.tolist())), np.int32)
+            srv.run_once(seeds, rng_seed=it + 1)
+            g = srv.fetch()
+            o = oracle.sample_batch(indptr, indices, seeds, fanout, it + 1)
+            assert_batch_equal(g, o)
+            hit, fill, out = lru.access(o.ids, host_rows)
+            np.testing.assert_array_equal(g.cache_index, hit)
+            assert g.features.tobytes() == out.tobytes()
+            keys, use = srv.cache_dump(n_sets * ways, with_aux=True)
+            okeys, ouse = lru.state()
+            np.testing.assert_array_equal(keys, okeys)
+            np.testing.assert_array_equal(use, ouse)
+        assert (hit >= 0).sum() > 0
+    finally:
+        srv.close()
+        feats.free()
+
+
+def test_lru_operator_chain(lmi, oracle):
+    rng = np.random.default_rng(3)
+    n_nodes, batch, fanout, dim = 800, 40, [4, 3], 16
+    indptr, indices = random_graph(rng, n_nodes, 6)
+    feats = make_features(lmi, rng, n_nodes, dim)
+    srv = lmi.Server(batch, fanout, dim)
+    lru = oracle.Lru(32, 4, dim * 4)
+    host_rows = feats.array.view(np.uint8).reshape(n_nodes, dim * 4)
+    try:
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        srv.build_lru_cache(32, 4)
+        for it in range(6):
+            seeds = rng.choice(200, batch, replace=False).astype(np.int32)
+            srv.op_batch_generate(seeds, rng_seed=it + 1)
+            srv.op_cache_lookup(0)
+            for k in range(2):
+                srv.op_random_sample(k)
+                srv.op_cache_lookup(k + 1)
+            srv.op_io_complete()
+            g = srv.fetch()
+            o = oracle.sample_batch(indptr, indices, seeds, fanout, it + 1)
+            assert_batch_equal(g, o)
+            hit, fill, out = lru.access(o.ids, host_rows)
+            np.testing.assert_array_equal(g.cache_index, hit)
+            assert g.features.tobytes() == out.tobytes()
+            keys, use = srv.cache_dump(128, with_aux=True)
+            okeys, ouse = lru.state()
+            np.testing.assert_array_equal(keys, okeys)
+            np.testing.assert_array_equal(use, ouse)
+    finally:
+        srv.close()
+        feats.free()
+
+
+@pytest.mark.parametrize("dim,dtype", [(768, np.float16), (128, np.float32), (100, np.float32), (48, np.float16),
+                                        (6, np.float16)])
+def test_int8_cache_parity(lmi, oracle, dim, dtype):
+    rng = np.random.default_rng(dim)
+    n_nodes, batch, fanout = 3000, 64, [8, 4]
+    indptr, indices = random_graph(rng, n_nodes, 8, hubs=4, hub_deg=200)
+    feats = make_features(lmi, rng, n_nodes, dim, dtype)
+    feats.array[7] = 0            # all-zero row: scale 0
+    feats.array[11, 0] = 3.0      # clear absmax
+    srv = lmi.Server(batch, fanout, dim, feat_dtype=lmi.F16 if dtype == np.float16 else lmi.F32)
+    try:
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        cap = 2000
+        srv.build_int8_cache(cap)
+        slot_ref = oracle.static_cache_build(indptr, cap)
+        np.testing.assert_array_equal(srv.cache_dump(n_nodes), slot_ref)
+        cached = np.flatnonzero(slot_ref >= 0)
+        q, sc = oracle.quantize_rows(feats.array[cached])
+        for it in range(3):
+            seeds = rng.choice(n_nodes, batch, replace=False).astype(np.int32)
+            if it == 0:
+                seeds[:2] = [7, 11]
+            srv.run_once(seeds, rng_seed=it + 1)
+            g = srv.fetch()
+            o = oracle.sample_batch(indptr, indices, seeds, fanout, it + 1)
+            assert_batch_equal(g, o)
+            np.testing.assert_array_equal(g.cache_index, slot_ref[o.ids])
+            ref = oracle.gather_rows_int8(o.ids, slot_ref[o.ids], q, sc, feats.array)
+            # tolerance: north-star allows 1 ulp on dequantised rows; both sides do one IEEE
+            # multiply (+ RNE to fp16), so the expected difference is 0
+            assert g.features.tobytes() == ref.tobytes()
+    finally:
+        srv.close()
+        feats.free()
+
+
+def test_synth_graph_matches_oracle(lmi, oracle):
+    cdf = lmi.zipf_cdf(2.0, 500, 9.0)
+    for mode in (0, 1):
+        ip, ix, ne = lmi.synth_graph(42, cdf, 20000, mode)
+        indptr = lmi.to_host(ip, 20001, np.int64)
+        indices = lmi.to_host(ix, ne, np.int32)
+        o_indptr, o_indices = oracle.synth_graph(42, cdf, 20000, mode)
+        np.testing.assert_array_equal(indptr, o_indptr)
+        np.testing.assert_array_equal(indices, o_indices)
+        lmi.check(lmi.lib().lmi_device_free(ip))
+        lmi.check(lmi.lib().lmi_device_free(ix))
+    np.testing.assert_array_equal(lmi.synth_trainset(7, 20000, 1500), oracle.synth_trainset(7, 20000, 1500))
+    mean = np.diff(indptr).mean()
+    assert 8.0 < mean < 10.0
