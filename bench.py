@@ -1,0 +1,277 @@
+#!/usr/bin/env python3
+"""Benchmark of the sampling-server hot path on one MI355X.
+
+A "step" is one mini-batch: seed ids in -> multi-hop sampled blocks + gathered
+feature rows resident in HBM.  Inputs (CSR graph, feature table, cache, train
+set) are synthetic, generated on the GPU from a fixed seed, and resident before
+the timed region starts.  One JSON line is printed on stdout.
+
+    python bench.py [--gpus 1] [--steps 50] [--warmup 5] [--workload paper100m]
+
+Workloads (BASELINE.json `configs`): paper100m (default, the configuration the
+metric is quoted on), products, paper100m-lru, mag240m-int8 (down-scaled node
+count, stated in the output), cora.  `--scale` shrinks node counts for quick runs.
+"""
+import argparse
+import importlib.util
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0      # MI355X HBM3E, published
+HOST_LINK_PEAK_GBS = 64.0  # PCIe Gen5 x16 per direction, nominal
+
+
+def load_package():
+    path = os.path.join(ROOT, "legion-ibp_amd", "__init__.py")
+    spec = importlib.util.spec_from_file_location("legion_ibp_amd", path)
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules["legion_ibp_amd"] = mod
+    spec.loader.exec_module(mod)
+    return mod
+
+
+WORKLOADS = {
+    # name: nodes, mean degree, alpha, d_max, dim, dtype, batch, fanout, train, cache
+    "paper100m": dict(nodes=111_059_956, mean_deg=14.548, alpha=2.0, d_max=100_000, dim=128, dtype="f32",
+                      batch=8000, fanout=[25, 10], train=1_200_000, cache=("static", 38e9)),
+    "products": dict(nodes=2_449_029, mean_deg=25.27, alpha=2.1, d_max=17_000, dim=100, dtype="f32",
+                     batch=800, fanout=[25, 10], train=196_615, cache=("static_frac", 0.30)),
+    "paper100m-lru": dict(nodes=111_059_956, mean_deg=14.548, alpha=2.0, d_max=100_000, dim=128, dtype="f32",
+                          batch=4096, fanout=[15, 10, 5], train=1_200_000, cache=("lru", 20e9)),
+    "mag240m-int8": dict(nodes=244_160_499, mean_deg=7.08, alpha=2.0, d_max=100_000, dim=768, dtype="f16",
+                         batch=1024, fanout=[25, 15], train=1_112_392, cache=("int8", 80e9)),
+    "cora": dict(nodes=2_708, mean_deg=7.8, alpha=None, d_max=40, dim=1433, dtype="f32",
+                 batch=64, fanout=[25, 10], train=2_708, cache=("static_frac", 1.0)),
+}
+
+
+def log(msg):
+    print("[bench] " + msg, file=sys.stderr, flush=True)
+
+
+def build_workload(lmi, w, seed, pipes, host_budget_gb):
+    """Generate the graph, features, train set and cache; returns (server, info)."""
+    np_dtype = np.float16 if w["dtype"] == "f16" else np.float32
+    esz = np.dtype(np_dtype).itemsize
+    n_nodes = w["nodes"]
+    note = None
+    feat_gb = n_nodes * w["dim"] * esz / 1e9
+    if feat_gb > host_budget_gb:
+        # the feature table must fit in pinned host memory on this box
+        scale = host_budget_gb / feat_gb
+        n_nodes = int(n_nodes * scale)
+        note = "node count down-scaled x%.3f so the %.0f GB feature table fits pinned host memory" % (scale, feat_gb)
+        log(note)
+    t0 = time.time()
+    if w["alpha"] is None:   # Erdos-Renyi-like: Poisson degrees, uniform neighbours
+        from math import exp
+        lam = w["mean_deg"]
+        pmf = [exp(-lam)]
+        for d in range(1, w["d_max"] + 1):
+            pmf.append(pmf[-1] * lam / d)
+        cdf = np.cumsum(pmf) / np.sum(pmf)
+        t = np.minimum(np.floor(cdf * 4294967296.0), 4294967295.0).astype(np.uint64)
+        t[-1] = 4294967295
+        cdf_u32, mode = t.astype(np.uint32), 0
+    else:
+        cdf_u32, mode = lmi.zipf_cdf(w["alpha"], w["d_max"], w["mean_deg"]), 1
+    d_indptr, d_indices, n_edges = lmi.synth_graph(seed, cdf_u32, n_nodes, mode)
+    log("graph: %d nodes, %d edges in HBM (%.1f s)" % (n_nodes, n_edges, time.time() - t0))
+    t0 = time.time()
+    feats = lmi.HostBuffer((n_nodes, w["dim"]), np_dtype)
+    lmi.synth_features(seed + 1, feats)
+    log("features: %.2f GB in pinned host memory (%.1f s)" % (feats.nbytes / 1e9, time.time() - t0))
+    srv = lmi.Server(w["batch"], w["fanout"], w["dim"], feat_dtype=lmi.F16 if w["dtype"] == "f16" else lmi.F32,
+                     pipes=pipes, seed=seed)
+    srv.attach_graph_device(d_indptr, d_indices, n_nodes, n_edges)
+    srv.attach_features(feats)
+    n_train = min(w["train"], n_nodes)
+    train = lmi.synth_trainset(seed + 2, n_nodes, n_train)
+    srv.load_idset(lmi.MODE_TRAIN, train)
+    t0 = time.time()
+    kind, amount = w["cache"]
+    row_bytes = w["dim"] * esz
+    if kind == "static":
+        rows = min(n_nodes, int(amount // row_bytes))
+        srv.build_static_cache(rows, lmi.TABLE_HASH)
+    elif kind == "static_frac":
+        rows = max(1, int(n_nodes * amount))
+        srv.build_static_cache(rows, lmi.TABLE_HASH)
+    elif kind == "lru":
+        ways = 8
+        rows = min(n_nodes, int(amount // row_bytes))
+        srv.build_lru_cache(max(1, rows // ways), ways)
+    elif kind == "int8":
+        rows = min(n_nodes, int(amount // (w["dim"] + 4)))
+        srv.build_int8_cache(rows, lmi.TABLE_HASH)
+    ci = srv.cache_info()
+    log("cache: kind=%d rows=%d (%.2f GB) table %.2f GB (%.1f s)" % (
+        ci.kind, ci.capacity_rows, ci.capacity_rows * ci.row_bytes / 1e9, ci.table_bytes / 1e9, time.time() - t0))
+    info = dict(n_nodes=n_nodes, n_edges=n_edges, n_train=n_train, note=note, feats=feats, d_indptr=d_indptr,
+                d_indices=d_indices, train=train, row_bytes=row_bytes, cache_rows=int(ci.capacity_rows),
+                cache_kind=kind)
+    return srv, info
+
+
+def cpu_baseline(lmi, srv, w, info, seed, budget_s):
+    """The CPU oracle on the same workload and host cores; also checks the GPU
+    output of the same batches bit for bit."""
+    from oracle import binding as orc
+    cores = len(os.sched_getaffinity(0))
+    box_share = int(os.environ.get("OMP_NUM_THREADS", "0") or 0)
+    threads = min(cores, box_share) if box_share > 0 else cores
+    n_nodes, n_edges = info["n_nodes"], info["n_edges"]
+    t0 = time.time()
+    indptr = lmi.to_host(info["d_indptr"], n_nodes + 1, np.int64)
+    indices = lmi.to_host(info["d_indices"], n_edges, np.int32)
+    log("cpu baseline: CSR copied to host (%.1f s), %d threads" % (time.time() - t0, threads))
+    feats = info["feats"].array
+    B = w["batch"]
+    done, spent, parity_ok, rows = 0, 0.0, True, 0
+    while done < 20 and spent < budget_s:
+        seeds = info["train"][done * B:(done + 1) * B]
+        rs = seed + done
+        t0 = time.time()
+        o = orc.sample_batch(indptr, indices, seeds, w["fanout"], rs, threads=threads)
+        out = orc.gather_rows(o.ids, np.full(len(o.ids), -1, np.int32), None, feats, threads=threads)
+        spent += time.time() - t0
+        rows += len(o.ids)
+        srv.run_once(None, batch_counter=done, rng_seed=rs)
+        g = srv.fetch()
+        same = (np.array_equal(g.ids, o.ids) and np.array_equal(g.agg_src_off, o.agg_src_off) and
+                np.array_equal(g.agg_dst_off, o.agg_dst_off) and np.array_equal(g.agg_src_ids, o.agg_src_ids) and
+                list(g.node_counter) == list(o.node_counter) and list(g.edge_counter) == list(o.edge_counter) and
+                all(np.array_equal(a, b) for a, b in zip(g.blk_indptr, o.blk_indptr)))
+        if info["cache_kind"] != "int8":
+            same = same and g.features.tobytes() == out.tobytes()
+        else:
+            miss = g.cache_index < 0
+            same = same and g.features[miss].tobytes() == out[miss].tobytes()
+        # threshold property of the degree-ordered static cache
+        if info["cache_kind"] in ("static", "static_frac", "int8") and len(o.ids):
+            deg = indptr[o.ids + 1] - indptr[o.ids]
+            hit = g.cache_index >= 0
+            if hit.any() and (~hit).any():
+                same = same and deg[hit].min() >= deg[~hit].max()
+        parity_ok = parity_ok and same
+        done += 1
+    return dict(value=done / spent, unit="batches/s", cores=threads, kind="port",
+                sample="%d batches of the same workload (oracle sample_batch + gather, OpenMP over %d threads); "
+                       "GPU output of the same batches %s" % (done, threads,
+                                                              "bit-exact" if parity_ok else "MISMATCH"),
+                gather_rows_per_s=rows / spent), parity_ok
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="paper100m", choices=sorted(WORKLOADS))
+    ap.add_argument("--scale", type=float, default=1.0, help="shrink node/train counts (testing only)")
+    ap.add_argument("--pipes", type=int, default=2)
+    ap.add_argument("--seed", type=int, default=20260101)
+    ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget (0 = skip)")
+    ap.add_argument("--host-gb", type=float, default=200.0, help="pinned host memory budget for the feature table")
+    ap.add_argument("--tune", action="append", default=[], help="key=value passed to lmi_tune")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU; there is no multi-GPU path (got --gpus %d)" % args.gpus,
+              file=sys.stderr)
+        sys.exit(2)
+    lmi = load_package()
+    w = dict(WORKLOADS[args.workload])
+    if args.scale != 1.0:
+        w["nodes"] = max(1000, int(w["nodes"] * args.scale))
+        w["train"] = max(w["batch"], int(w["train"] * args.scale))
+        if w["cache"][0] in ("static", "lru", "int8"):
+            w["cache"] = (w["cache"][0], w["cache"][1] * args.scale)
+    if w["cache"][0] == "lru":
+        args.pipes = 1   # the LRU state is batch-synchronous: batches may not overlap
+    srv, info = build_workload(lmi, w, args.seed, args.pipes, args.host_gb)
+    for kv in args.tune:
+        k, v = kv.split("=")
+        srv.tune(k, int(v))
+    steps_per_epoch = -(-info["n_train"] // w["batch"])
+    streams = [lmi.stream_create() for _ in range(args.pipes)]
+
+    def step(i):
+        p = i % args.pipes
+        srv.run_once(None, batch_counter=i % steps_per_epoch, rng_seed=args.seed + i, pipe=p, stream=streams[p])
+
+    for i in range(args.warmup):
+        step(i)
+    lmi.check(lmi.lib().lmi_device_sync())
+    srv.profile_read(reset=True)
+    srv.profile_enable(True)
+    t0 = time.perf_counter()
+    for i in range(args.warmup, args.warmup + args.steps):
+        step(i)
+    lmi.check(lmi.lib().lmi_device_sync())
+    t1 = time.perf_counter()
+    srv.profile_enable(False)
+    prof = srv.profile_read(reset=True)
+    ms_per_step = (t1 - t0) * 1e3 / args.steps
+
+    # algorithmic bytes per gathered row: row read + row written + 4 (id) + 4 (slot)
+    rb = info["row_bytes"]
+    if info["cache_kind"] == "int8":
+        hit_bytes = w["dim"] + 4 + rb + 8
+    else:
+        hit_bytes = 2 * rb + 8
+    hit_ms = prof.gather_hit_ms / max(prof.gather_hit_launches, 1)
+    hit_rows = prof.gather_hit_rows / max(prof.gather_hit_launches, 1)
+    miss_ms = prof.gather_miss_ms / max(prof.gather_miss_launches, 1)
+    miss_rows = prof.gather_miss_rows / max(prof.gather_miss_launches, 1)
+    achieved = hit_rows * hit_bytes / (hit_ms * 1e-3) / 1e9 if hit_ms > 0 else 0.0
+    copy_ms = lmi.bench_copy(1 << 30, 10)
+    copy_gbs = 2 * (1 << 30) / (copy_ms * 1e-3) / 1e9
+    roofline = dict(bound="hbm", kernel="move_rows_kernel (hit gather)", achieved=round(achieved, 1),
+                    peak=HBM_PEAK_GBS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBS, 4), traffic=None,
+                    rows_per_launch=round(hit_rows, 1), bytes_per_row=hit_bytes, avg_launch_ms=round(hit_ms, 4),
+                    measured_copy_gbs=round(copy_gbs, 1))
+    host_link = dict(bound="host-link", kernel="move_rows_kernel (miss gather)",
+                     achieved=round(miss_rows * rb / (miss_ms * 1e-3) / 1e9, 2) if miss_ms > 0 else 0.0,
+                     peak=HOST_LINK_PEAK_GBS, unit="GB/s", rows_per_launch=round(miss_rows, 1),
+                     avg_launch_ms=round(miss_ms, 4))
+    total_rows = prof.gather_hit_rows + prof.gather_miss_rows
+    out = {
+        "metric": "sampled mini-batches/sec", "value": round(args.steps / (t1 - t0), 2), "unit": "batches/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int32 ids / " + ("fp16" if w["dtype"] == "f16" else "fp32") + " rows (byte copy)",
+        "data": "synthetic",
+        "config": {"workload": args.workload, "nodes": info["n_nodes"], "edges": info["n_edges"],
+                   "feat_dim": w["dim"], "batch": w["batch"], "fanout": w["fanout"],
+                   "cache": "%s, %d rows" % (info["cache_kind"], info["cache_rows"]), "pipes": args.pipes,
+                   "graph": "Zipf-Mandelbrot degrees alpha=%s, degree-proportional neighbours" % w["alpha"],
+                   "note": info["note"]},
+        "feature_gather_gbs": round(achieved, 1),
+        "feature_gather_frac_hbm_peak": round(achieved / HBM_PEAK_GBS, 4),
+        "cache_hit_rate": round(prof.gather_hit_rows / total_rows, 4) if total_rows else None,
+        "rows_per_batch": round(total_rows / max(args.steps, 1), 1),
+        "kernel_ms_per_batch": {"sample": round(prof.sample_ms / max(prof.sample_launches, 1), 4),
+                                "lookup": round(prof.lookup_ms / max(prof.lookup_launches, 1), 4),
+                                "gather_hit": round(hit_ms, 4), "gather_miss": round(miss_ms, 4),
+                                "batch": round(prof.batch_ms / max(prof.batches, 1), 4)},
+        "roofline": roofline, "host_link": host_link,
+    }
+    if args.cpu_seconds > 0:
+        cb, ok = cpu_baseline(lmi, srv, w, info, args.seed, args.cpu_seconds)
+        out["cpu_baseline"] = cb
+        out["parity_at_bench_scale"] = "bit-exact" if ok else "MISMATCH"
+    else:
+        out["cpu_baseline"] = None
+    print(json.dumps(out), flush=True)
+    srv.close()
+
+
+if __name__ == "__main__":
+    main()
