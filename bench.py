@@ -56,7 +56,7 @@ def log(msg):
     print("[bench] " + msg, file=sys.stderr, flush=True)
 
 
-def build_workload(lmi, w, seed, pipes, host_budget_gb):
+def build_workload(lmi, w, seed, pipes, host_budget_gb, table=2):
     """Generate the graph, features, train set and cache; returns (server, info)."""
     np_dtype = np.float16 if w["dtype"] == "f16" else np.float32
     esz = np.dtype(np_dtype).itemsize
@@ -100,17 +100,17 @@ def build_workload(lmi, w, seed, pipes, host_budget_gb):
     row_bytes = w["dim"] * esz
     if kind == "static":
         rows = min(n_nodes, int(amount // row_bytes))
-        srv.build_static_cache(rows, lmi.TABLE_HASH)
+        srv.build_static_cache(rows, table)
     elif kind == "static_frac":
         rows = max(1, int(n_nodes * amount))
-        srv.build_static_cache(rows, lmi.TABLE_HASH)
+        srv.build_static_cache(rows, table)
     elif kind == "lru":
         ways = 8
         rows = min(n_nodes, int(amount // row_bytes))
         srv.build_lru_cache(max(1, rows // ways), ways)
     elif kind == "int8":
         rows = min(n_nodes, int(amount // (w["dim"] + 4)))
-        srv.build_int8_cache(rows, lmi.TABLE_HASH)
+        srv.build_int8_cache(rows, table)
     ci = srv.cache_info()
     log("cache: kind=%d rows=%d (%.2f GB) table %.2f GB (%.1f s)" % (
         ci.kind, ci.capacity_rows, ci.capacity_rows * ci.row_bytes / 1e9, ci.table_bytes / 1e9, time.time() - t0))
@@ -180,6 +180,7 @@ def main():
     ap.add_argument("--seed", type=int, default=20260101)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget (0 = skip)")
     ap.add_argument("--host-gb", type=float, default=200.0, help="pinned host memory budget for the feature table")
+    ap.add_argument("--table", default="rank", choices=["hash", "direct", "rank"], help="id->slot table layout")
     ap.add_argument("--tune", action="append", default=[], help="key=value passed to lmi_tune")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -195,16 +196,19 @@ def main():
             w["cache"] = (w["cache"][0], w["cache"][1] * args.scale)
     if w["cache"][0] == "lru":
         args.pipes = 1   # the LRU state is batch-synchronous: batches may not overlap
-    srv, info = build_workload(lmi, w, args.seed, args.pipes, args.host_gb)
+    srv, info = build_workload(lmi, w, args.seed, args.pipes, args.host_gb,
+                               {"hash": 0, "direct": 1, "rank": 2}[args.table])
     for kv in args.tune:
         k, v = kv.split("=")
         srv.tune(k, int(v))
     steps_per_epoch = -(-info["n_train"] // w["batch"])
-    streams = [lmi.stream_create() for _ in range(args.pipes)]
+    stream = lmi.stream_create()
 
     def step(i):
-        p = i % args.pipes
-        srv.run_once(None, batch_counter=i % steps_per_epoch, rng_seed=args.seed + i, pipe=p, stream=streams[p])
+        # one caller stream; consecutive batches alternate output buffer sets (pipes), so the
+        # host-link part of batch i (on the server's side stream) overlaps the sampling of batch i+1
+        srv.run_once(None, batch_counter=i % steps_per_epoch, rng_seed=args.seed + i, pipe=i % args.pipes,
+                     stream=stream)
 
     for i in range(args.warmup):
         step(i)
@@ -250,7 +254,8 @@ def main():
         "data": "synthetic",
         "config": {"workload": args.workload, "nodes": info["n_nodes"], "edges": info["n_edges"],
                    "feat_dim": w["dim"], "batch": w["batch"], "fanout": w["fanout"],
-                   "cache": "%s, %d rows" % (info["cache_kind"], info["cache_rows"]), "pipes": args.pipes,
+                   "cache": "%s, %d rows, %s id->slot table" % (info["cache_kind"], info["cache_rows"], args.table),
+                   "pipes": args.pipes,
                    "graph": "Zipf-Mandelbrot degrees alpha=%s, degree-proportional neighbours" % w["alpha"],
                    "note": info["note"]},
         "feature_gather_gbs": round(achieved, 1),

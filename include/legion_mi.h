@@ -46,7 +46,10 @@ enum {
 enum { LMI_F32 = 0, LMI_F16 = 1 };                       /* feature element type */
 enum { LMI_LOC_HOST = 0, LMI_LOC_DEVICE = 1 };           /* where an input pointer lives */
 enum { LMI_MODE_TRAIN = 0, LMI_MODE_VALID = 1, LMI_MODE_TEST = 2 }; /* TRAINMODE.. (include/system_config.cuh) */
-enum { LMI_TABLE_HASH = 0, LMI_TABLE_DIRECT = 1 };       /* id->slot table layout */
+/* id->slot table layout of the static / int8 caches: open-addressing hash (8 B per
+ * slot, load <= 0.5), direct map (4 B per node), or membership bitmap with a
+ * running rank (16 B per 64 nodes; slot = rank of the node among cached nodes) */
+enum { LMI_TABLE_HASH = 0, LMI_TABLE_DIRECT = 1, LMI_TABLE_RANK = 2 };
 enum { LMI_CACHE_NONE = 0, LMI_CACHE_STATIC = 1, LMI_CACHE_LRU = 2, LMI_CACHE_INT8 = 3 };
 
 typedef struct lmi_server lmi_server;
@@ -171,11 +174,19 @@ int lmi_op_io_submit(lmi_server *s, int pipe, void *stream);
  * misses into the LRU cache. */
 int lmi_op_io_complete(lmi_server *s, int pipe, void *stream);
 /* Runner::RunOnce (engine/server.cu:330-400): the whole operator chain with one
- * gather over all rows. */
+ * gather over all rows.  On a non-default stream the sampling part replays a HIP
+ * graph captured on first use.  Returns with the host-link part of the gather
+ * possibly still running on the server's side stream: see lmi_batch_wait. */
 int lmi_run_once(lmi_server *s, int pipe, void *stream, const int32_t *seeds, int32_t n,
                  int seeds_location, int32_t batch_counter, int mode, uint64_t rng_seed);
 
 /* ---- outputs ----------------------------------------------------------- */
+/* Makes `stream` wait until every output of the pipe's last batch is complete,
+ * including rows still being fetched over the host link on the server's own side
+ * stream.  This is the point where the reference's runner has seen its last
+ * operator's event and posts the batch (engine/server.cu:356-361,377).  Any other
+ * call on the same pipe waits in the same way first. */
+int lmi_batch_wait(lmi_server *s, int pipe, void *stream);
 int lmi_batch_view_get(lmi_server *s, int pipe, lmi_batch_view *out);
 /* Synchronises `stream`, copies both headers to the host, reports a bad seed id. */
 int lmi_batch_counters(lmi_server *s, int pipe, void *stream, int32_t node_counter[16],

@@ -17,7 +17,7 @@ MAX_HOPS, MAX_FANOUT, MAX_PIPES = 3, 64, 4
 F32, F16 = 0, 1
 LOC_HOST, LOC_DEVICE = 0, 1
 MODE_TRAIN, MODE_VALID, MODE_TEST = 0, 1, 2
-TABLE_HASH, TABLE_DIRECT = 0, 1
+TABLE_HASH, TABLE_DIRECT, TABLE_RANK = 0, 1, 2
 CACHE_NONE, CACHE_STATIC, CACHE_LRU, CACHE_INT8 = 0, 1, 2, 3
 
 # every symbol include/legion_mi.h declares
@@ -29,7 +29,7 @@ ABI_SYMBOLS = [
     "lmi_idset_load", "lmi_cache_build_static", "lmi_cache_build_lru", "lmi_cache_build_int8",
     "lmi_cache_info_get", "lmi_cache_dump", "lmi_op_batch_generate", "lmi_op_random_sample",
     "lmi_op_cache_lookup", "lmi_op_io_submit", "lmi_op_io_complete", "lmi_run_once",
-    "lmi_batch_view_get", "lmi_batch_counters", "lmi_steps_per_epoch", "lmi_profile_enable",
+    "lmi_batch_wait", "lmi_batch_view_get", "lmi_batch_counters", "lmi_steps_per_epoch", "lmi_profile_enable",
     "lmi_profile_read", "lmi_tune", "lmi_bench_copy", "lmi_synth_graph", "lmi_synth_trainset",
     "lmi_synth_features",
 ]
@@ -108,6 +108,7 @@ def lib():
         L.lmi_op_io_complete.argtypes = [C.c_void_p, C.c_int, C.c_void_p]
         L.lmi_run_once.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int32, C.c_int, C.c_int32,
                                    C.c_int, C.c_uint64]
+        L.lmi_batch_wait.argtypes = [C.c_void_p, C.c_int, C.c_void_p]
         L.lmi_batch_view_get.argtypes = [C.c_void_p, C.c_int, C.POINTER(BatchView)]
         L.lmi_batch_counters.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         L.lmi_steps_per_epoch.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_int32)]
@@ -254,6 +255,9 @@ class Server:
         check(lib().lmi_run_once(self.h, pipe, stream, p, n, LOC_HOST, batch_counter, mode, rng_seed))
 
     # outputs -----------------------------------------------------------------
+    def batch_wait(self, pipe=0, stream=None):
+        check(lib().lmi_batch_wait(self.h, pipe, stream))
+
     def counters(self, pipe=0, stream=None):
         nc = np.zeros(16, np.int32)
         ec = np.zeros(16, np.int32)

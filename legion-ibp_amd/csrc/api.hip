@@ -35,6 +35,8 @@ static hipEvent_t prof_event(Server *s) {
 int prof_begin(Server *s, hipStream_t st, int kind) {
   if (!s->prof_on) return -1;
   EventPair p{prof_event(s), prof_event(s), kind};
+  s->prof_used.push_back(p.a);
+  s->prof_used.push_back(p.b);
   (void)hipEventRecord(p.a, st);
   s->prof_events.push_back(p);
   return (int)s->prof_events.size() - 1;
@@ -44,6 +46,23 @@ int prof_end(Server *s, hipStream_t st, int handle) {
   if (handle < 0) return LMI_OK;
   (void)hipEventRecord(s->prof_events[handle].b, st);
   return LMI_OK;
+}
+
+void prof_phase(Server *s, hipStream_t st, int next_kind) {
+  if (!s->prof_on) {
+    s->prof_open = -1;
+    return;
+  }
+  if (s->prof_open < 0 && next_kind < 0) return;
+  hipEvent_t e = prof_event(s);
+  s->prof_used.push_back(e);
+  (void)hipEventRecord(e, st);
+  if (s->prof_open >= 0) s->prof_events[s->prof_open].b = e;
+  s->prof_open = -1;
+  if (next_kind >= 0) {
+    s->prof_events.push_back(EventPair{e, nullptr, next_kind});
+    s->prof_open = (int)s->prof_events.size() - 1;
+  }
 }
 
 static void prof_snapshot(Server *s, Pipe &p, hipStream_t st) {
@@ -66,9 +85,11 @@ static int dmalloc(T **p, int64_t count) {
 static void pipe_free(Pipe &p) {
   void *ptrs[] = {p.ids, p.features, p.labels, p.agg_src_ids, p.agg_src_off, p.agg_dst_off, p.blk_indptr[0],
                   p.blk_indptr[1], p.blk_indptr[2], p.cache_index, p.st, p.dedup.slots, p.eslot, p.firstv,
-                  p.cnt, p.rank, p.tile_sums, p.hit_list, p.miss_list, p.lru_fill};
+                  p.cnt, p.rank, p.tile_sums, p.miss_list, p.lru_fill, p.seed_stage};
   for (void *q : ptrs)
     if (q) (void)hipFree(q);
+  if (p.graph_exec) (void)hipGraphExecDestroy(p.graph_exec);
+  if (p.graph) (void)hipGraphDestroy(p.graph);
   if (p.side) (void)hipStreamDestroy(p.side);
   if (p.fork) (void)hipEventDestroy(p.fork);
   if (p.join) (void)hipEventDestroy(p.join);
@@ -96,18 +117,30 @@ static int pipe_alloc(Server *s, Pipe &p) {
   LMI_TRY(dmalloc(&p.cnt, scan_n + 1));
   LMI_TRY(dmalloc(&p.rank, s->max_edges_hop + 1));
   LMI_TRY(dmalloc(&p.tile_sums, ceil_div(scan_n, 2048) + 1));
-  LMI_TRY(dmalloc(&p.hit_list, s->max_nodes));
   LMI_TRY(dmalloc(&p.miss_list, s->max_nodes));
   LMI_TRY(dmalloc(&p.lru_fill, s->max_nodes));
+  LMI_TRY(dmalloc(&p.seed_stage, s->cfg.batch_size));
   LMI_HIP(hipStreamCreateWithFlags(&p.side, hipStreamNonBlocking));
   LMI_HIP(hipEventCreateWithFlags(&p.fork, hipEventDisableTiming));
   LMI_HIP(hipEventCreateWithFlags(&p.join, hipEventDisableTiming));
   return LMI_OK;
 }
 
-static __global__ void copy_kernel(const uint4 *__restrict__ src, uint4 *__restrict__ dst, size_t n) {
-  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x)
-    dst[i] = src[i];
+// Streaming copy, four 16-byte vectors in flight per lane: the measured HBM ceiling.
+typedef uint32_t cp_u32x4 __attribute__((ext_vector_type(4)));
+static __global__ __launch_bounds__(256) void copy_kernel(const cp_u32x4 *__restrict__ src, cp_u32x4 *__restrict__ dst,
+                                                          size_t n) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  for (; i + 3 * stride < n; i += 4 * stride) {
+    const cp_u32x4 a = __builtin_nontemporal_load(src + i), b = __builtin_nontemporal_load(src + i + stride),
+                   c = __builtin_nontemporal_load(src + i + 2 * stride), d = __builtin_nontemporal_load(src + i + 3 * stride);
+    __builtin_nontemporal_store(a, dst + i);
+    __builtin_nontemporal_store(b, dst + i + stride);
+    __builtin_nontemporal_store(c, dst + i + 2 * stride);
+    __builtin_nontemporal_store(d, dst + i + 3 * stride);
+  }
+  for (; i < n; i += stride) dst[i] = src[i];
 }
 
 }  // namespace lmi
@@ -187,10 +220,7 @@ int lmi_server_destroy(lmi_server *h) {
     if (s->set_ids[m]) (void)hipFree(s->set_ids[m]);
     if (s->set_labels[m]) (void)hipFree(s->set_labels[m]);
   }
-  for (auto &e : s->prof_events) {
-    (void)hipEventDestroy(e.a);
-    (void)hipEventDestroy(e.b);
-  }
+  for (auto &e : s->prof_used) (void)hipEventDestroy(e);
   for (auto &e : s->prof_free) (void)hipEventDestroy(e);
   if (s->prof_ring) (void)hipHostFree(s->prof_ring);
   if (s->d_scalar) (void)hipFree(s->d_scalar);
@@ -347,6 +377,7 @@ int lmi_cache_info_get(lmi_server *h, lmi_cache_info *out) {
   out->row_bytes = s->cache_row_bytes;
   out->table_bytes = s->cache_kind == LMI_CACHE_LRU ? s->cache_rows * 8
                      : s->table_kind == LMI_TABLE_DIRECT ? (s->slot_of ? s->n_nodes * 4 : 0)
+                     : s->table_kind == LMI_TABLE_RANK ? (s->rank_tab ? ceil_div(s->n_nodes, 64) * 16 : 0)
                                                          : (int64_t)s->id_table.bytes();
   out->n_sets = s->lru_sets;
   out->ways = s->lru_ways;
@@ -366,22 +397,17 @@ static int ready(Server *s) {
   return LMI_OK;
 }
 
-int lmi_op_batch_generate(lmi_server *h, int pipe, void *stream, const int32_t *seeds, int32_t n, int seeds_location,
-                          int32_t batch_counter, int mode, uint64_t rng_seed) {
-  Server *s = reinterpret_cast<Server *>(h);
-  LMI_TRY(check_pipe(s, pipe));
+// Resolves where this batch's seeds live and the per-batch scalars.
+static int batch_params(Server *s, Pipe &p, hipStream_t st, const int32_t *seeds, int32_t n, int seeds_location,
+                        int32_t batch_counter, int mode, uint64_t rng_seed, BatchParams *bp) {
   LMI_TRY(ready(s));
-  Pipe &p = s->pipes[pipe];
-  hipStream_t st = (hipStream_t)stream;
-  const int32_t *d_seeds = nullptr, *d_labels = nullptr;
+  bp->labels = nullptr;
   if (seeds) {
     if (n < 0 || n > s->cfg.batch_size) LMI_FAIL(LMI_ERR_CAPACITY, "%d seeds exceed batch_size %d", n, s->cfg.batch_size);
-    if (seeds_location == LMI_LOC_DEVICE) d_seeds = seeds;
+    if (seeds_location == LMI_LOC_DEVICE) bp->seeds = seeds;
     else {
-      // stage through the scan scratch, which the first hop only writes after the seeds are consumed
-      int32_t *stage = p.cnt;
-      LMI_HIP(hipMemcpyAsync(stage, seeds, (size_t)n * 4, hipMemcpyHostToDevice, st));
-      d_seeds = stage;
+      if (n) LMI_HIP(hipMemcpyAsync(p.seed_stage, seeds, (size_t)n * 4, hipMemcpyHostToDevice, st));
+      bp->seeds = p.seed_stage;
     }
   } else {
     // slice `batch_counter` of the id set (batch_generate, operator_impl.cu:40-53); a short last
@@ -390,12 +416,26 @@ int lmi_op_batch_generate(lmi_server *h, int pipe, void *stream, const int32_t *
     const int64_t off = (int64_t)batch_counter * s->cfg.batch_size;
     if (batch_counter < 0 || off >= s->set_n[mode]) LMI_FAIL(LMI_ERR_ARG, "batch %d is past the end of id set %d", batch_counter, mode);
     n = (int32_t)std::min<int64_t>(s->cfg.batch_size, s->set_n[mode] - off);
-    d_seeds = s->set_ids[mode] + off;
-    if (s->set_labels[mode]) d_labels = s->set_labels[mode] + off;
+    bp->seeds = s->set_ids[mode] + off;
+    if (s->set_labels[mode]) bp->labels = s->set_labels[mode] + off;
   }
-  p.rng_seed = rng_seed ? rng_seed : s->cfg.seed + (uint64_t)(uint32_t)batch_counter;
+  bp->n_seeds = n;
+  bp->rng_seed = rng_seed ? rng_seed : s->cfg.seed + (uint64_t)(uint32_t)batch_counter;
   if (s->cache_kind == LMI_CACHE_LRU) ++s->lru_tick;
-  return launch_batch_generate(s, p, st, d_seeds, n, d_labels);
+  bp->lru_tick = s->lru_tick;
+  return LMI_OK;
+}
+
+int lmi_op_batch_generate(lmi_server *h, int pipe, void *stream, const int32_t *seeds, int32_t n, int seeds_location,
+                          int32_t batch_counter, int mode, uint64_t rng_seed) {
+  Server *s = reinterpret_cast<Server *>(h);
+  LMI_TRY(check_pipe(s, pipe));
+  Pipe &p = s->pipes[pipe];
+  hipStream_t st = (hipStream_t)stream;
+  BatchParams bp{};
+  LMI_TRY(pipe_join(p, st));
+  LMI_TRY(batch_params(s, p, st, seeds, n, seeds_location, batch_counter, mode, rng_seed, &bp));
+  return launch_batch_generate(s, p, st, bp);
 }
 
 int lmi_op_random_sample(lmi_server *h, int pipe, void *stream, int hop) {
@@ -405,9 +445,9 @@ int lmi_op_random_sample(lmi_server *h, int pipe, void *stream, int hop) {
   Pipe &p = s->pipes[pipe];
   if (hop != p.hops_done || hop >= s->cfg.hops) LMI_FAIL(LMI_ERR_ARG, "hop %d out of order (next is %d)", hop, p.hops_done);
   hipStream_t st = (hipStream_t)stream;
-  int hnd = prof_begin(s, st, PROF_SAMPLE);
+  prof_phase(s, st, PROF_SAMPLE);
   LMI_TRY(launch_hop(s, p, st, hop));
-  prof_end(s, st, hnd);
+  prof_phase(s, st, -1);
   return LMI_OK;
 }
 
@@ -418,8 +458,12 @@ int lmi_op_cache_lookup(lmi_server *h, int pipe, void *stream, int segment) {
   Pipe &p = s->pipes[pipe];
   if (segment < 0 || segment > p.hops_done) LMI_FAIL(LMI_ERR_ARG, "segment %d not sampled yet", segment);
   hipStream_t st = (hipStream_t)stream;
+  LMI_TRY(pipe_join(p, st));
+  prof_phase(s, st, PROF_LOOKUP);
   LMI_TRY(launch_lookup(s, p, st, segment, segment));
-  return launch_gather_seg(s, p, st, segment, segment);
+  LMI_TRY(launch_gather_seg(s, p, st, segment, segment));
+  prof_phase(s, st, -1);
+  return LMI_OK;
 }
 
 int lmi_op_io_submit(lmi_server *h, int pipe, void *stream) {
@@ -432,8 +476,42 @@ int lmi_op_io_complete(lmi_server *h, int pipe, void *stream) {
   LMI_TRY(check_pipe(s, pipe));
   Pipe &p = s->pipes[pipe];
   hipStream_t st = (hipStream_t)stream;
+  LMI_TRY(pipe_join(p, st));
   LMI_TRY(launch_lru_insert(s, p, st, s->cfg.hops + 1));
   prof_snapshot(s, p, st);
+  return LMI_OK;
+}
+
+// Captures begin + hops + lookup of one pipe into a HIP graph.  Every kernel in it
+// reads its sizes and per-batch scalars from the pipe's DevState, so a replay only
+// needs the first node (batch_begin_kernel) re-pointed at the new batch.
+static int capture_batch_graph(Server *s, Pipe &p, hipStream_t st, const BatchParams &bp) {
+  const bool prof = s->prof_on;
+  s->prof_on = false;  // no event records inside the capture
+  LMI_HIP(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
+  int rc = launch_batch_generate(s, p, st, bp);
+  for (int k = 0; rc == LMI_OK && k < s->cfg.hops; ++k) rc = launch_hop(s, p, st, k);
+  if (rc == LMI_OK) rc = launch_lookup(s, p, st, 0, s->cfg.hops);
+  hipGraph_t g = nullptr;
+  const hipError_t e = hipStreamEndCapture(st, &g);
+  s->prof_on = prof;
+  if (rc != LMI_OK) {
+    if (g) (void)hipGraphDestroy(g);
+    return rc;
+  }
+  LMI_HIP(e);
+  size_t n_roots = 1;
+  hipGraphNode_t root = nullptr;
+  LMI_HIP(hipGraphGetRootNodes(g, &root, &n_roots));
+  hipGraphNodeType ty;
+  LMI_HIP(hipGraphNodeGetType(root, &ty));
+  if (n_roots != 1 || ty != hipGraphNodeTypeKernel) {
+    (void)hipGraphDestroy(g);
+    LMI_FAIL(LMI_ERR_HIP, "captured batch graph has an unexpected shape (%zu roots)", n_roots);
+  }
+  LMI_HIP(hipGraphInstantiate(&p.graph_exec, g, nullptr, nullptr, 0));
+  p.graph = g;
+  p.begin_node = root;
   return LMI_OK;
 }
 
@@ -444,17 +522,30 @@ int lmi_run_once(lmi_server *h, int pipe, void *stream, const int32_t *seeds, in
   if (!s->feat) LMI_FAIL(LMI_ERR_STATE, "no features attached");
   Pipe &p = s->pipes[pipe];
   hipStream_t st = (hipStream_t)stream;
-  int hb = prof_begin(s, st, PROF_BATCH);
-  LMI_TRY(lmi_op_batch_generate(h, pipe, stream, seeds, n, seeds_location, batch_counter, mode, rng_seed));
-  int hs = prof_begin(s, st, PROF_SAMPLE);
-  for (int k = 0; k < s->cfg.hops; ++k) LMI_TRY(launch_hop(s, p, st, k));
-  prof_end(s, st, hs);
-  LMI_TRY(launch_lookup(s, p, st, 0, s->cfg.hops));
+  BatchParams bp{};
+  LMI_TRY(batch_params(s, p, st, seeds, n, seeds_location, batch_counter, mode, rng_seed, &bp));
+  LMI_TRY(pipe_join(p, st));  // the previous batch of this pipe may still be gathering misses
+  prof_phase(s, st, PROF_SAMPLE);
+  if (s->use_graph && st != nullptr) {  // the legacy default stream cannot be captured
+    if (!p.graph_exec) LMI_TRY(capture_batch_graph(s, p, st, bp));
+    LMI_TRY(graph_update_begin(s, p, bp));
+    LMI_HIP(hipGraphLaunch(p.graph_exec, st));
+  } else {
+    LMI_TRY(launch_batch_generate(s, p, st, bp));
+    for (int k = 0; k < s->cfg.hops; ++k) LMI_TRY(launch_hop(s, p, st, k));
+    LMI_TRY(launch_lookup(s, p, st, 0, s->cfg.hops));
+  }
   LMI_TRY(launch_gather_seg(s, p, st, 0, s->cfg.hops));
   LMI_TRY(launch_lru_insert(s, p, st, 1));
-  prof_end(s, st, hb);
+  prof_phase(s, st, -1);
   prof_snapshot(s, p, st);
   return LMI_OK;
+}
+
+int lmi_batch_wait(lmi_server *h, int pipe, void *stream) {
+  Server *s = reinterpret_cast<Server *>(h);
+  LMI_TRY(check_pipe(s, pipe));
+  return pipe_join(s->pipes[pipe], (hipStream_t)stream);
 }
 
 // ------------------------------------------------------------------ outputs
@@ -483,6 +574,7 @@ int lmi_batch_counters(lmi_server *h, int pipe, void *stream, int32_t node_count
   Server *s = reinterpret_cast<Server *>(h);
   LMI_TRY(check_pipe(s, pipe));
   DevState hs;
+  LMI_TRY(pipe_join(s->pipes[pipe], (hipStream_t)stream));
   LMI_HIP(hipStreamSynchronize((hipStream_t)stream));
   LMI_HIP(hipMemcpy(&hs, s->pipes[pipe].st, sizeof(DevState), hipMemcpyDeviceToHost));
   if (node_counter) memcpy(node_counter, hs.node_counter, 64);
@@ -512,27 +604,27 @@ int lmi_profile_read(lmi_server *h, lmi_profile *out, int reset) {
   LMI_HIP(hipDeviceSynchronize());
   for (auto &e : s->prof_events) {
     float ms = 0.0f;
-    if (hipEventElapsedTime(&ms, e.a, e.b) == hipSuccess) {
+    if (e.b && hipEventElapsedTime(&ms, e.a, e.b) == hipSuccess) {
       switch (e.kind) {
         case PROF_GATHER_HIT: s->prof.gather_hit_ms += ms; s->prof.gather_hit_launches++; break;
         case PROF_GATHER_MISS: s->prof.gather_miss_ms += ms; s->prof.gather_miss_launches++; break;
         case PROF_SAMPLE: s->prof.sample_ms += ms; s->prof.sample_launches++; break;
         case PROF_LOOKUP: s->prof.lookup_ms += ms; s->prof.lookup_launches++; break;
-        case PROF_BATCH: s->prof.batch_ms += ms; s->prof.batches++; break;
       }
     } else {
       (void)hipGetLastError();
     }
-    s->prof_free.push_back(e.a);
-    s->prof_free.push_back(e.b);
   }
+  for (auto &ev : s->prof_used) s->prof_free.push_back(ev);
+  s->prof_used.clear();
+  s->prof_open = -1;
   s->prof_events.clear();
   for (int i = 0; i < s->prof_ring_n; ++i) {
     const DevState &d = s->prof_ring[i];
-    for (int k = 0; k <= LMI_MAX_HOPS; ++k) {
-      s->prof.gather_hit_rows += d.n_hit[k];
-      s->prof.gather_miss_rows += d.n_miss[k];
-    }
+    int64_t miss = 0;
+    for (int k = 0; k <= LMI_MAX_HOPS; ++k) miss += d.n_miss[k];
+    s->prof.gather_miss_rows += miss;
+    s->prof.gather_hit_rows += (int64_t)d.node_counter[7] - miss;
   }
   s->prof_ring_n = 0;
   *out = s->prof;
@@ -549,6 +641,9 @@ int lmi_tune(lmi_server *h, const char *key, int64_t value) {
   else if (!strcmp(key, "gather_nontemporal")) s->gather_nt = (int)value;
   else if (!strcmp(key, "lds_dedup")) s->lds_dedup = (int)value;
   else if (!strcmp(key, "split_miss")) s->split_miss = (int)value;
+  else if (!strcmp(key, "use_graph")) s->use_graph = (int)value;
+  else if (!strcmp(key, "miss_blocks")) s->miss_blocks = (int)value;
+  else if (!strcmp(key, "miss_unroll")) s->miss_unroll = (int)value;
   else LMI_FAIL(LMI_ERR_ARG, "unknown tuning key '%s'", key);
   return LMI_OK;
 }
@@ -563,10 +658,10 @@ int lmi_bench_copy(size_t bytes, int repeats, double *ms_per_copy) {
   LMI_HIP(hipEventCreate(&e0));
   LMI_HIP(hipEventCreate(&e1));
   const size_t n = bytes / 16;
-  hipLaunchKernelGGL(copy_kernel, dim3(4096), dim3(256), 0, 0, (const uint4 *)a, (uint4 *)b, n);
+  hipLaunchKernelGGL(copy_kernel, dim3(2048), dim3(256), 0, 0, (const cp_u32x4 *)a, (cp_u32x4 *)b, n);
   LMI_HIP(hipEventRecord(e0, 0));
   for (int r = 0; r < repeats; ++r)
-    hipLaunchKernelGGL(copy_kernel, dim3(4096), dim3(256), 0, 0, (const uint4 *)a, (uint4 *)b, n);
+    hipLaunchKernelGGL(copy_kernel, dim3(2048), dim3(256), 0, 0, (const cp_u32x4 *)a, (cp_u32x4 *)b, n);
   LMI_HIP(hipEventRecord(e1, 0));
   LMI_HIP(hipEventSynchronize(e1));
   float ms = 0;

@@ -21,19 +21,23 @@
 namespace lmi {
 
 // ------------------------------------------------------------------ gather
-// Generic row mover.  Row j of the work list names output row i = list[j] (or j);
-// its source row is src_index[i] (or i) and its destination row dst_index[i]
-// (or i); a negative source or destination skips the row.  LPR lanes cooperate
-// on a row, each moving sizeof(V) bytes per step, with U rows in flight.
+// Generic row mover over work items j in [*first_ptr, *n_ptr).  Entry j of the work
+// list is a pair (output row i, source row); without a list i = j.  With SRC_FROM_LIST the source row is the pair's
+// second word, so the only dependent load in front of the row itself is the pair;
+// otherwise it is src_index[i] (or i).  The destination row is dst_index[i] (or
+// i); a negative source or destination skips the row.  LPR lanes cooperate on a
+// row, each moving sizeof(V) bytes per step, with U rows in flight per lane.
 template <typename V, int LPR, int U, bool NT>
 static __global__ __launch_bounds__(256) void move_rows_kernel(
-    const int32_t *list, const int32_t *n_ptr, const int32_t *src_index, const int32_t *dst_index,
-    const uint8_t *src, uint8_t *dst, int chunks, int64_t src_row_bytes, int64_t dst_row_bytes) {
+    const int2 *list, const int32_t *first_ptr, const int32_t *n_ptr, const int32_t *src_index,
+    const int32_t *dst_index, int src_from_list, const uint8_t *src, uint8_t *dst, int chunks,
+    int64_t src_row_bytes, int64_t dst_row_bytes) {
   const int n = *n_ptr;
+  const int first = first_ptr ? *first_ptr : 0;
   const int lane = threadIdx.x & (LPR - 1);
   const int group = (blockIdx.x * blockDim.x + threadIdx.x) / LPR;
   const int n_groups = gridDim.x * blockDim.x / LPR;
-  for (int j0 = group; j0 < n; j0 += n_groups * U) {
+  for (int j0 = first + group; j0 < n; j0 += n_groups * U) {
     int64_t so[U], dofs[U];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
@@ -41,8 +45,13 @@ static __global__ __launch_bounds__(256) void move_rows_kernel(
       so[u] = -1;
       dofs[u] = -1;
       if (j < n) {
-        const int i = list ? list[j] : j;
-        const int si = src_index ? src_index[i] : i;
+        int i = j, si;
+        if (list) {
+          const int2 pr = list[j];
+          i = pr.x;
+          si = pr.y;
+        }
+        if (!list || !src_from_list) si = src_index ? src_index[i] : i;
         const int di = dst_index ? dst_index[i] : i;
         if (si >= 0 && di >= 0) {
           so[u] = (int64_t)si * src_row_bytes;
@@ -54,7 +63,7 @@ static __global__ __launch_bounds__(256) void move_rows_kernel(
       V v[U];
 #pragma unroll
       for (int u = 0; u < U; ++u)
-        if (so[u] >= 0) v[u] = *reinterpret_cast<const V *>(src + so[u] + (int64_t)c * sizeof(V));
+        if (so[u] >= 0) v[u] = __builtin_nontemporal_load(reinterpret_cast<const V *>(src + so[u] + (int64_t)c * sizeof(V)));
 #pragma unroll
       for (int u = 0; u < U; ++u)
         if (so[u] >= 0) {
@@ -70,7 +79,11 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 struct MoveArgs {
-  const int32_t *list, *n_ptr, *src_index, *dst_index;
+  const int2 *list;
+  const int32_t *first_ptr, *n_ptr, *src_index, *dst_index;
+  int src_from_list;
+  int max_blocks;  // 0 = fill the device
+  int unroll;      // 0 = the server's gather_unroll
   const uint8_t *src;
   uint8_t *dst;
   int64_t src_row_bytes, dst_row_bytes, row_bytes;  // row_bytes = bytes moved per row
@@ -81,11 +94,11 @@ template <typename V, int LPR, int U>
 static void launch_move_vlu(hipStream_t st, const MoveArgs &a, int grid, bool nt) {
   const int chunks = (int)(a.row_bytes / sizeof(V));
   if (nt)
-    hipLaunchKernelGGL((move_rows_kernel<V, LPR, U, true>), dim3(grid), dim3(256), 0, st, a.list, a.n_ptr,
-                       a.src_index, a.dst_index, a.src, a.dst, chunks, a.src_row_bytes, a.dst_row_bytes);
+    hipLaunchKernelGGL((move_rows_kernel<V, LPR, U, true>), dim3(grid), dim3(256), 0, st, a.list, a.first_ptr, a.n_ptr,
+                       a.src_index, a.dst_index, a.src_from_list, a.src, a.dst, chunks, a.src_row_bytes, a.dst_row_bytes);
   else
-    hipLaunchKernelGGL((move_rows_kernel<V, LPR, U, false>), dim3(grid), dim3(256), 0, st, a.list, a.n_ptr,
-                       a.src_index, a.dst_index, a.src, a.dst, chunks, a.src_row_bytes, a.dst_row_bytes);
+    hipLaunchKernelGGL((move_rows_kernel<V, LPR, U, false>), dim3(grid), dim3(256), 0, st, a.list, a.first_ptr, a.n_ptr,
+                       a.src_index, a.dst_index, a.src_from_list, a.src, a.dst, chunks, a.src_row_bytes, a.dst_row_bytes);
 }
 
 template <typename V, int LPR>
@@ -122,10 +135,10 @@ static int launch_move_rows(Server *s, hipStream_t st, const MoveArgs &a, bool n
     lpr = 8;
     while (lpr < chunks && lpr < 64) lpr <<= 1;
   }
-  const int unroll = s->gather_unroll;
+  const int unroll = a.unroll > 0 ? a.unroll : s->gather_unroll;
   const int64_t groups_per_block = 256 / lpr;
   int64_t want = ceil_div(a.n_max, groups_per_block * (unroll > 0 ? unroll : 1));
-  int64_t cap = s->gather_blocks > 0 ? s->gather_blocks : (int64_t)s->n_cu * 8;
+  int64_t cap = a.max_blocks > 0 ? a.max_blocks : s->gather_blocks > 0 ? s->gather_blocks : (int64_t)s->n_cu * 8;
   const int grid = (int)std::max<int64_t>(1, std::min(want, cap));
   if (vec == 16) launch_move_v<u32x4>(st, a, grid, nt, unroll, lpr);
   else if (vec == 8) launch_move_v<u32x2>(st, a, grid, nt, unroll, lpr);
@@ -169,15 +182,15 @@ static __global__ __launch_bounds__(256) void quantize_rows_kernel(
 // y = float(q) * scale, rounded to the output type (RNE for fp16).
 template <typename OUT, int LPR>
 static __global__ __launch_bounds__(256) void gather_int8_kernel(
-    const int32_t *list, const int32_t *n_ptr, const int32_t *cache_index, const int8_t *q,
+    const int32_t *first_ptr, const int32_t *n_ptr, const int32_t *cache_index, const int8_t *q,
     const float *scale, OUT *out, int dim) {
   const int n = *n_ptr;
+  const int first = first_ptr ? *first_ptr : 0;
   const int lane = threadIdx.x & (LPR - 1);
   const int group = (blockIdx.x * blockDim.x + threadIdx.x) / LPR;
   const int n_groups = gridDim.x * blockDim.x / LPR;
   const int chunks = dim / 16;
-  for (int j = group; j < n; j += n_groups) {
-    const int i = list[j];
+  for (int i = first + group; i < n; i += n_groups) {
     const int slot = cache_index[i];
     if (slot < 0) continue;
     const float sc = scale[slot];
@@ -206,14 +219,14 @@ static __global__ __launch_bounds__(256) void gather_int8_kernel(
 // Element-wise fallback for row lengths that are not a multiple of 16.
 template <typename OUT>
 static __global__ __launch_bounds__(256) void gather_int8_generic_kernel(
-    const int32_t *list, const int32_t *n_ptr, const int32_t *cache_index, const int8_t *q,
+    const int32_t *first_ptr, const int32_t *n_ptr, const int32_t *cache_index, const int8_t *q,
     const float *scale, OUT *out, int dim) {
   const int n = *n_ptr;
+  const int first = first_ptr ? *first_ptr : 0;
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = (blockIdx.x * blockDim.x + threadIdx.x) / kWave;
   const int n_waves = gridDim.x * blockDim.x / kWave;
-  for (int j = wave; j < n; j += n_waves) {
-    const int i = list[j];
+  for (int i = first + wave; i < n; i += n_waves) {
     const int slot = cache_index[i];
     if (slot < 0) continue;
     const float sc = scale[slot];
@@ -233,56 +246,85 @@ struct LookupArgs {
   const HashSlot *slots;
   int log2cap;
   const int32_t *slot_of;
+  const uint4 *rank_tab;
   const int32_t *lru_keys;
   int32_t *lru_use;
   int64_t lru_sets;
-  int lru_ways, tick;
-  int32_t *cache_index, *hit_list, *miss_list, *lru_fill;
+  int lru_ways;
+  int32_t *cache_index, *lru_fill;
+  int2 *miss_list;
   DevState *st;
   int seg_first, seg_last, seg;
 };
 
-// id -> slot for rows [first, last) of the batch; rows are appended to the
-// segment's hit or miss list with one atomic per wavefront (ballot + prefix
-// popcount).  List order is arbitrary; it only schedules the gather.
-static __global__ __launch_bounds__(256) void lookup_kernel(LookupArgs a) {
+// Bitmap + rank table: the slot of a cached node is the number of cached nodes
+// with a smaller id = rank at the start of its 64-id word + set bits below it.
+__device__ __forceinline__ int32_t rank_find(const uint4 *tab, int32_t id) {
+  const uint4 e = tab[id >> 6];
+  const uint64_t bits = (uint64_t)e.x | ((uint64_t)e.y << 32);
+  const int b = id & 63;
+  if (!((bits >> b) & 1ull)) return -1;
+  return (int32_t)e.z + __popcll(bits & ((1ull << b) - 1ull));
+}
+
+__device__ __forceinline__ int32_t static_find(int table_kind, const HashSlot *slots, int log2cap,
+                                               const int32_t *slot_of, const uint4 *rank_tab, int32_t id) {
+  if (table_kind == LMI_TABLE_RANK) return rank_find(rank_tab, id);
+  if (table_kind == LMI_TABLE_DIRECT) return slot_of[id];
+  return table_find(slots, log2cap, id);
+}
+
+// id -> slot for rows [first, last) of the batch -> cache_index[].  Rows that
+// miss are appended to the segment's miss list as (row, id) pairs: ballot +
+// prefix popcount inside each wavefront, one LDS pass over the 16 wavefronts of
+// the block, one atomic per block.  The HBM gather needs no list: it walks the
+// rows directly and skips the misses.  List order is arbitrary; it only
+// schedules the host-link gather.
+constexpr int kLookupBlock = 1024;
+static __global__ __launch_bounds__(kLookupBlock) void lookup_kernel(LookupArgs a) {
+  __shared__ int wave_cnt[kLookupBlock / kWave];
+  __shared__ int block_base;
   const int first = (a.seg_first == 0) ? 0 : a.st->node_counter[9 + a.seg_first - 1];
   const int last = a.st->node_counter[9 + a.seg_last];
-  const int lane = threadIdx.x & (kWave - 1);
-  const int wave0 = (blockIdx.x * blockDim.x + threadIdx.x) - lane;
+  const int lane = threadIdx.x & (kWave - 1), wid = threadIdx.x / kWave;
   const int stride = gridDim.x * blockDim.x;
-  for (int b = first + wave0; b < last; b += stride) {
-    const int i = b + lane;
-    bool valid = false;
-    int slot = -1;
+  for (int b = first + blockIdx.x * blockDim.x; b < last; b += stride) {
+    const int i = b + threadIdx.x;
+    bool miss = false;
+    int32_t id = -1;
     if (i < last) {
-      const int32_t id = a.ids[i];
-      valid = (id >= 0 && id < a.n_nodes);
-      if (valid) {
+      id = a.ids[i];
+      int slot = -1;
+      if (id >= 0 && id < a.n_nodes) {
         if (a.kind == LMI_CACHE_LRU) {
           const int64_t base = ((int64_t)id % a.lru_sets) * a.lru_ways;
           for (int w = 0; w < a.lru_ways; ++w)
             if (a.lru_keys[base + w] == id) slot = (int)(base + w);
-          if (slot >= 0) a.lru_use[slot] = a.tick;
+          if (slot >= 0) a.lru_use[slot] = a.st->lru_tick;
           a.lru_fill[i] = -1;
         } else if (a.kind != LMI_CACHE_NONE) {
-          slot = (a.table_kind == LMI_TABLE_DIRECT) ? a.slot_of[id] : table_find(a.slots, a.log2cap, id);
+          slot = static_find(a.table_kind, a.slots, a.log2cap, a.slot_of, a.rank_tab, id);
         }
+        miss = slot < 0;
       }
       a.cache_index[i] = slot;
     }
-    const bool hit = valid && slot >= 0, miss = valid && slot < 0;
-    const uint64_t hm = __ballot(hit), mm = __ballot(miss);
-    int hb = 0, mb = 0;
-    if (lane == 0) {
-      if (hm) hb = atomicAdd(&a.st->n_hit[a.seg], __popcll(hm));
-      if (mm) mb = atomicAdd(&a.st->n_miss[a.seg], __popcll(mm));
+    const uint64_t mm = __ballot(miss);
+    if (lane == 0) wave_cnt[wid] = __popcll(mm);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      int t = 0;
+#pragma unroll
+      for (int w = 0; w < kLookupBlock / kWave; ++w) {
+        const int c = wave_cnt[w];
+        wave_cnt[w] = t;
+        t += c;
+      }
+      block_base = t ? atomicAdd(&a.st->n_miss[a.seg], t) : 0;
     }
-    hb = __shfl(hb, 0, kWave);
-    mb = __shfl(mb, 0, kWave);
-    const uint64_t lt = lanemask_lt();
-    if (hit) a.hit_list[hb + __popcll(hm & lt)] = i;
-    if (miss) a.miss_list[mb + __popcll(mm & lt)] = i;
+    __syncthreads();
+    if (miss) a.miss_list[block_base + wave_cnt[wid] + __popcll(mm & lanemask_lt())] = make_int2(i, id);
+    __syncthreads();
   }
 }
 
@@ -297,14 +339,13 @@ int launch_lookup(Server *s, Pipe &p, hipStream_t st, int seg_first, int seg_las
   a.slots = s->id_table.slots;
   a.log2cap = s->id_table.log2cap;
   a.slot_of = s->slot_of;
+  a.rank_tab = s->rank_tab;
   a.lru_keys = s->lru_keys;
   a.lru_use = s->lru_use;
   a.lru_sets = s->lru_sets;
   a.lru_ways = s->lru_ways;
-  a.tick = s->lru_tick;
   a.cache_index = p.cache_index;
   const int64_t base = seg_list_base(s, seg_first);
-  a.hit_list = p.hit_list + base;
   a.miss_list = p.miss_list + base;
   a.lru_fill = p.lru_fill;
   a.st = p.st;
@@ -312,92 +353,106 @@ int launch_lookup(Server *s, Pipe &p, hipStream_t st, int seg_first, int seg_las
   a.seg_last = seg_last;
   a.seg = seg_first;
   const int64_t n_max = s->node_cap[seg_last];
-  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(n_max, 256), (int64_t)s->n_cu * 8));
-  int h = prof_begin(s, st, PROF_LOOKUP);
-  hipLaunchKernelGGL(lookup_kernel, dim3(grid), dim3(256), 0, st, a);
+  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(n_max, kLookupBlock), (int64_t)s->n_cu * 2));
+  hipLaunchKernelGGL(lookup_kernel, dim3(grid), dim3(kLookupBlock), 0, st, a);
   LMI_HIP(hipGetLastError());
-  prof_end(s, st, h);
   return LMI_OK;
 }
 
-// Gathers the rows of segment `seg`'s hit and miss lists into the pipe's feature
-// buffer.  Hits stream from HBM on `st`; misses stream over the host link on the
-// pipe's side stream so the two overlap; `st` waits for both.
+int pipe_join(Pipe &p, hipStream_t st) {
+  if (p.side_pending) {
+    LMI_HIP(hipStreamWaitEvent(st, p.join, 0));
+    p.side_pending = false;
+  }
+  return LMI_OK;
+}
+
+// Gathers the rows [first, last) of a segment into the pipe's feature buffer.
+// Cache hits stream from HBM on `st`.  Misses come over the host link; with
+// split_miss they run on the pipe's side stream AFTER the HBM gather (host-link
+// reads in flight beside it cut its bandwidth by more than half) and the caller's
+// stream does not wait for them here: the next call on this pipe, or
+// lmi_batch_wait, joins.  The LRU cache joins at once (its insert copies the rows).
 int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last) {
   const int64_t base = seg_list_base(s, seg);
   const int64_t n_max = s->node_cap[seg_last];
   const bool split = s->split_miss && s->feat_loc == LMI_LOC_HOST && s->cache_kind != LMI_CACHE_NONE;
   hipStream_t ms = split ? p.side : st;
-  if (split) {
-    LMI_HIP(hipEventRecord(p.fork, st));
-    LMI_HIP(hipStreamWaitEvent(p.side, p.fork, 0));
-  }
-  // misses: raw rows from the feature table
-  {
-    MoveArgs m{};
-    m.list = p.miss_list + base;
-    m.n_ptr = &p.st->n_miss[seg];
-    m.src_index = p.ids;
-    m.dst_index = nullptr;
-    m.src = s->feat;
-    m.dst = (uint8_t *)p.features;
-    m.src_row_bytes = m.dst_row_bytes = m.row_bytes = s->row_bytes;
-    m.n_max = n_max;
-    int h = prof_begin(s, ms, PROF_GATHER_MISS);
-    LMI_TRY(launch_move_rows(s, ms, m, s->gather_nt != 0));
-    prof_end(s, ms, h);
-  }
   if (s->cache_kind != LMI_CACHE_NONE) {
-    int h = prof_begin(s, st, PROF_GATHER_HIT);
+    prof_phase(s, st, PROF_GATHER_HIT);
     if (s->cache_kind == LMI_CACHE_INT8) {
       const int dim = s->cfg.feat_dim;
       const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(n_max, 4), (int64_t)s->n_cu * 8));
-      const int32_t *list = p.hit_list + base;
-      const int32_t *n_ptr = &p.st->n_hit[seg];
+      const int32_t *first_ptr = seg == 0 ? nullptr : &p.st->node_counter[9 + seg - 1];
+      const int32_t *n_ptr = &p.st->node_counter[9 + seg_last];
       const int8_t *q = (const int8_t *)s->cache_data;
       if (dim % 16 == 0) {
         const int chunks = dim / 16;
         if (s->cfg.feat_dtype == LMI_F16) {
           if (chunks <= 32)
-            hipLaunchKernelGGL((gather_int8_kernel<__half, 32>), dim3(grid), dim3(256), 0, st, list, n_ptr,
+            hipLaunchKernelGGL((gather_int8_kernel<__half, 32>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
                                p.cache_index, q, s->cache_scale, (__half *)p.features, dim);
           else
-            hipLaunchKernelGGL((gather_int8_kernel<__half, 64>), dim3(grid), dim3(256), 0, st, list, n_ptr,
+            hipLaunchKernelGGL((gather_int8_kernel<__half, 64>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
                                p.cache_index, q, s->cache_scale, (__half *)p.features, dim);
         } else {
           if (chunks <= 32)
-            hipLaunchKernelGGL((gather_int8_kernel<float, 32>), dim3(grid), dim3(256), 0, st, list, n_ptr,
+            hipLaunchKernelGGL((gather_int8_kernel<float, 32>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
                                p.cache_index, q, s->cache_scale, (float *)p.features, dim);
           else
-            hipLaunchKernelGGL((gather_int8_kernel<float, 64>), dim3(grid), dim3(256), 0, st, list, n_ptr,
+            hipLaunchKernelGGL((gather_int8_kernel<float, 64>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
                                p.cache_index, q, s->cache_scale, (float *)p.features, dim);
         }
       } else {
         if (s->cfg.feat_dtype == LMI_F16)
-          hipLaunchKernelGGL((gather_int8_generic_kernel<__half>), dim3(grid), dim3(256), 0, st, list, n_ptr,
+          hipLaunchKernelGGL((gather_int8_generic_kernel<__half>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
                              p.cache_index, q, s->cache_scale, (__half *)p.features, dim);
         else
-          hipLaunchKernelGGL((gather_int8_generic_kernel<float>), dim3(grid), dim3(256), 0, st, list, n_ptr,
+          hipLaunchKernelGGL((gather_int8_generic_kernel<float>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
                              p.cache_index, q, s->cache_scale, (float *)p.features, dim);
       }
       LMI_HIP(hipGetLastError());
     } else {
       MoveArgs m{};
-      m.list = p.hit_list + base;
-      m.n_ptr = &p.st->n_hit[seg];
+      m.list = nullptr;  // rows [first, n) directly; cache_index < 0 (a miss) skips the row
+      m.first_ptr = seg == 0 ? nullptr : &p.st->node_counter[9 + seg - 1];
+      m.n_ptr = &p.st->node_counter[9 + seg_last];
       m.src_index = p.cache_index;
-      m.dst_index = nullptr;
       m.src = s->cache_data;
       m.dst = (uint8_t *)p.features;
       m.src_row_bytes = m.dst_row_bytes = m.row_bytes = s->row_bytes;
       m.n_max = n_max;
       LMI_TRY(launch_move_rows(s, st, m, s->gather_nt != 0));
     }
-    prof_end(s, st, h);
+  }
+  // misses: raw rows from the feature table, on a small grid (the host link needs
+  // few bytes in flight)
+  MoveArgs m{};
+  m.list = p.miss_list + base;
+  m.n_ptr = &p.st->n_miss[seg];
+  m.src_from_list = 1;
+  m.src = s->feat;
+  m.dst = (uint8_t *)p.features;
+  m.src_row_bytes = m.dst_row_bytes = m.row_bytes = s->row_bytes;
+  m.n_max = n_max;
+  if (s->feat_loc == LMI_LOC_HOST) {
+    m.max_blocks = s->miss_blocks > 0 ? s->miss_blocks : s->n_cu;
+    m.unroll = s->miss_unroll;
   }
   if (split) {
+    prof_phase(s, st, -1);
+    LMI_HIP(hipEventRecord(p.fork, st));
+    LMI_HIP(hipStreamWaitEvent(p.side, p.fork, 0));
+    int h = prof_begin(s, ms, PROF_GATHER_MISS);
+    LMI_TRY(launch_move_rows(s, ms, m, s->gather_nt != 0));
+    prof_end(s, ms, h);
     LMI_HIP(hipEventRecord(p.join, p.side));
-    LMI_HIP(hipStreamWaitEvent(st, p.join, 0));
+    p.side_pending = true;
+    if (s->cache_kind == LMI_CACHE_LRU) LMI_TRY(pipe_join(p, st));
+  } else {
+    prof_phase(s, st, PROF_GATHER_MISS);
+    LMI_TRY(launch_move_rows(s, ms, m, s->gather_nt != 0));
+    prof_phase(s, st, -1);
   }
   return LMI_OK;
 }
@@ -410,19 +465,19 @@ int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last)
 // every set has granted all the ways it can.
 struct LruArgs {
   const int32_t *ids;
-  const int32_t *miss_list[LMI_MAX_HOPS + 1];
+  const int2 *miss_list[LMI_MAX_HOPS + 1];
   const DevState *st;
   int n_lists;
   int32_t *keys, *use, *claim_cur, *claim_next, *fill;
   int64_t sets;
-  int ways, tick, round, last_round;
+  int ways, round, last_round;
 };
 
 static __global__ __launch_bounds__(256) void lru_bid_kernel(LruArgs a) {
   for (int l = 0; l < a.n_lists; ++l) {
     const int n = a.st->n_miss[l];
     for (int j = blockIdx.x * blockDim.x + threadIdx.x; j < n; j += gridDim.x * blockDim.x) {
-      const int i = a.miss_list[l][j];
+      const int i = a.miss_list[l][j].x;
       atomicMin(&a.claim_cur[(int64_t)a.ids[i] % a.sets], i);
     }
   }
@@ -432,20 +487,21 @@ static __global__ __launch_bounds__(256) void lru_round_kernel(LruArgs a) {
   for (int l = 0; l < a.n_lists; ++l) {
     const int n = a.st->n_miss[l];
     for (int j = blockIdx.x * blockDim.x + threadIdx.x; j < n; j += gridDim.x * blockDim.x) {
-      const int i = a.miss_list[l][j];
+      const int i = a.miss_list[l][j].x;
       if (a.fill[i] != -1) continue;  // placed (>= 0) or refused (-2) earlier
       const int32_t id = a.ids[i];
       const int64_t set = (int64_t)id % a.sets;
       if (a.claim_cur[set] == i) {
         const int64_t base = set * a.ways;
         int best = -1, best_use = kIntMax;
+        const int tick = a.st->lru_tick;
         for (int w = 0; w < a.ways; ++w) {
           const int u = a.use[base + w];
-          if (u < a.tick && u < best_use) best = w, best_use = u;
+          if (u < tick && u < best_use) best = w, best_use = u;
         }
         if (best >= 0) {
           a.keys[base + best] = id;
-          a.use[base + best] = a.tick;
+          a.use[base + best] = tick;
           a.fill[i] = (int)(base + best);
         } else {
           a.fill[i] = -2;
@@ -470,7 +526,6 @@ int launch_lru_insert(Server *s, Pipe &p, hipStream_t st, int n_lists) {
   a.fill = p.lru_fill;
   a.sets = s->lru_sets;
   a.ways = s->lru_ways;
-  a.tick = s->lru_tick;
   const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(s->max_nodes, 256), (int64_t)s->n_cu * 4));
   a.claim_cur = s->lru_claim[0];
   a.claim_next = s->lru_claim[1];
@@ -489,6 +544,7 @@ int launch_lru_insert(Server *s, Pipe &p, hipStream_t st, int n_lists) {
     m.list = p.miss_list + seg_list_base(s, l);
     m.n_ptr = &p.st->n_miss[l];
     m.src_index = nullptr;
+    m.src_from_list = 0;
     m.dst_index = p.lru_fill;
     m.src = (const uint8_t *)p.features;
     m.dst = s->cache_data;
@@ -564,6 +620,19 @@ static __global__ __launch_bounds__(256) void publish_slots_kernel(const int32_t
   }
 }
 
+// One thread per 64-id word of the bitmap + rank table.
+static __global__ __launch_bounds__(256) void publish_rank_kernel(const int32_t *member, const int32_t *slot,
+                                                                  int64_t n, uint4 *tab) {
+  const int64_t n_words = (n + 63) / 64;
+  for (int64_t w = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; w < n_words; w += (int64_t)gridDim.x * blockDim.x) {
+    uint64_t bits = 0;
+    const int64_t v0 = w * 64;
+    for (int b = 0; b < 64 && v0 + b < n; ++b)
+      if (member[v0 + b]) bits |= 1ull << b;
+    tab[w] = make_uint4((uint32_t)bits, (uint32_t)(bits >> 32), (uint32_t)slot[v0], 0u);
+  }
+}
+
 static __global__ void fill_i32_kernel(int32_t *p, int64_t n, int32_t v) {
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
     p[i] = v;
@@ -587,6 +656,7 @@ void cache_free(Server *s) {
   if (s->cache_scale) (void)hipFree(s->cache_scale);
   if (s->id_table.slots) (void)hipFree(s->id_table.slots);
   if (s->slot_of) (void)hipFree(s->slot_of);
+  if (s->rank_tab) (void)hipFree(s->rank_tab);
   if (s->lru_keys) (void)hipFree(s->lru_keys);
   if (s->lru_use) (void)hipFree(s->lru_use);
   if (s->lru_claim[0]) (void)hipFree(s->lru_claim[0]);
@@ -595,6 +665,7 @@ void cache_free(Server *s) {
   s->cache_scale = nullptr;
   s->id_table = Table{};
   s->slot_of = nullptr;
+  s->rank_tab = nullptr;
   s->lru_keys = s->lru_use = s->lru_claim[0] = s->lru_claim[1] = nullptr;
   s->cache_kind = LMI_CACHE_NONE;
   s->cache_rows = 0;
@@ -616,7 +687,8 @@ static int count_ge(const Server *s, int64_t thr, unsigned long long *d_pair, in
 // slot(v) = number of cached nodes with a smaller id.
 int cache_build_static(Server *s, int64_t capacity_rows, int table_kind, bool int8) {
   if (!s->indptr || !s->feat) LMI_FAIL(LMI_ERR_STATE, "load the graph and attach features before building a cache");
-  if (table_kind != LMI_TABLE_HASH && table_kind != LMI_TABLE_DIRECT) LMI_FAIL(LMI_ERR_ARG, "bad table kind");
+  if (table_kind != LMI_TABLE_HASH && table_kind != LMI_TABLE_DIRECT && table_kind != LMI_TABLE_RANK)
+    LMI_FAIL(LMI_ERR_ARG, "bad table kind");
   if (s->n_nodes >= (int64_t(1) << 31) - kScanTile) LMI_FAIL(LMI_ERR_CAPACITY, "too many nodes");
   cache_free(s);
   const int64_t N = s->n_nodes;
@@ -669,8 +741,11 @@ int cache_build_static(Server *s, int64_t capacity_rows, int table_kind, bool in
     s->id_table.log2cap = lg;
     LMI_HIP(hipMalloc(&s->id_table.slots, size_t(8) << lg));
     LMI_TRY(launch_table_clear(s->id_table, 0));
-  } else {
+  } else if (table_kind == LMI_TABLE_DIRECT) {
     LMI_HIP(hipMalloc(&s->slot_of, N * 4));
+  } else {
+    LMI_HIP(hipMalloc(&s->rank_tab, (size_t)ceil_div(N, 64) * 16));
+    hipLaunchKernelGGL(publish_rank_kernel, dim3(s->n_cu * 8), dim3(256), 0, 0, d_cnt, d_slot, N, s->rank_tab);
   }
   hipLaunchKernelGGL(publish_slots_kernel, dim3(s->n_cu * 8), dim3(256), 0, 0, d_cnt, d_slot, N, table_kind,
                      s->id_table.slots, s->id_table.log2cap, s->slot_of, d_cached);
@@ -731,9 +806,10 @@ int cache_build_lru(Server *s, int64_t n_sets, int32_t ways) {
   return LMI_OK;
 }
 
-static __global__ void dump_hash_kernel(const HashSlot *slots, int log2cap, int64_t n, int32_t *out) {
+static __global__ void dump_static_kernel(int table_kind, const HashSlot *slots, int log2cap, const int32_t *slot_of,
+                                          const uint4 *rank_tab, int64_t n, int32_t *out) {
   for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < n; v += (int64_t)gridDim.x * blockDim.x)
-    out[v] = table_find(slots, log2cap, (int32_t)v);
+    out[v] = static_find(table_kind, slots, log2cap, slot_of, rank_tab, (int32_t)v);
 }
 
 int cache_dump(Server *s, int32_t *slot_of, int64_t n, int32_t *aux) {
@@ -746,16 +822,12 @@ int cache_dump(Server *s, int32_t *slot_of, int64_t n, int32_t *aux) {
     return LMI_OK;
   }
   if (n != s->n_nodes) LMI_FAIL(LMI_ERR_ARG, "dump needs n == n_nodes");
-  if (s->table_kind == LMI_TABLE_DIRECT) {
-    LMI_HIP(hipMemcpy(slot_of, s->slot_of, n * 4, hipMemcpyDeviceToHost));
-  } else {
-    int32_t *d = nullptr;
-    LMI_HIP(hipMalloc(&d, n * 4));
-    hipLaunchKernelGGL(dump_hash_kernel, dim3(s->n_cu * 4), dim3(256), 0, 0, s->id_table.slots,
-                       s->id_table.log2cap, n, d);
-    LMI_HIP(hipMemcpy(slot_of, d, n * 4, hipMemcpyDeviceToHost));
-    (void)hipFree(d);
-  }
+  int32_t *d = nullptr;
+  LMI_HIP(hipMalloc(&d, n * 4));
+  hipLaunchKernelGGL(dump_static_kernel, dim3(s->n_cu * 4), dim3(256), 0, 0, s->table_kind, s->id_table.slots,
+                     s->id_table.log2cap, s->slot_of, s->rank_tab, n, d);
+  LMI_HIP(hipMemcpy(slot_of, d, n * 4, hipMemcpyDeviceToHost));
+  (void)hipFree(d);
   return LMI_OK;
 }
 

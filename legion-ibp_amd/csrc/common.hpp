@@ -45,13 +45,19 @@ void set_error(const char *fmt, ...);
 struct DevState {
   int32_t node_counter[16];
   int32_t edge_counter[16];
-  // One hit list and one miss list per lookup segment (0 = seeds or the whole
+  // One miss list per lookup segment (0 = seeds or the whole
   // batch, k = nodes added by hop k); zeroed at batch start.
-  int32_t n_hit[LMI_MAX_HOPS + 1];
   int32_t n_miss[LMI_MAX_HOPS + 1];
+  int32_t reserved[LMI_MAX_HOPS + 1];
   int32_t bad_id;      // set when a seed id is outside [0, n_nodes)
   int32_t scan_total;  // total of the last device scan
-  int32_t pad[6];
+  // per-batch parameters, written by the first kernel of a batch so that every
+  // later kernel (and a replayed HIP graph) reads them from HBM
+  uint32_t rng_lo, rng_hi;   // 64-bit Philox key of this batch
+  int32_t lru_tick;
+  int32_t n_seeds;
+  const int32_t *seeds;      // device address of this batch's seed ids
+  const int32_t *labels_in;  // device address of their labels (or null)
 };
 
 struct HashSlot {  // 8-byte open-addressing slot: one 64-bit load per probe
@@ -82,16 +88,30 @@ struct Pipe {
   int32_t *cnt = nullptr;      // [max(max_nodes, max_edges_hop)] scan input
   int32_t *rank = nullptr;     // [max_edges_hop + 1] scan output
   int32_t *tile_sums = nullptr;
-  int32_t *hit_list = nullptr, *miss_list = nullptr;  // [max_nodes] row indices
+  int2 *miss_list = nullptr;   // [max_nodes] (row, id) pairs of cache misses
   int32_t *lru_fill = nullptr;                        // [max_nodes] slot granted to a miss
-  hipStream_t side = nullptr;  // second stream: host-link misses overlap HBM hits
+  hipStream_t side = nullptr;  // second stream for the host-link gather
   hipEvent_t fork = nullptr, join = nullptr;
-  uint64_t rng_seed = 0;
+  bool side_pending = false;   // the side stream still owes this pipe's miss rows (join not yet waited on)
+  int32_t *seed_stage = nullptr;  // [batch_size] host seeds land here
   int32_t n_seeds = 0;
   int32_t hops_done = 0;
+  // HIP graph of one whole batch minus the feature gather (captured on first use)
+  hipGraphExec_t graph_exec = nullptr;
+  hipGraph_t graph = nullptr;
+  hipGraphNode_t begin_node = nullptr;
 };
 
-struct EventPair {
+// per-batch scalars, the only arguments that change between graph replays
+struct BatchParams {
+  int32_t n_seeds;
+  int32_t lru_tick;
+  uint64_t rng_seed;
+  const int32_t *seeds;
+  const int32_t *labels;
+};
+
+struct EventPair {  // device time between two recorded events, attributed to `kind`
   hipEvent_t a, b;
   int kind;
 };
@@ -122,6 +142,7 @@ struct Server {
   float *cache_scale = nullptr;      // int8: per-row scale
   Table id_table;                    // hash id -> slot
   int32_t *slot_of = nullptr;        // direct id -> slot
+  uint4 *rank_tab = nullptr;         // per 64 ids: {bits lo, bits hi, rank of first id, 0}
   int64_t lru_sets = 0;
   int32_t lru_ways = 0;
   int32_t lru_tick = 0;
@@ -134,11 +155,16 @@ struct Server {
   int gather_blocks = 0;  // 0 = auto
   int gather_nt = 1;      // non-temporal output stores
   int lds_dedup = 1;
-  int split_miss = 1;     // misses on the side stream
+  int split_miss = 1;     // 1: host-link gather on the pipe's side stream, after the HBM gather
+  int use_graph = 1;      // lmi_run_once replays a captured HIP graph
+  int miss_blocks = 0;    // grid of the host-link gather (0 = one block per CU)
+  int miss_unroll = 1;    // rows in flight per lane in the host-link gather
   // profiling
   bool prof_on = false;
   std::vector<EventPair> prof_events;   // recorded, not yet resolved
+  std::vector<hipEvent_t> prof_used;    // every event recorded since the last read (pairs may share one)
   std::vector<hipEvent_t> prof_free;    // recycled events
+  int prof_open = -1;                   // pair still waiting for its end event on the caller's stream
   DevState *prof_ring = nullptr;        // pinned host snapshots of finished batches
   int prof_ring_n = 0;
   lmi_profile prof{};
@@ -151,10 +177,13 @@ enum { PROF_GATHER_HIT = 0, PROF_GATHER_MISS = 1, PROF_SAMPLE = 2, PROF_LOOKUP =
 // profiling helpers (api.hip)
 int prof_begin(Server *s, hipStream_t st, int kind);
 int prof_end(Server *s, hipStream_t st, int handle);
+// One event closes the pair left open on the caller's stream and opens the next
+// phase (next_kind < 0: only close), so a batch costs one event per phase boundary.
+void prof_phase(Server *s, hipStream_t st, int next_kind);
 
 // sampler.hip
-int launch_batch_generate(Server *s, Pipe &p, hipStream_t st, const int32_t *d_seeds, int32_t n,
-                          const int32_t *d_labels);
+int launch_batch_generate(Server *s, Pipe &p, hipStream_t st, const BatchParams &bp);
+int graph_update_begin(Server *s, Pipe &p, const BatchParams &bp);
 int launch_hop(Server *s, Pipe &p, hipStream_t st, int hop);
 int launch_table_clear(Table &t, hipStream_t st);
 
@@ -167,6 +196,7 @@ void cache_free(Server *s);
 int launch_lookup(Server *s, Pipe &p, hipStream_t st, int seg_first, int seg_last);
 int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last);
 int launch_lru_insert(Server *s, Pipe &p, hipStream_t st, int n_lists);
+int pipe_join(Pipe &p, hipStream_t st);  // make `st` wait for the pipe's side-stream work
 int cache_dump(Server *s, int32_t *slot_of, int64_t n, int32_t *aux);
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }

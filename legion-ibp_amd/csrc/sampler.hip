@@ -17,9 +17,10 @@
 namespace lmi {
 
 // ------------------------------------------------------------ batch start
-// Clears the dedup table (key = -1, value = INT_MAX) and resets the pipe state.
+// Clears the dedup table (key = -1, value = INT_MAX), resets the pipe state and
+// stores the per-batch parameters where the later kernels read them.
 static __global__ __launch_bounds__(256) void batch_begin_kernel(HashSlot *slots, int64_t n_slots,
-                                                                 DevState *st, int hops, int n_seeds) {
+                                                                 DevState *st, int hops, BatchParams bp) {
   const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   // two slots (16 bytes) per store
@@ -30,22 +31,27 @@ static __global__ __launch_bounds__(256) void batch_begin_kernel(HashSlot *slots
     int32_t *w = reinterpret_cast<int32_t *>(st);
     for (int i = 0; i < (int)(sizeof(DevState) / 4); ++i) w[i] = 0;
     st->node_counter[8] = hops;
-    st->node_counter[9] = n_seeds;
-    st->node_counter[1] = st->node_counter[3] = st->node_counter[5] = n_seeds;
-    st->node_counter[7] = n_seeds;
+    st->node_counter[9] = bp.n_seeds;
+    st->node_counter[1] = st->node_counter[3] = st->node_counter[5] = bp.n_seeds;
+    st->node_counter[7] = bp.n_seeds;
+    st->rng_lo = (uint32_t)bp.rng_seed;
+    st->rng_hi = (uint32_t)(bp.rng_seed >> 32);
+    st->lru_tick = bp.lru_tick;
+    st->n_seeds = bp.n_seeds;
+    st->seeds = bp.seeds;
+    st->labels_in = bp.labels;
   }
 }
 
 // Stage the seeds: ids[i] = seed, labels, and table[seed] = min(i) so that a
 // repeated seed resolves to its first row.
-static __global__ __launch_bounds__(256) void batch_generate_kernel(
-    const int32_t *seeds, const int32_t *labels_in, int n, int64_t n_nodes, int32_t *ids,
-    int32_t *labels, HashSlot *slots, int log2cap, DevState *st) {
+static __global__ __launch_bounds__(256) void batch_generate_kernel(int64_t n_nodes, int32_t *ids, int32_t *labels,
+                                                                    HashSlot *slots, int log2cap, DevState *st) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
-  if (i >= n) return;
-  const int32_t id = seeds[i];
+  if (i >= st->n_seeds) return;
+  const int32_t id = st->seeds[i];
   ids[i] = id;
-  labels[i] = labels_in ? labels_in[i] : -1;
+  labels[i] = st->labels_in ? st->labels_in[i] : -1;
   if (id < 0 || id >= n_nodes) {
     st->bad_id = 1;
     return;
@@ -91,8 +97,9 @@ static __global__ __launch_bounds__(kScanBlock) void hop_count_kernel(
 template <int G>
 static __global__ __launch_bounds__(256) void hop_sample_kernel(
     const int32_t *ids, const int64_t *indptr, const int32_t *indices, int64_t n_nodes, int fanout,
-    int hop, uint64_t seed, const DevState *st, const int32_t *row_ptr, int32_t *agg_src_ids,
-    int32_t *agg_dst_off, HashSlot *slots, int log2cap, int32_t *eslot) {
+    int hop, const DevState *st, const int32_t *row_ptr, int32_t *agg_src_ids, int32_t *agg_dst_off,
+    HashSlot *slots, int log2cap, int32_t *eslot) {
+  const uint64_t seed = (uint64_t)st->rng_lo | ((uint64_t)st->rng_hi << 32);
   const int n_prev = st->node_counter[9 + hop];
   const int eoff = st->edge_counter[12 + hop + 1];
   const int lane = threadIdx.x & (G - 1);
@@ -184,25 +191,55 @@ static __global__ __launch_bounds__(256) void hop_relabel_kernel(
 }
 
 // ---------------------------------------------------------------- launchers
-int launch_batch_generate(Server *s, Pipe &p, hipStream_t st, const int32_t *d_seeds, int32_t n,
-                          const int32_t *d_labels) {
+static void begin_args(Server *s, Pipe &p, const BatchParams &bp, void **args, HashSlot **slots, int64_t *n_slots,
+                       DevState **st, int *hops, BatchParams *bpc) {
+  *slots = p.dedup.slots;
+  *n_slots = int64_t(1) << p.dedup.log2cap;
+  *st = p.st;
+  *hops = s->cfg.hops;
+  *bpc = bp;
+  args[0] = slots; args[1] = n_slots; args[2] = st; args[3] = hops; args[4] = bpc;
+}
+
+static int begin_grid(const Pipe &p) {
   const int64_t n_slots = int64_t(1) << p.dedup.log2cap;
-  int grid = (int)std::min<int64_t>(ceil_div(n_slots / 2, 256), 2048);
-  hipLaunchKernelGGL(batch_begin_kernel, dim3(grid), dim3(256), 0, st, p.dedup.slots, n_slots, p.st,
-                     s->cfg.hops, n);
-  if (n > 0)
-    hipLaunchKernelGGL(batch_generate_kernel, dim3((n + 255) / 256), dim3(256), 0, st, d_seeds, d_labels,
-                       n, s->n_nodes, p.ids, p.labels, p.dedup.slots, p.dedup.log2cap, p.st);
+  return (int)std::min<int64_t>(ceil_div(n_slots / 2, 256), 2048);
+}
+
+int launch_batch_generate(Server *s, Pipe &p, hipStream_t st, const BatchParams &bp) {
+  const int64_t n_slots = int64_t(1) << p.dedup.log2cap;
+  hipLaunchKernelGGL(batch_begin_kernel, dim3(begin_grid(p)), dim3(256), 0, st, p.dedup.slots, n_slots, p.st,
+                     s->cfg.hops, bp);
+  hipLaunchKernelGGL(batch_generate_kernel, dim3((s->cfg.batch_size + 255) / 256), dim3(256), 0, st, s->n_nodes,
+                     p.ids, p.labels, p.dedup.slots, p.dedup.log2cap, p.st);
   LMI_HIP(hipGetLastError());
-  p.n_seeds = n;
+  p.n_seeds = bp.n_seeds;
   p.hops_done = 0;
+  return LMI_OK;
+}
+
+// Re-points the captured graph's first kernel at this batch's parameters.
+int graph_update_begin(Server *s, Pipe &p, const BatchParams &bp) {
+  HashSlot *slots; int64_t n_slots; DevState *st; int hops; BatchParams bpc;
+  void *args[5];
+  begin_args(s, p, bp, args, &slots, &n_slots, &st, &hops, &bpc);
+  hipKernelNodeParams kp{};
+  kp.func = reinterpret_cast<void *>(batch_begin_kernel);
+  kp.gridDim = dim3(begin_grid(p));
+  kp.blockDim = dim3(256);
+  kp.sharedMemBytes = 0;
+  kp.kernelParams = args;
+  kp.extra = nullptr;
+  LMI_HIP(hipGraphExecKernelNodeSetParams(p.graph_exec, p.begin_node, &kp));
+  p.n_seeds = bp.n_seeds;
+  p.hops_done = s->cfg.hops;
   return LMI_OK;
 }
 
 template <int G>
 static void launch_sample_g(Server *s, Pipe &p, hipStream_t st, int hop, int grid) {
   hipLaunchKernelGGL(hop_sample_kernel<G>, dim3(grid), dim3(256), 0, st, p.ids, s->indptr, s->indices,
-                     s->n_nodes, s->cfg.fanout[hop], hop, p.rng_seed, p.st, p.blk_indptr[hop],
+                     s->n_nodes, s->cfg.fanout[hop], hop, p.st, p.blk_indptr[hop],
                      p.agg_src_ids, p.agg_dst_off, p.dedup.slots, p.dedup.log2cap, p.eslot);
 }
 

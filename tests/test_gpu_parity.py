@@ -99,7 +99,7 @@ def test_bad_seed_is_reported(lmi):
         feats.free()
 
 
-@pytest.mark.parametrize("table", [0, 1])
+@pytest.mark.parametrize("table", [0, 1, 2])
 @pytest.mark.parametrize("dim,dtype", [(128, np.float32), (100, np.float32), (1433, np.float32), (768, np.float16),
                                         (6, np.float16)])
 def test_static_cache_parity(lmi, oracle, table, dim, dtype):
@@ -289,3 +289,58 @@ def test_synth_graph_matches_oracle(lmi, oracle):
     np.testing.assert_array_equal(lmi.synth_trainset(7, 20000, 1500), oracle.synth_trainset(7, 20000, 1500))
     mean = np.diff(indptr).mean()
     assert 8.0 < mean < 10.0
+
+
+@pytest.mark.parametrize("cache", ["static", "lru", "int8"])
+def test_graph_replay_matches_eager_and_oracle(lmi, oracle, cache):
+    """lmi_run_once on a real stream replays a captured HIP graph; every replay is
+    checked against the oracle, with eager batches and synchronisations in between."""
+    rng = np.random.default_rng(21)
+    n_nodes, batch, fanout, dim = 6000, 200, [10, 5, 3], 64
+    indptr, indices = random_graph(rng, n_nodes, 9, hubs=6, hub_deg=400)
+    feats = make_features(lmi, rng, n_nodes, dim)
+    host_rows = feats.array.view(np.uint8).reshape(n_nodes, dim * 4)
+    train = rng.permutation(n_nodes)[:1000].astype(np.int32)
+    srv = lmi.Server(batch, fanout, dim, pipes=2, seed=9)
+    streams = [lmi.stream_create(), lmi.stream_create()]
+    lru = oracle.Lru(128, 4, dim * 4)
+    try:
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        srv.load_idset(lmi.MODE_TRAIN, train)
+        if cache == "static":
+            srv.build_static_cache(2500, lmi.TABLE_RANK)
+            slot_ref = oracle.static_cache_build(indptr, 2500)
+        elif cache == "int8":
+            srv.build_int8_cache(2500, lmi.TABLE_RANK)
+            slot_ref = oracle.static_cache_build(indptr, 2500)
+            q, sc = oracle.quantize_rows(feats.array[np.flatnonzero(slot_ref >= 0)])
+        else:
+            srv.build_lru_cache(128, 4)
+        for it in range(10):
+            pipe = it % 2
+            graph = it % 3 != 2          # every third batch runs eagerly on the default stream
+            if it == 6:
+                seeds = rng.choice(n_nodes, 77, replace=False).astype(np.int32)   # caller seeds, short batch
+                ref_seeds = seeds
+            else:
+                seeds = None
+                ref_seeds = train[(it % 5) * batch:(it % 5 + 1) * batch]
+            st = streams[pipe] if graph else None
+            srv.run_once(seeds, batch_counter=it % 5, rng_seed=50 + it, pipe=pipe, stream=st)
+            g = srv.fetch(pipe=pipe, stream=st)
+            o = oracle.sample_batch(indptr, indices, ref_seeds, fanout, 50 + it)
+            assert_batch_equal(g, o)
+            if cache == "static":
+                np.testing.assert_array_equal(g.cache_index, slot_ref[o.ids])
+                assert g.features.tobytes() == feats.array[o.ids].tobytes()
+            elif cache == "int8":
+                ref = oracle.gather_rows_int8(o.ids, slot_ref[o.ids], q, sc, feats.array)
+                assert g.features.tobytes() == ref.tobytes()
+            else:
+                hit, fill, out = lru.access(o.ids, host_rows)
+                np.testing.assert_array_equal(g.cache_index, hit)
+                assert g.features.tobytes() == out.tobytes()
+    finally:
+        srv.close()
+        feats.free()

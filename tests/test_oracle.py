@@ -1,0 +1,309 @@
+"""CPU tests that pin the oracle itself.
+
+The reference tree holds no golden vectors or tests for this path, so every
+function of the oracle is pinned by something independent of its own formula:
+published known-answer vectors (Philox), closed forms and special cases,
+exact enumeration and chi-square statistics over many seeds (Floyd sampling),
+brute force in plain Python structured differently from the C++ (dict-based
+relabel, list-scan LRU), and numpy's IEEE arithmetic (fp16 conversion, int8
+codec, lexsort ranking)."""
+import collections
+import itertools
+
+import numpy as np
+import pytest
+
+from conftest import random_graph
+
+
+# ------------------------------------------------------------------ Philox
+PHILOX_KATS = [  # Random123 kat_vectors, philox4x32 10 rounds: (counter, key, expected)
+    ([0, 0, 0, 0], [0, 0], [0x6627e8d5, 0xe169c58d, 0xbc57ac4c, 0x9b00dbd8]),
+    ([0xffffffff] * 4, [0xffffffff] * 2, [0x408f276d, 0x41c83b0e, 0xa20bc7c6, 0x6d5451fd]),
+    ([0x243f6a88, 0x85a308d3, 0x13198a2e, 0x03707344], [0xa4093822, 0x299f31d0],
+     [0xd16cfe09, 0x94fdcceb, 0x5001e420, 0x24126ea1]),
+]
+
+
+@pytest.mark.parametrize("ctr,key,expected", PHILOX_KATS)
+def test_philox_known_answers(oracle, ctr, key, expected):
+    assert [int(x) for x in oracle.philox4x32_10(ctr, key)] == expected
+
+
+def test_draw_is_word0_of_node_hop_slot_counter(oracle):
+    for seed, hop, node, slot in [(0, 0, 0, 0), (0xa4093822299f31d0 >> 0, 1, 77, 3), (2**64 - 1, 2, 2**31 - 1, 63)]:
+        key = [seed & 0xffffffff, seed >> 32]
+        assert oracle.draw(seed, hop, node, slot) == int(oracle.philox4x32_10([node, hop, slot, 0], key)[0])
+    # changing any one of (seed, hop, node, slot) changes the stream
+    base = oracle.draw(5, 1, 9, 2)
+    assert len({base, oracle.draw(6, 1, 9, 2), oracle.draw(5, 2, 9, 2), oracle.draw(5, 1, 10, 2),
+                oracle.draw(5, 1, 9, 3)}) == 5
+
+
+# ------------------------------------------------------------- pick positions
+def test_short_rows_are_taken_whole_in_order(oracle):
+    for deg, f in [(0, 5), (1, 1), (3, 5), (25, 25), (10, 64)]:
+        assert list(oracle.sample_positions(9, 0, 4, deg, f)) == list(range(deg))
+
+
+def test_long_rows_give_distinct_in_range_positions(oracle):
+    rng = np.random.default_rng(0)
+    for _ in range(300):
+        f = int(rng.integers(1, 65))
+        deg = int(rng.integers(f + 1, 5000))
+        pos = oracle.sample_positions(int(rng.integers(1, 2**62)), int(rng.integers(0, 3)),
+                                      int(rng.integers(0, 2**31)), deg, f)
+        assert len(pos) == f and len(set(pos.tolist())) == f
+        assert pos.min() >= 0 and pos.max() < deg
+
+
+def test_positions_depend_only_on_seed_hop_node(oracle):
+    a = oracle.sample_positions(123, 1, 42, 900, 10)
+    assert np.array_equal(a, oracle.sample_positions(123, 1, 42, 900, 10))
+    assert not np.array_equal(a, oracle.sample_positions(124, 1, 42, 900, 10))
+    assert not np.array_equal(a, oracle.sample_positions(123, 0, 42, 900, 10))
+    assert not np.array_equal(a, oracle.sample_positions(123, 1, 43, 900, 10))
+
+
+def test_every_subset_is_equally_likely(oracle):
+    """deg=6, f=3: 20 subsets; Floyd's rule must make them equiprobable.  An off-by-one in
+    the range (j instead of j+1), a wrong collision fallback or a dropped slot fails this."""
+    deg, f, trials = 6, 3, 40000
+    counts = collections.Counter()
+    for s in range(trials):
+        counts[tuple(sorted(oracle.sample_positions(1000 + s, 0, 7, deg, f).tolist()))] += 1
+    subsets = list(itertools.combinations(range(deg), f))
+    assert set(counts) == set(subsets)
+    expect = trials / len(subsets)
+    chi2 = sum((counts[s] - expect) ** 2 / expect for s in subsets)
+    assert chi2 < 50.0  # 19 dof: P(chi2 > 50) ~ 1e-4
+
+
+def test_each_position_is_hit_uniformly(oracle):
+    deg, f, trials = 37, 10, 20000
+    hits = np.zeros(deg)
+    for node in range(trials):
+        hits[oracle.sample_positions(77, 1, node, deg, f)] += 1
+    expect = trials * f / deg
+    chi2 = ((hits - expect) ** 2 / expect).sum()
+    assert chi2 < 90.0  # 36 dof
+
+
+# ------------------------------------------------------------------ a batch
+def brute_force_batch(indptr, indices, seeds, fanout, seed, oracle):
+    """Plain-python restatement with a different structure: per-node adjacency
+    lists, a dict for first-occurrence ids, lists for the edges."""
+    ids = list(seeds)
+    local = {}
+    for i, s in enumerate(seeds):
+        local.setdefault(int(s), i)
+    blocks = []
+    for k, f in enumerate(fanout):
+        n_prev = len(ids)
+        src_g, dst_l, rowptr = [], [], [0]
+        for i in range(n_prev):
+            v = ids[i]
+            row = indices[indptr[v]:indptr[v + 1]]
+            for p in oracle.sample_positions(seed, k, v, len(row), f):
+                src_g.append(int(row[p]))
+                dst_l.append(i)
+            rowptr.append(len(src_g))
+        src_l = []
+        for g in src_g:
+            if g not in local:
+                local[g] = len(ids)
+                ids.append(g)
+            src_l.append(local[g])
+        blocks.append((src_g, src_l, dst_l, rowptr))
+    return ids, blocks
+
+
+@pytest.mark.parametrize("fanout", [[25, 10], [3], [5, 4, 3]])
+def test_sample_batch_against_brute_force(oracle, fanout):
+    rng = np.random.default_rng(len(fanout))
+    indptr, indices = random_graph(rng, 400, 9, hubs=3, hub_deg=150)
+    seeds = rng.choice(400, 24, replace=False).astype(np.int32)
+    b = oracle.sample_batch(indptr, indices, seeds, fanout, 31337)
+    ids, blocks = brute_force_batch(indptr, indices, seeds.tolist(), fanout, 31337, oracle)
+    assert b.ids.tolist() == ids
+    e0 = 0
+    for k, (src_g, src_l, dst_l, rowptr) in enumerate(blocks):
+        e1 = e0 + len(src_g)
+        assert b.edge_off[k] == e0 and b.n_edges[k] == len(src_g)
+        assert b.agg_src_ids[e0:e1].tolist() == src_g
+        assert b.agg_src_off[e0:e1].tolist() == src_l
+        assert b.agg_dst_off[e0:e1].tolist() == dst_l
+        assert b.blk_indptr[k].tolist() == rowptr
+        e0 = e1
+
+
+def test_batch_invariants_and_headers(oracle):
+    rng = np.random.default_rng(8)
+    indptr, indices = random_graph(rng, 3000, 14, hubs=5, hub_deg=800)
+    fanout = [15, 10, 5]
+    seeds = rng.choice(3000, 100, replace=False).astype(np.int32)
+    b = oracle.sample_batch(indptr, indices, seeds, fanout, 99)
+    nc, ec = b.node_counter, b.edge_counter
+    assert nc[8] == 3 and nc[9] == 100 and nc[7] == len(b.ids) == nc[12]
+    assert nc[0] == nc[11] and nc[1] == nc[12] - nc[11]           # last frontier: offset, size
+    assert [ec[13], ec[14], ec[15]] == [0, ec[10], ec[10] + ec[11]]  # edge offsets are prefix sums
+    assert len(set(b.ids.tolist())) == len(b.ids)                # ids unique
+    assert b.ids[:100].tolist() == seeds.tolist()                # seeds are local 0..B-1
+    adj = [set(indices[indptr[v]:indptr[v + 1]].tolist()) for v in range(3000)]
+    for k in range(3):
+        e0, e1 = b.edge_off[k], b.edge_off[k] + b.n_edges[k]
+        src, dst = b.agg_src_off[e0:e1], b.agg_dst_off[e0:e1]
+        assert (dst < b.n_nodes[k]).all() and (src < b.n_nodes[k + 1]).all()
+        assert (np.diff(dst) >= 0).all()                          # rows sorted: COO is row-major CSR
+        assert np.array_equal(np.bincount(dst, minlength=b.n_nodes[k]), np.diff(b.blk_indptr[k]))
+        for s, d in zip(src[:500], dst[:500]):
+            assert int(b.ids[s]) in adj[int(b.ids[d])]            # every edge is a real edge
+        deg = np.diff(indptr)[b.ids[:b.n_nodes[k]]]
+        assert np.array_equal(np.diff(b.blk_indptr[k]), np.minimum(deg, fanout[k]))
+
+
+def test_batch_errors(oracle):
+    indptr = np.array([0, 1, 2], np.int64)
+    indices = np.array([1, 0], np.int32)
+    with pytest.raises(RuntimeError):
+        oracle.sample_batch(indptr, indices, [5], [2], 1)       # seed out of range
+    with pytest.raises(RuntimeError):
+        oracle.sample_batch(indptr, indices, [0], [2, 2, 2, 2], 1)  # too many hops
+
+
+# ------------------------------------------------------------- static cache
+@pytest.mark.parametrize("cap", [0, 1, 37, 500, 1000])
+def test_static_cache_is_top_by_degree_then_id(oracle, cap):
+    rng = np.random.default_rng(cap)
+    indptr, _ = random_graph(rng, 1000, 5)       # many degree ties
+    deg = np.diff(indptr)
+    slot = oracle.static_cache_build(indptr, cap)
+    order = np.lexsort((np.arange(1000), -deg))   # degree desc, id asc
+    members = np.sort(order[:cap])
+    assert np.array_equal(np.flatnonzero(slot >= 0), members)
+    assert np.array_equal(slot[members], np.arange(cap))       # slot = rank among cached ids
+
+
+# ---------------------------------------------------------------------- LRU
+class PyLru:
+    """Independent model: a list of [key, last_use] per set, plain loops."""
+
+    def __init__(self, sets, ways):
+        self.sets, self.ways, self.t = sets, ways, 0
+        self.tab = [[[-1, 0] for _ in range(ways)] for _ in range(sets)]
+
+    def access(self, ids):
+        self.t += 1
+        hit, fill = [], []
+        for v in ids:
+            ways = self.tab[v % self.sets]
+            where = [w for w in range(self.ways) if ways[w][0] == v]
+            hit.append(v % self.sets * self.ways + where[0] if where else -1)
+            if where:
+                ways[where[0]][1] = self.t
+        for v, h in zip(ids, hit):
+            if h >= 0:
+                fill.append(-1)
+                continue
+            ways = self.tab[v % self.sets]
+            cands = sorted((ways[w][1], w) for w in range(self.ways) if ways[w][1] < self.t)
+            if not cands:
+                fill.append(-1)
+                continue
+            w = cands[0][1]
+            ways[w][0], ways[w][1] = v, self.t
+            fill.append(v % self.sets * self.ways + w)
+        return hit, fill
+
+
+@pytest.mark.parametrize("sets,ways", [(16, 4), (1, 8), (130, 2)])
+def test_lru_trace_replay(oracle, sets, ways):
+    """Toy workload shaped like the reference's manual driver
+    (comp_cache/tests/test_cache.cu:4-9,48-53): 1000 nodes, 130 hot, 128 ids/iter, 90 % hot."""
+    rng = np.random.default_rng(sets)
+    hot = rng.choice(1000, 130, replace=False)
+    lru, ref = oracle.Lru(sets, ways, 8), PyLru(sets, ways)
+    rows = rng.integers(0, 255, (1000, 8)).astype(np.uint8)
+    for _ in range(40):
+        ids = np.unique(np.concatenate([rng.choice(hot, 115), rng.choice(1000, 13)])).astype(np.int32)
+        rng.shuffle(ids)
+        hit, fill, out = lru.access(ids, rows)
+        rhit, rfill = ref.access(ids.tolist())
+        assert hit.tolist() == rhit and fill.tolist() == rfill
+        assert np.array_equal(out, rows[ids])                   # cached rows are the right rows
+        keys, use = lru.state()
+        live = keys[keys >= 0]
+        assert len(set(live.tolist())) == len(live) <= sets * ways
+        assert all(k % sets == i // ways for i, k in enumerate(keys) if k >= 0)
+    if sets * ways >= 64:
+        assert (np.array(rhit) >= 0).mean() > 0.3       # the hot set mostly stays resident
+
+
+# --------------------------------------------------------------- int8 codec
+def test_fp16_conversion_matches_numpy(oracle):
+    halves = np.arange(65536, dtype=np.uint16)
+    as32 = halves.view(np.float16).astype(np.float32)
+    for h in range(0, 65536, 7):
+        v = oracle.f16_to_f32(h)
+        assert (np.isnan(v) and np.isnan(as32[h])) or np.float32(v).tobytes() == as32[h].tobytes()
+    rng = np.random.default_rng(1)
+    x = (rng.standard_normal(20000) * rng.choice([1e-8, 1e-5, 1e-3, 1, 100, 7e4], 20000)).astype(np.float32)
+    ties = as32[np.isfinite(as32)][::5]
+    ties = ((ties.view(np.uint32) + 0x1000).view(np.float32))     # exactly between two halves
+    x = np.concatenate([x, ties, -ties])
+    with np.errstate(over="ignore"):
+        want = x.astype(np.float16).view(np.uint16)
+    got = np.array([oracle.f32_to_f16(v) for v in x], np.uint16)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("dtype", [np.float32, np.float16])
+def test_int8_codec_matches_numpy_ieee(oracle, dtype):
+    rng = np.random.default_rng(2)
+    rows = (rng.standard_normal((64, 100)) * rng.choice([1e-3, 1, 50], (64, 1))).astype(dtype)
+    rows[3] = 0
+    rows[5, 0] = rows[5].astype(np.float32).__abs__().max() * 2   # a clear absmax
+    q, sc = oracle.quantize_rows(rows)
+    x = rows.astype(np.float32)
+    a = np.abs(x).max(axis=1)
+    want_sc = (a / np.float32(127.0)).astype(np.float32)
+    assert sc.tobytes() == want_sc.tobytes()
+    with np.errstate(divide="ignore", invalid="ignore"):
+        want_q = np.where(a[:, None] == 0, 0, np.clip(np.rint(x / want_sc[:, None]), -127, 127)).astype(np.int8)
+    assert np.array_equal(q, want_q)
+    assert (q[3] == 0).all() and sc[3] == 0 and abs(int(q[5, 0])) == 127
+    for out_dtype in (np.float32, np.float16):
+        y = oracle.dequant_rows(q, sc, out_dtype)
+        want = (q.astype(np.float32) * sc[:, None]).astype(np.float32).astype(out_dtype)
+        assert y.tobytes() == want.tobytes()
+    # a value at +-absmax dequantises to exactly 127 * (absmax / 127)
+    y32 = oracle.dequant_rows(q, sc, np.float32)
+    assert abs(y32[5, 0]) == np.float32(127.0) * sc[5]
+
+
+def test_gather_rows_is_fancy_indexing(oracle):
+    rng = np.random.default_rng(3)
+    host = rng.standard_normal((500, 33)).astype(np.float32)
+    cache = rng.standard_normal((50, 33)).astype(np.float32)
+    ids = rng.integers(0, 500, 200).astype(np.int32)
+    slot = np.where(rng.random(200) < 0.4, rng.integers(0, 50, 200), -1).astype(np.int32)
+    out = oracle.gather_rows(ids, slot, cache, host)
+    want = np.where((slot >= 0)[:, None], cache[np.maximum(slot, 0)], host[ids])
+    assert out.tobytes() == want.tobytes()
+
+
+# ------------------------------------------------------- synthetic generator
+def test_synth_graph_properties(oracle, lmi):
+    cdf = lmi.zipf_cdf(2.0, 2000, 12.0)
+    assert cdf[0] == 0 and cdf[-1] == 0xFFFFFFFF and (np.diff(cdf.astype(np.int64)) >= 0).all()
+    indptr, indices = oracle.synth_graph(11, cdf, 50000, mode=1)
+    deg = np.diff(indptr)
+    assert deg.min() >= 0 and deg.max() <= 2000 and 10.5 < deg.mean() < 13.5
+    # degree-proportional neighbours: in-degree correlates with out-degree
+    indeg = np.bincount(indices, minlength=50000)
+    assert np.corrcoef(indeg, deg)[0, 1] > 0.8
+    i0, x0 = oracle.synth_graph(11, cdf, 50000, mode=0)
+    assert np.array_equal(i0, indptr)
+    assert abs(np.corrcoef(np.bincount(x0, minlength=50000), deg)[0, 1]) < 0.05
+    train = oracle.synth_trainset(3, 50000, 4000)
+    assert len(set(train.tolist())) == 4000 and train.min() >= 0 and train.max() < 50000
