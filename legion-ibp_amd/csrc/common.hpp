@@ -157,7 +157,8 @@ struct Server {
   int lds_dedup = 1;
   int split_miss = 1;     // 1: host-link gather on the pipe's side stream, after the HBM gather
   int use_graph = 1;      // lmi_run_once replays a captured HIP graph
-  int miss_blocks = 0;    // grid of the host-link gather (0 = one block per CU)
+  int miss_blocks = 32;   // grid of the host-link gather: enough reads in flight to fill the link, few enough
+                          // not to crowd HBM traffic out of the memory pipeline
   int miss_unroll = 1;    // rows in flight per lane in the host-link gather
   // profiling
   bool prof_on = false;

@@ -1,0 +1,356 @@
+// Host shim: the reference's Server / Runner / Operator classes on top of the C ABI.
+// Plain C++17, no HIP headers: every device interaction is an lmi_* call.
+//
+// Reference behaviour followed here (Legion-IBP sampling_server/src):
+//   engine/server.cu:48-170     GPUServer: Initialize -> PreSc -> Run -> Finalize
+//   engine/server.cu:178-400    GPURunner: operator table, two output buffer sets
+//   engine/operator.cu:10-150   operator classes forwarding to the extern "C" layer
+//   storage/storage_management.cu:33-279   ./meta_config + dataset files
+#include "legion_host.hpp"
+
+#include <sys/mman.h>
+#include <sys/stat.h>
+#include <fcntl.h>
+#include <unistd.h>
+
+#include <chrono>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <fstream>
+#include <iostream>
+#include <sstream>
+
+namespace {
+
+[[noreturn]] void die(const char *what) {
+  std::fprintf(stderr, "legion_mi failure in %s: %s\n", what, lmi_last_error());
+  std::exit(EXIT_FAILURE);
+}
+#define LMI_MUST(call)                 \
+  do {                                 \
+    if ((call) != LMI_OK) die(#call);  \
+  } while (0)
+
+// Reads a whole binary file into `dst` (at most `bytes`); returns bytes read or -1.
+// The reference mmaps and never unmaps (storage_management_impl.cuh:48-123); a
+// buffered read into the final buffer does the same job without the leak.
+int64_t read_file(const std::string &path, void *dst, int64_t bytes) {
+  const int fd = open(path.c_str(), O_RDONLY);
+  if (fd < 0) return -1;
+  int64_t done = 0;
+  while (done < bytes) {
+    const ssize_t r = read(fd, (char *)dst + done, (size_t)std::min<int64_t>(bytes - done, int64_t(1) << 30));
+    if (r <= 0) break;
+    done += r;
+  }
+  close(fd);
+  return done;
+}
+
+void must_read(const std::string &path, void *dst, int64_t bytes) {
+  const int64_t got = read_file(path, dst, bytes);
+  if (got != bytes) {
+    std::fprintf(stderr, "cannot read %lld bytes from %s (got %lld)\n", (long long)bytes, path.c_str(), (long long)got);
+    std::exit(EXIT_FAILURE);
+  }
+}
+
+// ---------------------------------------------------------------- operators
+class BatchGenerateOP : public Operator {
+ public:
+  explicit BatchGenerateOP(int id) : op_id_(id) {}
+  void run(OpParams *p) override {
+    LMI_MUST(lmi_op_batch_generate((lmi_server *)p->env, p->pipe, p->stream, nullptr, 0, LMI_LOC_DEVICE,
+                                   p->global_batch_id, p->mode, 0));
+  }
+ private:
+  int op_id_;
+};
+
+class RandomSampleOP : public Operator {
+ public:
+  explicit RandomSampleOP(int id) : op_id_(id) {}
+  void run(OpParams *p) override {
+    LMI_MUST(lmi_op_random_sample((lmi_server *)p->env, p->pipe, p->stream, op_id_ / 3 - 1));
+  }
+ private:
+  int op_id_;
+};
+
+class CacheLookupOP : public Operator {
+ public:
+  explicit CacheLookupOP(int id) : op_id_(id) {}
+  void run(OpParams *p) override {
+    if (p->is_presc) return;  // presampling gathers nothing (engine/operator.cu:73-98)
+    LMI_MUST(lmi_op_cache_lookup((lmi_server *)p->env, p->pipe, p->stream, op_id_ / 3));
+  }
+ private:
+  int op_id_;
+};
+
+class SSDIOSubmitOP : public Operator {
+ public:
+  explicit SSDIOSubmitOP(int id) : op_id_(id) {}
+  void run(OpParams *p) override { LMI_MUST(lmi_op_io_submit((lmi_server *)p->env, p->pipe, p->stream)); }
+ private:
+  int op_id_;
+};
+
+class SSDIOCompleteOP : public Operator {
+ public:
+  explicit SSDIOCompleteOP(int id) : op_id_(id) {}
+  void run(OpParams *p) override { LMI_MUST(lmi_op_io_complete((lmi_server *)p->env, p->pipe, p->stream)); }
+ private:
+  int op_id_;
+};
+
+// ------------------------------------------------------------------- runner
+class GPURunner : public Runner {
+ public:
+  void Initialize(RunnerParams *params) override {
+    hops_ = (int)params->fanout.size();
+    LMI_MUST(lmi_stream_create(&stream_));
+    // slot table: [BatchGen, Lookup, IOSubmit, (Sample, Lookup, IOSubmit) x hops, IOComplete]
+    ops_.push_back(NewBatchGenerateOP(0));
+    ops_.push_back(NewCacheLookupOP(1));
+    ops_.push_back(NewSSDIOSubmitOP(2));
+    for (int k = 1; k <= hops_; ++k) {
+      ops_.push_back(NewRandomSampleOP(3 * k));
+      ops_.push_back(NewCacheLookupOP(3 * k + 1));
+      ops_.push_back(NewSSDIOSubmitOP(3 * k + 2));
+    }
+    ops_.push_back(NewSSDIOCompleteOP(3 * (hops_ + 1)));
+    op_params_.resize(ops_.size());
+    for (size_t i = 0; i < ops_.size(); ++i) {
+      OpParams &o = op_params_[i];
+      o = OpParams{};
+      o.device_id = params->device_id;
+      o.stream = stream_;
+      o.env = params->env;
+      o.in_memory = params->in_memory;
+      o.hop_num = hops_;
+      o.dyn_cache = params->dyn_cache;
+      const int hop = (int)i / 3 - 1;
+      o.neighbor_count = (i % 3 == 0 && hop >= 0 && hop < hops_) ? params->fanout[hop] : 0;
+    }
+  }
+  void InitializeFeaturesBuffer(RunnerParams *) override {}
+  void RunPreSc(RunnerParams *params) override { run_table(params, true); }
+  void RunOnce(RunnerParams *params) override {
+    pipe_ ^= 1;  // two output buffer sets, as INTERBATCH_CON = 2
+    if (params->fused) {
+      LMI_MUST(lmi_run_once((lmi_server *)params->env, pipe_, stream_, nullptr, 0, LMI_LOC_DEVICE,
+                            params->global_batch_id, params->mode, 0));
+    } else {
+      run_table(params, false);
+    }
+    LMI_MUST(lmi_batch_wait((lmi_server *)params->env, pipe_, stream_));
+  }
+  void Finalize(RunnerParams *) override {
+    if (stream_) {
+      LMI_MUST(lmi_stream_sync(stream_));
+      LMI_MUST(lmi_stream_destroy(stream_));
+      stream_ = nullptr;
+    }
+    for (Operator *o : ops_) delete o;
+    ops_.clear();
+  }
+  int CurrentPipe() const override { return pipe_; }
+  void *Stream() const override { return stream_; }
+
+ private:
+  void run_table(RunnerParams *params, bool presc) {
+    for (size_t i = 0; i < ops_.size(); ++i) {
+      OpParams &o = op_params_[i];
+      o.pipe = pipe_;
+      o.global_batch_id = params->global_batch_id;
+      o.mode = params->mode;
+      o.is_presc = presc;
+      ops_[i]->run(&o);
+    }
+  }
+  int hops_ = 0, pipe_ = 1;
+  void *stream_ = nullptr;
+  std::vector<Operator *> ops_;
+  std::vector<OpParams> op_params_;
+};
+
+// ------------------------------------------------------------------- server
+class GPUServer : public Server {
+ public:
+  void Initialize(int global_shard_count, std::vector<int> fanout, int in_memory_mode, int dyn_cache) override {
+    if (global_shard_count != 1) {
+      std::fprintf(stderr, "this build drives one GPU; got gpu_number=%d\n", global_shard_count);
+      std::exit(EXIT_FAILURE);
+    }
+    std::string err;
+    if (!LegionReadMetaConfig("./meta_config", &meta_, &err)) {
+      std::fprintf(stderr, "%s\n", err.c_str());
+      std::exit(EXIT_FAILURE);
+    }
+    fanout_ = fanout;
+    dyn_cache_ = dyn_cache;
+    lmi_config cfg;
+    std::memset(&cfg, 0, sizeof(cfg));
+    cfg.device_id = 0;
+    cfg.batch_size = meta_.batch_size;
+    cfg.hops = (int)fanout.size();
+    for (int k = 0; k < cfg.hops && k < LMI_MAX_HOPS; ++k) cfg.fanout[k] = fanout[k];
+    cfg.feat_dim = meta_.feature_dim;
+    cfg.feat_dtype = LMI_F32;
+    cfg.pipes = 2;
+    cfg.seed = 1;
+    LMI_MUST(lmi_server_create(&cfg, &h_));
+
+    const std::string &dp = meta_.dataset_path;
+    const std::string fp = meta_.feature_path.empty() ? dp : meta_.feature_path;
+    // topology: int64 row pointers, int32 neighbour ids (dataset/README.md:3-10)
+    std::vector<int64_t> indptr((size_t)meta_.node_num + 1);
+    std::vector<int32_t> indices((size_t)meta_.edge_num);
+    must_read(dp + "edge_src", indptr.data(), (meta_.node_num + 1) * 8);
+    must_read(dp + "edge_dst", indices.data(), meta_.edge_num * 4);
+    LMI_MUST(lmi_graph_load(h_, indptr.data(), indices.data(), meta_.node_num, meta_.edge_num, LMI_LOC_HOST));
+    // features: pinned + mapped host memory, read zero-copy on cache misses
+    const int64_t fbytes = meta_.node_num * (int64_t)meta_.feature_dim * 4;
+    LMI_MUST(lmi_host_alloc((size_t)fbytes, &host_features_));
+    must_read(fp + "features", host_features_, fbytes);
+    LMI_MUST(lmi_features_attach(h_, host_features_, meta_.node_num, LMI_LOC_HOST));
+    // id sets with their labels
+    std::vector<int32_t> labels((size_t)meta_.node_num, -1);
+    const bool have_labels = read_file(fp + "labels", labels.data(), meta_.node_num * 4) == meta_.node_num * 4;
+    const char *names[3] = {"trainingset", "validationset", "testingset"};
+    const int64_t counts[3] = {meta_.training_set_num, meta_.validation_set_num, meta_.testing_set_num};
+    for (int m = 0; m < 3; ++m) {
+      if (counts[m] <= 0) continue;
+      std::vector<int32_t> ids((size_t)counts[m]), lab((size_t)counts[m], -1);
+      must_read(dp + names[m], ids.data(), counts[m] * 4);
+      if (have_labels)
+        for (int64_t i = 0; i < counts[m]; ++i)
+          if (ids[i] >= 0 && ids[i] < meta_.node_num) lab[i] = labels[ids[i]];
+      LMI_MUST(lmi_idset_load(h_, m, ids.data(), have_labels ? lab.data() : nullptr, counts[m], LMI_LOC_HOST));
+    }
+    runner_ = NewGPURunner();
+    params_.device_id = 0;
+    params_.fanout = fanout;
+    params_.cache = params_.graph = params_.feature = nullptr;
+    params_.env = h_;
+    params_.global_batch_id = 0;
+    params_.in_memory = in_memory_mode != 0;
+    params_.dyn_cache = dyn_cache;
+    params_.fused = std::getenv("LEGION_MI_OPERATOR_TABLE") == nullptr;
+    runner_->Initialize(&params_);
+    std::cout << "Storage Initialized\n";
+  }
+
+  void PreSc(int cache_agg_mode) override {
+    if (cache_agg_mode != 0) {
+      std::fprintf(stderr, "cache aggregation across GPUs is not part of this build (mode %d)\n", cache_agg_mode);
+      std::exit(EXIT_FAILURE);
+    }
+    const int64_t row_bytes = (int64_t)meta_.feature_dim * 4;
+    if (dyn_cache_ & LEGION_DYN_COMP) {
+      const int64_t rows = std::max<int64_t>(1, meta_.cache_memory / (meta_.feature_dim + 4));
+      LMI_MUST(lmi_cache_build_int8(h_, rows, LMI_TABLE_RANK));
+    } else if (dyn_cache_ & LEGION_DYN_ENABLE) {
+      const int ways = 8;  // cache/cache.cu:629
+      const int64_t sets = std::max<int64_t>(1, meta_.cache_memory / row_bytes / ways);
+      LMI_MUST(lmi_cache_build_lru(h_, sets, ways));
+    } else {
+      const int64_t rows = std::max<int64_t>(1, meta_.cache_memory / row_bytes);
+      LMI_MUST(lmi_cache_build_static(h_, rows, LMI_TABLE_RANK));
+    }
+    lmi_cache_info ci;
+    LMI_MUST(lmi_cache_info_get(h_, &ci));
+    std::cout << "Cache rows: " << ci.capacity_rows << " (" << ci.capacity_rows * ci.row_bytes << " bytes)\n";
+    std::cout << "System is ready for serving\n";  // the line the reference's scripts wait for
+  }
+
+  void Run() override {
+    int32_t steps = 0;
+    LMI_MUST(lmi_steps_per_epoch(h_, LMI_MODE_TRAIN, &steps));
+    const auto t0 = std::chrono::steady_clock::now();
+    int64_t batches = 0;
+    for (int e = 0; e < meta_.epoch; ++e) {
+      for (int i = 0; i < steps; ++i) {
+        params_.global_batch_id = i;
+        runner_->RunOnce(&params_);
+        if (sink_) {
+          lmi_batch_view v;
+          LMI_MUST(lmi_batch_view_get(h_, runner_->CurrentPipe(), &v));
+          sink_(&v, 0, runner_->CurrentPipe(), runner_->Stream(), sink_user_);
+        }
+        ++batches;
+      }
+    }
+    LMI_MUST(lmi_stream_sync(runner_->Stream()));
+    const double sec = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    std::printf("batches: %lld  time per sample: %.1f us  (%.1f batches/s)\n", (long long)batches,
+                batches ? sec * 1e6 / batches : 0.0, sec > 0 ? batches / sec : 0.0);
+  }
+
+  void Finalize() override {
+    if (runner_) {
+      runner_->Finalize(&params_);
+      delete runner_;
+      runner_ = nullptr;
+    }
+    if (h_) LMI_MUST(lmi_server_destroy(h_));
+    h_ = nullptr;
+    if (host_features_) LMI_MUST(lmi_host_free(host_features_));
+    host_features_ = nullptr;
+  }
+
+  void SetBatchSink(LegionBatchSink sink, void *user) override {
+    sink_ = sink;
+    sink_user_ = user;
+  }
+  lmi_server *Handle(int) override { return h_; }
+
+ private:
+  LegionMetaConfig meta_;
+  std::vector<int> fanout_;
+  int dyn_cache_ = 0;
+  lmi_server *h_ = nullptr;
+  void *host_features_ = nullptr;
+  Runner *runner_ = nullptr;
+  RunnerParams params_{};
+  LegionBatchSink sink_ = nullptr;
+  void *sink_user_ = nullptr;
+};
+
+}  // namespace
+
+bool LegionReadMetaConfig(const std::string &path, LegionMetaConfig *out, std::string *error) {
+  std::ifstream f(path);
+  if (!f.is_open()) {
+    if (error) *error = "unable to open meta config file " + path;
+    return false;
+  }
+  std::string line;
+  std::getline(f, line);
+  std::istringstream iss(line);
+  LegionMetaConfig m;
+  if (!(iss >> m.dataset_path >> m.batch_size >> m.node_num >> m.edge_num >> m.feature_dim >> m.training_set_num >>
+        m.validation_set_num >> m.testing_set_num >> m.cache_memory >> m.epoch)) {
+    if (error) *error = "meta config needs: path batch nodes edges dim train valid test cache_bytes epoch [feat_path]";
+    return false;
+  }
+  iss >> m.feature_path;  // optional
+  if (m.batch_size < 1 || m.node_num < 1 || m.edge_num < 0 || m.feature_dim < 1 || m.epoch < 0) {
+    if (error) *error = "meta config holds a non-positive size";
+    return false;
+  }
+  if (!m.dataset_path.empty() && m.dataset_path.back() != '/') m.dataset_path += '/';
+  if (!m.feature_path.empty() && m.feature_path.back() != '/') m.feature_path += '/';
+  *out = m;
+  return true;
+}
+
+Server *NewGPUServer() { return new GPUServer(); }
+Runner *NewGPURunner() { return new GPURunner(); }
+Operator *NewBatchGenerateOP(int op_id) { return new BatchGenerateOP(op_id); }
+Operator *NewRandomSampleOP(int op_id) { return new RandomSampleOP(op_id); }
+Operator *NewCacheLookupOP(int op_id) { return new CacheLookupOP(op_id); }
+Operator *NewSSDIOSubmitOP(int op_id) { return new SSDIOSubmitOP(op_id); }
+Operator *NewSSDIOCompleteOP(int op_id) { return new SSDIOCompleteOP(op_id); }

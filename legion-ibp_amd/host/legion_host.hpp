@@ -1,0 +1,129 @@
+// Host-side C++ interface of the sampling server, above the C ABI.
+//
+// Same class and factory names, argument meaning and call order as the
+// reference's host interface, so its callers keep compiling against this header:
+//   Server / Runner / RunnerParams / NewGPUServer / NewGPURunner
+//       (Legion-IBP sampling_server/src/engine/server.h:5-34; callers main.cu:8-16,
+//        sampling_server.cpp:9-13)
+//   Operator / OpParams / New*OP factories
+//       (sampling_server/src/engine/operator.h:6-35)
+// Everything below these classes goes through include/legion_mi.h; no HIP type
+// appears here (streams and events travel as void*).
+//
+// Differences a caller can observe:
+//   * one GPU: Initialize() rejects global_shard_count != 1 and PreSc() rejects a
+//     cache aggregation mode other than 0 (no cross-GPU cache pooling);
+//   * errors are printed and end the process, like the reference's cudaCheckError,
+//     but every message names the failing C-ABI call and its error text;
+//   * `dyn_cache` keeps the reference's bit meaning where a counterpart exists:
+//     0 = static hot-set cache, DYN_ENABLE (1) = LRU dynamic cache,
+//     DYN_COMP (8) = compressed (int8) cache; other bits are ignored;
+//   * the hand-off to a trainer is a callback (SetBatchSink) instead of CUDA IPC +
+//     POSIX semaphores; the buffers it receives are the reference's output contract.
+#pragma once
+
+#include <cstdint>
+#include <string>
+#include <vector>
+
+#include "../../include/legion_mi.h"
+
+// dyn_cache bits understood here (reference: comp_cache/cache_helper.cuh:34-45)
+enum LegionDynFlags : int { LEGION_DYN_ENABLE = 1 << 0, LEGION_DYN_COMP = 1 << 3 };
+
+struct RunnerParams {
+  int device_id;
+  std::vector<int> fanout;
+  void *cache;    // unused: the caches live behind the lmi_server handle
+  void *graph;    // unused
+  void *feature;  // unused
+  void *env;      // lmi_server* of this GPU
+  int global_batch_id;
+  bool in_memory;
+  int dyn_cache;
+  // additions (defaulted, so reference-style aggregate use still works)
+  bool fused = false;  // true: RunOnce calls lmi_run_once instead of the operator table
+  int mode = LMI_MODE_TRAIN;
+};
+
+// Called once per finished batch with the pipe's device buffers; the stream has
+// been made to wait for the whole batch (lmi_batch_wait) before the call.
+typedef void (*LegionBatchSink)(const lmi_batch_view *batch, int device_id, int pipe, void *stream, void *user);
+
+class Server {
+ public:
+  virtual ~Server() {}
+  // Reads ./meta_config and the dataset it names, creates the per-GPU server.
+  virtual void Initialize(int global_shard_count, std::vector<int> fanout, int in_memory_mode, int dyn_cache) = 0;
+  // Builds the feature cache (the reference presamples here; this build ranks by degree).
+  virtual void PreSc(int cache_agg_mode) = 0;
+  // epoch x steps mini-batches through the runner.
+  virtual void Run() = 0;
+  virtual void Finalize() = 0;
+  // additions
+  virtual void SetBatchSink(LegionBatchSink sink, void *user) = 0;
+  virtual lmi_server *Handle(int device_id) = 0;
+};
+Server *NewGPUServer();
+
+class Runner {
+ public:
+  virtual ~Runner() {}
+  virtual void Initialize(RunnerParams *params) = 0;
+  virtual void InitializeFeaturesBuffer(RunnerParams *params) = 0;  // buffers are sized at create: no-op
+  virtual void RunPreSc(RunnerParams *params) = 0;                  // sampling only, no gather
+  virtual void RunOnce(RunnerParams *params) = 0;
+  virtual void Finalize(RunnerParams *params) = 0;
+  virtual int CurrentPipe() const = 0;  // pipe holding the batch RunOnce produced last
+  virtual void *Stream() const = 0;
+};
+Runner *NewGPURunner();
+
+struct OpParams {
+  int device_id;
+  void *stream;  // hipStream_t
+  void *event;   // hipEvent_t (unused: ordering is by stream)
+  void *memorypool;  // unused
+  void *cache;       // unused
+  void *graph;       // unused
+  void *feature;     // unused
+  void *env;         // lmi_server*
+  int neighbor_count;  // fanout of the hop this operator samples
+  bool is_presc;
+  bool in_memory;
+  int hop_num;
+  int dyn_cache;
+  // additions
+  int pipe = 0;
+  int global_batch_id = 0;
+  int mode = LMI_MODE_TRAIN;
+};
+
+class Operator {
+ public:
+  virtual ~Operator() {}
+  virtual void run(OpParams *params) = 0;
+};
+
+// op_id is the slot in the runner's table, as in the reference: slot 0 stages the
+// seeds, slots 3k sample hop k, slots 3k+1 look up and gather, slots 3k+2 are the
+// (empty) IO submit, the last slot completes the batch (engine/server.cu:218-228).
+Operator *NewBatchGenerateOP(int op_id);
+Operator *NewRandomSampleOP(int op_id);
+Operator *NewCacheLookupOP(int op_id);
+Operator *NewSSDIOSubmitOP(int op_id);
+Operator *NewSSDIOCompleteOP(int op_id);
+
+// The one-line ./meta_config the reference's launcher writes
+// (legion_server.py:43-44; parsed positionally in storage_management.cu:33-104).
+struct LegionMetaConfig {
+  std::string dataset_path;
+  int batch_size = 0;
+  int64_t node_num = 0, edge_num = 0;
+  int feature_dim = 0;
+  int64_t training_set_num = 0, validation_set_num = 0, testing_set_num = 0;
+  int64_t cache_memory = 0;  // bytes
+  int epoch = 1;
+  std::string feature_path;  // optional alternative directory for features / labels
+};
+bool LegionReadMetaConfig(const std::string &path, LegionMetaConfig *out, std::string *error);
