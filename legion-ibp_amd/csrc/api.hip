@@ -85,7 +85,8 @@ static int dmalloc(T **p, int64_t count) {
 static void pipe_free(Pipe &p) {
   void *ptrs[] = {p.ids, p.features, p.labels, p.agg_src_ids, p.agg_src_off, p.agg_dst_off, p.blk_indptr[0],
                   p.blk_indptr[1], p.blk_indptr[2], p.cache_index, p.st, p.dedup.slots, p.eslot, p.firstv,
-                  p.cnt, p.rank, p.tile_sums, p.miss_list, p.lru_fill, p.seed_stage};
+                  p.cnt, p.rank, p.tile_sums, p.miss_list, p.lru_fill, p.seed_stage,
+                  p.chain_status[0], p.chain_status[1]};
   for (void *q : ptrs)
     if (q) (void)hipFree(q);
   if (p.graph_exec) (void)hipGraphExecDestroy(p.graph_exec);
@@ -107,8 +108,10 @@ static int pipe_alloc(Server *s, Pipe &p) {
   LMI_TRY(dmalloc(&p.cache_index, s->max_nodes));
   LMI_TRY(dmalloc(&p.st, 1));
   LMI_HIP(hipMemset(p.st, 0, sizeof(DevState)));
+  // load factor <= 2/3 in the worst case (every sampled edge a new node); real batches
+  // fill a few percent, and a smaller table is cheaper to clear and to probe
   int lg = 4;
-  while ((int64_t(1) << lg) < 2 * s->max_nodes) ++lg;
+  while ((int64_t(1) << lg) * 2 < 3 * s->max_nodes) ++lg;
   p.dedup.log2cap = lg;
   LMI_HIP(hipMalloc(&p.dedup.slots, size_t(8) << lg));
   LMI_TRY(dmalloc(&p.eslot, s->max_edges_hop));
@@ -117,6 +120,9 @@ static int pipe_alloc(Server *s, Pipe &p) {
   LMI_TRY(dmalloc(&p.cnt, scan_n + 1));
   LMI_TRY(dmalloc(&p.rank, s->max_edges_hop + 1));
   LMI_TRY(dmalloc(&p.tile_sums, ceil_div(scan_n, 2048) + 1));
+  p.max_tiles = (int32_t)ceil_div(scan_n, 256) + 1;  // the finest tiling any scan kernel uses
+  LMI_TRY(dmalloc(&p.chain_status[0], p.max_tiles));
+  LMI_TRY(dmalloc(&p.chain_status[1], p.max_tiles));
   LMI_TRY(dmalloc(&p.miss_list, s->max_nodes));
   LMI_TRY(dmalloc(&p.lru_fill, s->max_nodes));
   LMI_TRY(dmalloc(&p.seed_stage, s->cfg.batch_size));
@@ -435,7 +441,7 @@ int lmi_op_batch_generate(lmi_server *h, int pipe, void *stream, const int32_t *
   BatchParams bp{};
   LMI_TRY(pipe_join(p, st));
   LMI_TRY(batch_params(s, p, st, seeds, n, seeds_location, batch_counter, mode, rng_seed, &bp));
-  return launch_batch_generate(s, p, st, bp);
+  return launch_batch_generate(s, p, st, bp, true);
 }
 
 int lmi_op_random_sample(lmi_server *h, int pipe, void *stream, int hop) {
@@ -446,7 +452,7 @@ int lmi_op_random_sample(lmi_server *h, int pipe, void *stream, int hop) {
   if (hop != p.hops_done || hop >= s->cfg.hops) LMI_FAIL(LMI_ERR_ARG, "hop %d out of order (next is %d)", hop, p.hops_done);
   hipStream_t st = (hipStream_t)stream;
   prof_phase(s, st, PROF_SAMPLE);
-  LMI_TRY(launch_hop(s, p, st, hop));
+  LMI_TRY(launch_hop(s, p, st, hop, false));
   prof_phase(s, st, -1);
   return LMI_OK;
 }
@@ -489,8 +495,8 @@ static int capture_batch_graph(Server *s, Pipe &p, hipStream_t st, const BatchPa
   const bool prof = s->prof_on;
   s->prof_on = false;  // no event records inside the capture
   LMI_HIP(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
-  int rc = launch_batch_generate(s, p, st, bp);
-  for (int k = 0; rc == LMI_OK && k < s->cfg.hops; ++k) rc = launch_hop(s, p, st, k);
+  int rc = launch_batch_generate(s, p, st, bp, false);
+  for (int k = 0; rc == LMI_OK && k < s->cfg.hops; ++k) rc = launch_hop(s, p, st, k, true);
   if (rc == LMI_OK) rc = launch_lookup(s, p, st, 0, s->cfg.hops);
   hipGraph_t g = nullptr;
   const hipError_t e = hipStreamEndCapture(st, &g);
@@ -531,8 +537,8 @@ int lmi_run_once(lmi_server *h, int pipe, void *stream, const int32_t *seeds, in
     LMI_TRY(graph_update_begin(s, p, bp));
     LMI_HIP(hipGraphLaunch(p.graph_exec, st));
   } else {
-    LMI_TRY(launch_batch_generate(s, p, st, bp));
-    for (int k = 0; k < s->cfg.hops; ++k) LMI_TRY(launch_hop(s, p, st, k));
+    LMI_TRY(launch_batch_generate(s, p, st, bp, false));
+    for (int k = 0; k < s->cfg.hops; ++k) LMI_TRY(launch_hop(s, p, st, k, true));
     LMI_TRY(launch_lookup(s, p, st, 0, s->cfg.hops));
   }
   LMI_TRY(launch_gather_seg(s, p, st, 0, s->cfg.hops));
@@ -579,6 +585,7 @@ int lmi_batch_counters(lmi_server *h, int pipe, void *stream, int32_t node_count
   LMI_HIP(hipMemcpy(&hs, s->pipes[pipe].st, sizeof(DevState), hipMemcpyDeviceToHost));
   if (node_counter) memcpy(node_counter, hs.node_counter, 64);
   if (edge_counter) memcpy(edge_counter, hs.edge_counter, 64);
+  if (hs.scan_fault) LMI_FAIL(LMI_ERR_HIP, "a device scan timed out waiting for an earlier tile");
   if (hs.bad_id) LMI_FAIL(LMI_ERR_BAD_ID, "a seed id outside [0, %lld) was skipped", (long long)s->n_nodes);
   return LMI_OK;
 }

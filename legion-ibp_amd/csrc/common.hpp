@@ -48,7 +48,8 @@ struct DevState {
   // One miss list per lookup segment (0 = seeds or the whole
   // batch, k = nodes added by hop k); zeroed at batch start.
   int32_t n_miss[LMI_MAX_HOPS + 1];
-  int32_t reserved[LMI_MAX_HOPS + 1];
+  int32_t scan_fault;  // a look-back scan gave up waiting (never expected; reported as an error)
+  int32_t reserved[LMI_MAX_HOPS];
   int32_t bad_id;      // set when a seed id is outside [0, n_nodes)
   int32_t scan_total;  // total of the last device scan
   // per-batch parameters, written by the first kernel of a batch so that every
@@ -88,6 +89,8 @@ struct Pipe {
   int32_t *cnt = nullptr;      // [max(max_nodes, max_edges_hop)] scan input
   int32_t *rank = nullptr;     // [max_edges_hop + 1] scan output
   int32_t *tile_sums = nullptr;
+  unsigned long long *chain_status[2] = {nullptr, nullptr};  // look-back scan state: [0] node scans, [1] edge scans
+  int32_t max_tiles = 0;
   int2 *miss_list = nullptr;   // [max_nodes] (row, id) pairs of cache misses
   int32_t *lru_fill = nullptr;                        // [max_nodes] slot granted to a miss
   hipStream_t side = nullptr;  // second stream for the host-link gather
@@ -183,9 +186,10 @@ int prof_end(Server *s, hipStream_t st, int handle);
 void prof_phase(Server *s, hipStream_t st, int next_kind);
 
 // sampler.hip
-int launch_batch_generate(Server *s, Pipe &p, hipStream_t st, const BatchParams &bp);
+// stage_seeds: also run the seed-staging kernel now (otherwise hop 0 stages them itself)
+int launch_batch_generate(Server *s, Pipe &p, hipStream_t st, const BatchParams &bp, bool stage_seeds);
 int graph_update_begin(Server *s, Pipe &p, const BatchParams &bp);
-int launch_hop(Server *s, Pipe &p, hipStream_t st, int hop);
+int launch_hop(Server *s, Pipe &p, hipStream_t st, int hop, bool stage_seeds);
 int launch_table_clear(Table &t, hipStream_t st);
 
 enum { SCAN_EPI_NONE = 0, SCAN_EPI_HOP_EDGES = 1, SCAN_EPI_HOP_NODES = 2 };

@@ -40,23 +40,29 @@ __device__ __forceinline__ uint32_t hash_id(int32_t key, int log2cap) {
 }
 
 // Insert `key` (if absent) and lower its value to min(value, cand); returns the
-// slot index.  Keys only ever go EMPTY -> key, so a stale non-empty read is
-// still correct and a stale EMPTY read is resolved by the CAS.
+// slot index.  One 8-byte load reads key and value together.  Keys only ever go
+// EMPTY -> key, so a stale non-empty read is still correct and a stale EMPTY read
+// is resolved by the CAS.  Values only ever decrease, so a stale value is never
+// too low: when the value read is already <= cand the atomic can be skipped, which
+// removes almost all same-address atomics on frequently sampled hub nodes.
 __device__ __forceinline__ uint32_t table_insert_min(HashSlot *slots, int log2cap, int32_t key,
                                                      int32_t cand) {
   const uint32_t mask = (1u << log2cap) - 1u;
   uint32_t h = hash_id(key, log2cap);
   while (true) {
-    int32_t k = slots[h].key;
+    const int2 kv = *reinterpret_cast<const int2 *>(&slots[h]);
+    int32_t k = kv.x, v = kv.y;
     if (k == kEmptyKey) {
       k = atomicCAS(&slots[h].key, kEmptyKey, key);
       if (k == kEmptyKey) k = key;
+      v = kIntMax;  // unknown: take the atomic path
     }
-    if (k == key) break;
+    if (k == key) {
+      if (v > cand) atomicMin(&slots[h].val, cand);
+      return h;
+    }
     h = (h + 1) & mask;
   }
-  atomicMin(&slots[h].val, cand);
-  return h;
 }
 
 // Read-only probe: value or -1.

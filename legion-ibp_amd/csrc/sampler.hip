@@ -12,21 +12,53 @@
 // minstd_rand; an open-addressing hash table in HBM instead of an N-bit bitmap
 // plus an N-entry position map; scans instead of atomics for placement, so the
 // edge order is (node, slot) and local ids follow first occurrence in that order.
+//
+// A hop is four kernels:
+//   1. hop_count_scan   per-node output counts -> block-CSR row pointers (single-pass
+//                       scan); for hop 0 it also stages the seeds
+//   2. hop_sample       draw positions, write edges, insert sources into the dedup table
+//   3. hop_flag_scan    first-occurrence flags -> ranks (single-pass scan), new node count
+//   4. hop_relabel      local ids of edge sources, append new nodes to ids[]
+#include <algorithm>
+
 #include "scan.hpp"
 
 namespace lmi {
 
+struct HopArgs {
+  // graph
+  const int64_t *indptr;
+  const int32_t *indices;
+  int64_t n_nodes;
+  int fanout, hop;
+  // pipe
+  DevState *st;
+  int32_t *ids, *labels;
+  int32_t *row_ptr;  // block CSR row pointers of this hop
+  int32_t *agg_src_ids, *agg_src_off, *agg_dst_off;
+  HashSlot *slots;
+  int log2cap;
+  int32_t *eslot, *firstv, *rank;
+  ScanChain chain_nodes, chain_edges;
+  int max_tiles;
+  int stage_seeds;  // hop 0 only: the seeds have not been staged by batch_generate_kernel yet
+};
+
 // ------------------------------------------------------------ batch start
 // Clears the dedup table (key = -1, value = INT_MAX), resets the pipe state and
-// stores the per-batch parameters where the later kernels read them.
-static __global__ __launch_bounds__(256) void batch_begin_kernel(HashSlot *slots, int64_t n_slots,
-                                                                 DevState *st, int hops, BatchParams bp) {
+// the scan chains, and stores the per-batch parameters where later kernels read them.
+static __global__ __launch_bounds__(256) void batch_begin_kernel(HashSlot *slots, int64_t n_slots, DevState *st,
+                                                                 int hops, ScanChain chain_nodes,
+                                                                 ScanChain chain_edges, int max_tiles,
+                                                                 BatchParams bp) {
   const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   // two slots (16 bytes) per store
   const int4 fill = make_int4(kEmptyKey, kIntMax, kEmptyKey, kIntMax);
   int4 *p = reinterpret_cast<int4 *>(slots);
   for (int64_t i = tid; i < n_slots / 2; i += stride) p[i] = fill;
+  scan_chain_reset(chain_nodes, max_tiles, tid, stride);
+  scan_chain_reset(chain_edges, max_tiles, tid, stride);
   if (tid == 0) {
     int32_t *w = reinterpret_cast<int32_t *>(st);
     for (int i = 0; i < (int)(sizeof(DevState) / 4); ++i) w[i] = 0;
@@ -43,8 +75,8 @@ static __global__ __launch_bounds__(256) void batch_begin_kernel(HashSlot *slots
   }
 }
 
-// Stage the seeds: ids[i] = seed, labels, and table[seed] = min(i) so that a
-// repeated seed resolves to its first row.
+// Stage the seeds on their own (operator-by-operator use, where the seeds' cache
+// lookup runs before the first hop): ids[i] = seed, labels, table[seed] = min(i).
 static __global__ __launch_bounds__(256) void batch_generate_kernel(int64_t n_nodes, int32_t *ids, int32_t *labels,
                                                                     HashSlot *slots, int log2cap, DevState *st) {
   const int i = blockIdx.x * blockDim.x + threadIdx.x;
@@ -60,31 +92,83 @@ static __global__ __launch_bounds__(256) void batch_generate_kernel(int64_t n_no
 }
 
 // ------------------------------------------------------------- hop, phase 1
-// cnt[i] = min(deg(ids[i]), fanout) for every node known so far, plus tile sums.
-static __global__ __launch_bounds__(kScanBlock) void hop_count_kernel(
-    const int32_t *ids, const int64_t *indptr, int64_t n_nodes, int fanout, int hop, const DevState *st,
-    int32_t *cnt, int32_t *tile_sums) {
-  __shared__ int lds[kScanBlock / kWave];
-  const int n = st->node_counter[9 + hop];
-  const int n_tiles = (n + kScanTile - 1) / kScanTile;
-  for (int tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
-    const int base = tile * kScanTile + threadIdx.x * kScanItems;
-    int sum = 0;
+// row_ptr[i] = exclusive prefix of min(deg(ids[i]), fanout) over every node known
+// so far; the total is the hop's edge count.  Hop 0 first stages the seeds:
+// ids[i] = seed, labels, and table[seed] = min(i) so that a repeated seed resolves
+// to its first row.
+template <int ITEMS>
+static __global__ __launch_bounds__(kScanBlock) void hop_count_scan_kernel(HopArgs a) {
+  constexpr int TILE = kScanBlock * ITEMS;
+  __shared__ int lds[kScanBlock / kWave + 1];
+  __shared__ int s_prefix;
+  DevState *st = a.st;
+  const int n = st->node_counter[9 + a.hop];
+  const int n_tiles = (n + TILE - 1) / TILE;
+  if (n_tiles == 0) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+      a.row_ptr[0] = 0;
+      scan_epilogue(SCAN_EPI_HOP_EDGES, st, a.hop, 0);
+    }
+    return;
+  }
+  const int tile = blockIdx.x;
+  if (tile < n_tiles) {
+    const int base = tile * TILE + threadIdx.x * ITEMS;
+    int32_t id[ITEMS];
+    // 1. node ids (hop 0: stage the seeds)
 #pragma unroll
-    for (int j = 0; j < kScanItems; ++j) {
+    for (int j = 0; j < ITEMS; ++j) {
       const int i = base + j;
+      id[j] = -1;
       if (i < n) {
-        const int32_t v = ids[i];
-        int c = 0;
-        if (v >= 0 && v < n_nodes) {
-          const int64_t deg = indptr[v + 1] - indptr[v];
-          c = (int)(deg < (int64_t)fanout ? deg : (int64_t)fanout);
+        if (a.stage_seeds) {
+          id[j] = st->seeds[i];
+          a.ids[i] = id[j];
+          a.labels[i] = st->labels_in ? st->labels_in[i] : -1;
+        } else {
+          id[j] = a.ids[i];
         }
-        cnt[i] = c;
-        sum += c;
+        if (id[j] < 0 || id[j] >= a.n_nodes) {
+          if (a.stage_seeds) st->bad_id = 1;
+          id[j] = -1;
+        }
       }
     }
-    tile_reduce_store(sum, tile_sums, tile, lds);
+    // 2. all row-pointer loads in flight together
+    int64_t lo[ITEMS], hi[ITEMS];
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+      lo[j] = hi[j] = 0;
+      if (id[j] >= 0) {
+        lo[j] = a.indptr[id[j]];
+        hi[j] = a.indptr[id[j] + 1];
+      }
+    }
+    if (a.stage_seeds) {
+#pragma unroll
+      for (int j = 0; j < ITEMS; ++j)
+        if (id[j] >= 0) table_insert_min(a.slots, a.log2cap, id[j], base + j);
+    }
+    int v[ITEMS], sum = 0;
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+      const int64_t deg = hi[j] - lo[j];
+      v[j] = (int)(deg < (int64_t)a.fanout ? deg : (int64_t)a.fanout);
+      sum += v[j];
+    }
+    int total;
+    const int ex = block_exclusive_scan<kScanBlock>(sum, lds, total);
+    const int prefix = scan_tile_prefix(a.chain_nodes, tile, total, &s_prefix, &st->scan_fault);
+    int run = prefix + ex;
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+      if (base + j < n) a.row_ptr[base + j] = run;
+      run += v[j];
+    }
+    if (tile == n_tiles - 1 && threadIdx.x == 0) {
+      a.row_ptr[n] = prefix + total;
+      scan_epilogue(SCAN_EPI_HOP_EDGES, st, a.hop, prefix + total);
+    }
   }
 }
 
@@ -95,22 +179,23 @@ static __global__ __launch_bounds__(kScanBlock) void hop_count_kernel(
 // Every sampled edge is inserted into the dedup table with candidate value
 // n_prev + e (e = edge index inside the hop); atomicMin keeps the first edge.
 template <int G>
-static __global__ __launch_bounds__(256) void hop_sample_kernel(
-    const int32_t *ids, const int64_t *indptr, const int32_t *indices, int64_t n_nodes, int fanout,
-    int hop, const DevState *st, const int32_t *row_ptr, int32_t *agg_src_ids, int32_t *agg_dst_off,
-    HashSlot *slots, int log2cap, int32_t *eslot) {
+static __global__ __launch_bounds__(256) void hop_sample_kernel(HopArgs a) {
+  const DevState *st = a.st;
+  const int64_t flat = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  scan_chain_reset(a.chain_edges, a.max_tiles, flat, (int64_t)gridDim.x * blockDim.x);
   const uint64_t seed = (uint64_t)st->rng_lo | ((uint64_t)st->rng_hi << 32);
-  const int n_prev = st->node_counter[9 + hop];
-  const int eoff = st->edge_counter[12 + hop + 1];
+  const int n_prev = st->node_counter[9 + a.hop];
+  const int eoff = st->edge_counter[12 + a.hop + 1];
+  const int fanout = a.fanout;
   const int lane = threadIdx.x & (G - 1);
-  const int group = (blockIdx.x * blockDim.x + threadIdx.x) / G;
+  const int group = (int)(flat / G);
   const int n_groups = gridDim.x * blockDim.x / G;
   for (int i = group; i < n_prev; i += n_groups) {
-    const int32_t v = ids[i];
-    if (v < 0 || v >= n_nodes) continue;
-    const int64_t beg = indptr[v];
-    const int64_t deg = indptr[v + 1] - beg;
-    const int base = row_ptr[i];
+    const int32_t v = a.ids[i];
+    if (v < 0 || v >= a.n_nodes) continue;
+    const int64_t beg = a.indptr[v];
+    const int64_t deg = a.indptr[v + 1] - beg;
+    const int base = a.row_ptr[i];
     int64_t pick = lane;
     int count;
     if (deg <= (int64_t)fanout) {
@@ -119,7 +204,7 @@ static __global__ __launch_bounds__(256) void hop_sample_kernel(
       count = fanout;
       const uint32_t j = (uint32_t)(deg - fanout) + (uint32_t)lane;
       uint32_t t = 0xFFFFFFFFu;
-      if (lane < fanout) t = __umulhi(sample_draw(seed, (uint32_t)hop, (uint32_t)v, (uint32_t)lane), j + 1u);
+      if (lane < fanout) t = __umulhi(sample_draw(seed, (uint32_t)a.hop, (uint32_t)v, (uint32_t)lane), j + 1u);
       bool dup = false;
       for (int q = 0; q + 1 < fanout; ++q) {
         const uint32_t mine = dup ? j : t;
@@ -129,40 +214,58 @@ static __global__ __launch_bounds__(256) void hop_sample_kernel(
       pick = dup ? j : t;
     }
     if (lane < count) {
-      const int32_t nbr = indices[beg + pick];
+      const int32_t nbr = a.indices[beg + pick];
       const int e = base + lane;
-      agg_src_ids[eoff + e] = nbr;
-      agg_dst_off[eoff + e] = i;
-      eslot[e] = (int)table_insert_min(slots, log2cap, nbr, n_prev + e);
+      a.agg_src_ids[eoff + e] = nbr;
+      a.agg_dst_off[eoff + e] = i;
+      a.eslot[e] = (int)table_insert_min(a.slots, a.log2cap, nbr, n_prev + e);
     }
   }
 }
 
 // ------------------------------------------------------------- hop, phase 3
 // firstv[e] = table value of the edge's source; an edge is the first occurrence
-// of a new node iff that value names the edge itself.  cnt[e] = flag, tile sums.
-static __global__ __launch_bounds__(kScanBlock) void hop_flag_kernel(
-    const HashSlot *slots, const int32_t *eslot, int hop, const DevState *st, int32_t *firstv,
-    int32_t *cnt, int32_t *tile_sums) {
-  __shared__ int lds[kScanBlock / kWave];
-  const int n_prev = st->node_counter[9 + hop];
-  const int n = st->edge_counter[9 + hop + 1];
-  const int n_tiles = (n + kScanTile - 1) / kScanTile;
-  for (int tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
-    const int base = tile * kScanTile + threadIdx.x * kScanItems;
-    int sum = 0;
+// of a new node iff that value names the edge itself.  rank[e] = number of first
+// occurrences before e; the total is the number of new nodes.
+template <int ITEMS>
+static __global__ __launch_bounds__(kScanBlock) void hop_flag_scan_kernel(HopArgs a) {
+  constexpr int TILE = kScanBlock * ITEMS;
+  __shared__ int lds[kScanBlock / kWave + 1];
+  __shared__ int s_prefix;
+  DevState *st = a.st;
+  const int n_prev = st->node_counter[9 + a.hop];
+  const int n = st->edge_counter[9 + a.hop + 1];
+  const int n_tiles = (n + TILE - 1) / TILE;
+  if (n_tiles == 0) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) scan_epilogue(SCAN_EPI_HOP_NODES, st, a.hop, 0);
+    return;
+  }
+  const int tile = blockIdx.x;
+  if (tile < n_tiles) {
+    const int base = tile * TILE + threadIdx.x * ITEMS;
+    int v[ITEMS], sum = 0;
 #pragma unroll
-    for (int j = 0; j < kScanItems; ++j) {
+    for (int j = 0; j < ITEMS; ++j) {
       const int e = base + j;
+      int flag = 0;
       if (e < n) {
-        const int32_t val = slots[eslot[e]].val;
-        firstv[e] = val;
-        const int flag = (val == n_prev + e) ? 1 : 0;
-        cnt[e] = flag;
-        sum += flag;
+        const int32_t val = a.slots[a.eslot[e]].val;
+        a.firstv[e] = val;
+        flag = (val == n_prev + e) ? 1 : 0;
       }
+      v[j] = flag;
+      sum += flag;
     }
-    tile_reduce_store(sum, tile_sums, tile, lds);
+    int total;
+    const int ex = block_exclusive_scan<kScanBlock>(sum, lds, total);
+    const int prefix = scan_tile_prefix(a.chain_edges, tile, total, &s_prefix, &st->scan_fault);
+    int run = prefix + ex;
+#pragma unroll
+    for (int j = 0; j < ITEMS; ++j) {
+      if (base + j < n) a.rank[base + j] = run;
+      run += v[j];
+    }
+    if (tile == n_tiles - 1 && threadIdx.x == 0) scan_epilogue(SCAN_EPI_HOP_NODES, st, a.hop, prefix + total);
   }
 }
 
@@ -170,48 +273,42 @@ static __global__ __launch_bounds__(kScanBlock) void hop_flag_kernel(
 // local id of an edge source: an old node keeps its id; a new node gets
 // n_prev + (rank of its first edge among first edges).  First edges also
 // append the node to ids[] and publish the final id in the table.
-static __global__ __launch_bounds__(256) void hop_relabel_kernel(
-    const int32_t *firstv, const int32_t *rank, const int32_t *eslot, int hop, const DevState *st,
-    const int32_t *agg_src_ids, int32_t *agg_src_off, int32_t *ids, HashSlot *slots) {
-  const int n_prev = st->node_counter[9 + hop];
-  const int n = st->edge_counter[9 + hop + 1];
-  const int eoff = st->edge_counter[12 + hop + 1];
-  for (int e = blockIdx.x * blockDim.x + threadIdx.x; e < n; e += gridDim.x * blockDim.x) {
-    const int32_t val = firstv[e];
+static __global__ __launch_bounds__(256) void hop_relabel_kernel(HopArgs a) {
+  const DevState *st = a.st;
+  const int64_t flat = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  scan_chain_reset(a.chain_nodes, a.max_tiles, flat, (int64_t)gridDim.x * blockDim.x);  // for the next hop
+  const int n_prev = st->node_counter[9 + a.hop];
+  const int n = st->edge_counter[9 + a.hop + 1];
+  const int eoff = st->edge_counter[12 + a.hop + 1];
+  for (int e = (int)flat; e < n; e += gridDim.x * blockDim.x) {
+    const int32_t val = a.firstv[e];
     int32_t local = val;
     if (val >= n_prev) {
-      local = n_prev + rank[val - n_prev];
+      local = n_prev + a.rank[val - n_prev];
       if (val == n_prev + e) {
-        ids[local] = agg_src_ids[eoff + e];
-        slots[eslot[e]].val = local;
+        a.ids[local] = a.agg_src_ids[eoff + e];
+        a.slots[a.eslot[e]].val = local;
       }
     }
-    agg_src_off[eoff + e] = local;
+    a.agg_src_off[eoff + e] = local;
   }
 }
 
 // ---------------------------------------------------------------- launchers
-static void begin_args(Server *s, Pipe &p, const BatchParams &bp, void **args, HashSlot **slots, int64_t *n_slots,
-                       DevState **st, int *hops, BatchParams *bpc) {
-  *slots = p.dedup.slots;
-  *n_slots = int64_t(1) << p.dedup.log2cap;
-  *st = p.st;
-  *hops = s->cfg.hops;
-  *bpc = bp;
-  args[0] = slots; args[1] = n_slots; args[2] = st; args[3] = hops; args[4] = bpc;
-}
+static ScanChain chain_of(const Pipe &p, int which) { return ScanChain{p.chain_status[which]}; }
 
 static int begin_grid(const Pipe &p) {
   const int64_t n_slots = int64_t(1) << p.dedup.log2cap;
   return (int)std::min<int64_t>(ceil_div(n_slots / 2, 256), 2048);
 }
 
-int launch_batch_generate(Server *s, Pipe &p, hipStream_t st, const BatchParams &bp) {
+int launch_batch_generate(Server *s, Pipe &p, hipStream_t st, const BatchParams &bp, bool stage_seeds) {
   const int64_t n_slots = int64_t(1) << p.dedup.log2cap;
   hipLaunchKernelGGL(batch_begin_kernel, dim3(begin_grid(p)), dim3(256), 0, st, p.dedup.slots, n_slots, p.st,
-                     s->cfg.hops, bp);
-  hipLaunchKernelGGL(batch_generate_kernel, dim3((s->cfg.batch_size + 255) / 256), dim3(256), 0, st, s->n_nodes,
-                     p.ids, p.labels, p.dedup.slots, p.dedup.log2cap, p.st);
+                     s->cfg.hops, chain_of(p, 0), chain_of(p, 1), p.max_tiles, bp);
+  if (stage_seeds)
+    hipLaunchKernelGGL(batch_generate_kernel, dim3((s->cfg.batch_size + 255) / 256), dim3(256), 0, st, s->n_nodes,
+                       p.ids, p.labels, p.dedup.slots, p.dedup.log2cap, p.st);
   LMI_HIP(hipGetLastError());
   p.n_seeds = bp.n_seeds;
   p.hops_done = 0;
@@ -220,9 +317,14 @@ int launch_batch_generate(Server *s, Pipe &p, hipStream_t st, const BatchParams 
 
 // Re-points the captured graph's first kernel at this batch's parameters.
 int graph_update_begin(Server *s, Pipe &p, const BatchParams &bp) {
-  HashSlot *slots; int64_t n_slots; DevState *st; int hops; BatchParams bpc;
-  void *args[5];
-  begin_args(s, p, bp, args, &slots, &n_slots, &st, &hops, &bpc);
+  HashSlot *slots = p.dedup.slots;
+  int64_t n_slots = int64_t(1) << p.dedup.log2cap;
+  DevState *st = p.st;
+  int hops = s->cfg.hops;
+  ScanChain c0 = chain_of(p, 0), c1 = chain_of(p, 1);
+  int max_tiles = p.max_tiles;
+  BatchParams bpc = bp;
+  void *args[8] = {&slots, &n_slots, &st, &hops, &c0, &c1, &max_tiles, &bpc};
   hipKernelNodeParams kp{};
   kp.func = reinterpret_cast<void *>(batch_begin_kernel);
   kp.gridDim = dim3(begin_grid(p));
@@ -236,41 +338,62 @@ int graph_update_begin(Server *s, Pipe &p, const BatchParams &bp) {
   return LMI_OK;
 }
 
-template <int G>
-static void launch_sample_g(Server *s, Pipe &p, hipStream_t st, int hop, int grid) {
-  hipLaunchKernelGGL(hop_sample_kernel<G>, dim3(grid), dim3(256), 0, st, p.ids, s->indptr, s->indices,
-                     s->n_nodes, s->cfg.fanout[hop], hop, p.st, p.blk_indptr[hop],
-                     p.agg_src_ids, p.agg_dst_off, p.dedup.slots, p.dedup.log2cap, p.eslot);
-}
-
-int launch_hop(Server *s, Pipe &p, hipStream_t st, int hop) {
+int launch_hop(Server *s, Pipe &p, hipStream_t st, int hop, bool stage_seeds) {
   const int f = s->cfg.fanout[hop];
   const int64_t n_max = s->node_cap[hop], e_max = s->edge_cap[hop];
-  // 1. per-node counts -> row pointers of the block CSR (= edge placement)
-  hipLaunchKernelGGL(hop_count_kernel, dim3(scan_grid(n_max)), dim3(kScanBlock), 0, st, p.ids, s->indptr,
-                     s->n_nodes, f, hop, p.st, p.cnt, p.tile_sums);
-  LMI_TRY(launch_scan_phases(st, p.cnt, p.blk_indptr[hop], p.tile_sums, &p.st->node_counter[9 + hop],
-                             n_max, SCAN_EPI_HOP_EDGES, p.st, hop, &p.st->scan_total));
-  // 2. sample + insert
+  HopArgs a{};
+  a.indptr = s->indptr;
+  a.indices = s->indices;
+  a.n_nodes = s->n_nodes;
+  a.fanout = f;
+  a.hop = hop;
+  a.st = p.st;
+  a.ids = p.ids;
+  a.labels = p.labels;
+  a.row_ptr = p.blk_indptr[hop];
+  a.agg_src_ids = p.agg_src_ids;
+  a.agg_src_off = p.agg_src_off;
+  a.agg_dst_off = p.agg_dst_off;
+  a.slots = p.dedup.slots;
+  a.log2cap = p.dedup.log2cap;
+  a.eslot = p.eslot;
+  a.firstv = p.firstv;
+  a.rank = p.rank;
+  a.chain_nodes = chain_of(p, 0);
+  a.chain_edges = chain_of(p, 1);
+  a.max_tiles = p.max_tiles;
+  a.stage_seeds = (hop == 0 && stage_seeds) ? 1 : 0;
+  // one tile per block (blocks past the real item count leave at once); few items per
+  // thread while that keeps the tile count near a thousand: the row-pointer reads are
+  // dependent random accesses, so parallelism matters more than per-thread work
+  const int64_t nm = std::max<int64_t>(n_max, 1);
+  if (nm <= 256 * 1024)
+    hipLaunchKernelGGL(hop_count_scan_kernel<1>, dim3((int)ceil_div(nm, kScanBlock)), dim3(kScanBlock), 0, st, a);
+  else if (nm <= 512 * 1024)
+    hipLaunchKernelGGL(hop_count_scan_kernel<2>, dim3((int)ceil_div(nm, kScanBlock * 2)), dim3(kScanBlock), 0, st, a);
+  else if (nm <= 1024 * 1024)
+    hipLaunchKernelGGL(hop_count_scan_kernel<4>, dim3((int)ceil_div(nm, kScanBlock * 4)), dim3(kScanBlock), 0, st, a);
+  else
+    hipLaunchKernelGGL(hop_count_scan_kernel<8>, dim3((int)ceil_div(nm, kScanBlock * 8)), dim3(kScanBlock), 0, st, a);
   int G = 4;
   while (G < f) G <<= 1;
   const int grid = (int)std::min<int64_t>(ceil_div(n_max * G, 256), 8192);
   switch (G) {
-    case 4: launch_sample_g<4>(s, p, st, hop, grid); break;
-    case 8: launch_sample_g<8>(s, p, st, hop, grid); break;
-    case 16: launch_sample_g<16>(s, p, st, hop, grid); break;
-    case 32: launch_sample_g<32>(s, p, st, hop, grid); break;
-    default: launch_sample_g<64>(s, p, st, hop, grid); break;
+    case 4: hipLaunchKernelGGL(hop_sample_kernel<4>, dim3(grid), dim3(256), 0, st, a); break;
+    case 8: hipLaunchKernelGGL(hop_sample_kernel<8>, dim3(grid), dim3(256), 0, st, a); break;
+    case 16: hipLaunchKernelGGL(hop_sample_kernel<16>, dim3(grid), dim3(256), 0, st, a); break;
+    case 32: hipLaunchKernelGGL(hop_sample_kernel<32>, dim3(grid), dim3(256), 0, st, a); break;
+    default: hipLaunchKernelGGL(hop_sample_kernel<64>, dim3(grid), dim3(256), 0, st, a); break;
   }
-  // 3. first-occurrence flags -> ranks
-  hipLaunchKernelGGL(hop_flag_kernel, dim3(scan_grid(e_max)), dim3(kScanBlock), 0, st, p.dedup.slots,
-                     p.eslot, hop, p.st, p.firstv, p.cnt, p.tile_sums);
-  LMI_TRY(launch_scan_phases(st, p.cnt, p.rank, p.tile_sums, &p.st->edge_counter[9 + hop + 1], e_max,
-                             SCAN_EPI_HOP_NODES, p.st, hop, &p.st->scan_total));
-  // 4. relabel
+  const int64_t em = std::max<int64_t>(e_max, 1);
+  if (em <= 1024 * 1024)
+    hipLaunchKernelGGL(hop_flag_scan_kernel<2>, dim3((int)ceil_div(em, kScanBlock * 2)), dim3(kScanBlock), 0, st, a);
+  else if (em <= 2560 * 1024)
+    hipLaunchKernelGGL(hop_flag_scan_kernel<4>, dim3((int)ceil_div(em, kScanBlock * 4)), dim3(kScanBlock), 0, st, a);
+  else
+    hipLaunchKernelGGL(hop_flag_scan_kernel<8>, dim3((int)ceil_div(em, kScanBlock * 8)), dim3(kScanBlock), 0, st, a);
   const int rgrid = (int)std::min<int64_t>(ceil_div(e_max, 256), 4096);
-  hipLaunchKernelGGL(hop_relabel_kernel, dim3(rgrid), dim3(256), 0, st, p.firstv, p.rank, p.eslot, hop,
-                     p.st, p.agg_src_ids, p.agg_src_off, p.ids, p.dedup.slots);
+  hipLaunchKernelGGL(hop_relabel_kernel, dim3(rgrid), dim3(256), 0, st, a);
   LMI_HIP(hipGetLastError());
   p.hops_done = hop + 1;
   return LMI_OK;

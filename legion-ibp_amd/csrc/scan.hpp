@@ -97,6 +97,82 @@ static __global__ __launch_bounds__(kScanBlock) void scan_apply_kernel(const int
   }
 }
 
+// ---------------------------------------------------------------------------
+// Single-pass scan (decoupled look-back, Merrill & Garland 2016) for the kernels on
+// the per-batch path: the producer kernel itself turns its per-item counts into
+// exclusive prefixes, so a hop needs one launch where the three-phase scan needs
+// three.  One tile per block, tile = blockIdx.x: a tile only ever waits for
+// lower-numbered blocks, which the dispatcher started earlier, and every block
+// publishes its own sum before it looks back, so the wait always ends.  (An
+// atomic ticket would drop the reliance on dispatch order, but 500 same-address
+// atomics cost more than the whole scan.)  The wait is bounded all the same.
+//
+// status[t] = (flag << 32) | value in one 64-bit word, written and read with
+// relaxed device-scope atomics (flag and value travel together, nothing else is
+// exchanged): flag 0 = not ready, 1 = value is the tile's own sum, 2 = value is
+// the inclusive prefix up to and including the tile.  The status words must be
+// zeroed by an earlier kernel of the same stream before each use.
+struct ScanChain {
+  unsigned long long *status;  // [max_tiles]
+};
+
+constexpr unsigned long long kScanAggregate = 1ull << 32, kScanInclusive = 2ull << 32;
+constexpr int kScanSpinLimit = 1 << 16;  // look-back re-reads before a tile gives up and raises DevState::scan_fault
+
+// Zeroes a chain for a later kernel; call from any grid with a flat thread index.
+__device__ __forceinline__ void scan_chain_reset(ScanChain c, int max_tiles, int64_t tid, int64_t n_threads) {
+  for (int64_t i = tid; i < max_tiles; i += n_threads) c.status[i] = 0ull;
+}
+
+__device__ __forceinline__ void scan_publish(ScanChain c, int tile, unsigned long long word) {
+  __hip_atomic_store(&c.status[tile], word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// Publishes this tile's aggregate and returns the exclusive prefix of the tile
+// (sum of all earlier tiles) to every thread of the block.  Wavefront 0 looks back
+// 64 tiles per step.  lds_prefix is one shared int.  Contains __syncthreads.
+__device__ __forceinline__ int scan_tile_prefix(ScanChain c, int tile, int aggregate, int *lds_prefix,
+                                                int32_t *fault) {
+  if (threadIdx.x < kWave) {
+    const int lane = threadIdx.x;
+    int prefix = 0;
+    if (tile == 0) {
+      if (lane == 0) scan_publish(c, 0, kScanInclusive | (unsigned int)aggregate);
+    } else {
+      if (lane == 0) scan_publish(c, tile, kScanAggregate | (unsigned int)aggregate);
+      int base = tile - 1;
+      int spins = 0;
+      // a legitimate wait is a few hundred re-reads (one tile's worth of loads); after a first
+      // fault every later tile gives up almost at once, so a broken chain drains in milliseconds
+      const int spin_limit = *fault ? 64 : kScanSpinLimit;
+      while (true) {
+        const int j = base - lane;
+        unsigned long long w = kScanInclusive;  // before tile 0: an inclusive prefix of 0
+        if (j >= 0) w = __hip_atomic_load(&c.status[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned flag = (unsigned)(w >> 32);
+        const unsigned long long inc = __ballot(flag == 2u), inv = __ballot(flag == 0u);
+        const int first_inc = inc ? (__ffsll((long long)inc) - 1) : (kWave - 1);
+        const unsigned long long window = (first_inc >= kWave - 1) ? ~0ull : ((1ull << (first_inc + 1)) - 1ull);
+        if (inv & window) {  // a tile we need has not published yet: read again
+          if (++spins < spin_limit) continue;
+          if (lane == 0) *fault = 1;  // never expected; bounded so that the grid always drains
+          break;
+        }
+        int contrib = (lane <= first_inc) ? (int)(unsigned)w : 0;
+#pragma unroll
+        for (int d = kWave / 2; d > 0; d >>= 1) contrib += __shfl_xor(contrib, d, kWave);
+        prefix += contrib;
+        if (inc) break;
+        base -= kWave;
+      }
+      if (lane == 0) scan_publish(c, tile, kScanInclusive | (unsigned int)(prefix + aggregate));
+    }
+    if (lane == 0) *lds_prefix = prefix;
+  }
+  __syncthreads();
+  return *lds_prefix;
+}
+
 // Phases 2 and 3.  n_max bounds *n_ptr and sizes the apply grid.
 static inline int launch_scan_phases(hipStream_t st, const int32_t *cnt, int32_t *out,
                                      int32_t *tile_sums, const int32_t *n_ptr, int64_t n_max,
