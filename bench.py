@@ -52,6 +52,19 @@ WORKLOADS = {
 }
 
 
+def recorded_traffic(workload):
+    """HBM bytes per launch of the hit gather, from the committed rocprofv3 --pmc summary
+    (FETCH_SIZE + WRITE_SIZE, calibrated on the copy kernel); None when no summary exists."""
+    path = os.path.join(ROOT, "profiles", "%s_hit_gather_hbm_traffic.txt" % workload)
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch="):
+                return int(line.split("=")[1])
+    except OSError:
+        pass
+    return None
+
+
 def log(msg):
     print("[bench] " + msg, file=sys.stderr, flush=True)
 
@@ -238,7 +251,8 @@ def main():
     copy_ms = lmi.bench_copy(1 << 30, 10)
     copy_gbs = 2 * (1 << 30) / (copy_ms * 1e-3) / 1e9
     roofline = dict(bound="hbm", kernel="move_rows_kernel (hit gather)", achieved=round(achieved, 1),
-                    peak=HBM_PEAK_GBS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBS, 4), traffic=None,
+                    peak=HBM_PEAK_GBS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBS, 4),
+                    traffic=recorded_traffic(args.workload) if args.scale == 1.0 else None,
                     rows_per_launch=round(hit_rows, 1), bytes_per_row=hit_bytes, avg_launch_ms=round(hit_ms, 4),
                     measured_copy_gbs=round(copy_gbs, 1))
     host_link = dict(bound="host-link", kernel="move_rows_kernel (miss gather)",
