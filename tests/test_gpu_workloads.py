@@ -1,0 +1,136 @@
+"""BASELINE.json's five configurations as parity cases: the synthetic workload
+builder of bench.py (graph generated on the GPU) at full size where that is
+cheap (cora, products) and at a stated fraction of the node count otherwise,
+compared with the CPU oracle batch by batch."""
+import os
+import sys
+
+import numpy as np
+import pytest
+
+from conftest import ROOT
+
+pytestmark = pytest.mark.gpu
+sys.path.insert(0, ROOT)
+
+
+def build(lmi, name, scale):
+    import bench
+    w = dict(bench.WORKLOADS[name])
+    if scale != 1.0:
+        w["nodes"] = max(1000, int(w["nodes"] * scale))
+        w["train"] = max(4 * w["batch"], int(w["train"] * scale))
+        if w["cache"][0] in ("static", "lru", "int8"):
+            w["cache"] = (w["cache"][0], w["cache"][1] * scale)
+    srv, info = bench.build_workload(lmi, w, 4242, 2, 8.0)
+    indptr = lmi.to_host(info["d_indptr"], info["n_nodes"] + 1, np.int64)
+    indices = lmi.to_host(info["d_indices"], info["n_edges"], np.int32)
+    return srv, info, w, indptr, indices
+
+
+def check_batch(g, o):
+    assert list(g.node_counter) == list(o.node_counter) and list(g.edge_counter) == list(o.edge_counter)
+    for name in ("ids", "agg_src_ids", "agg_src_off", "agg_dst_off"):
+        assert np.array_equal(getattr(g, name), getattr(o, name)), name
+    for a, b in zip(g.blk_indptr, o.blk_indptr):
+        assert np.array_equal(a, b)
+
+
+@pytest.mark.parametrize("name,scale", [("cora", 1.0), ("products", 1.0), ("paper100m", 0.02)])
+def test_static_cache_workloads(lmi, oracle, name, scale):
+    srv, info, w, indptr, indices = build(lmi, name, scale)
+    stream = lmi.stream_create()
+    feats = info["feats"].array
+    try:
+        slot_ref = oracle.static_cache_build(indptr, info["cache_rows"])
+        assert np.array_equal(srv.cache_dump(info["n_nodes"]), slot_ref)
+        B = w["batch"]
+        for it in range(4):
+            srv.run_once(None, batch_counter=it, rng_seed=900 + it, pipe=it % 2, stream=stream)
+            g = srv.fetch(pipe=it % 2, stream=stream)
+            o = oracle.sample_batch(indptr, indices, info["train"][it * B:(it + 1) * B], w["fanout"], 900 + it)
+            check_batch(g, o)
+            assert np.array_equal(g.cache_index, slot_ref[o.ids])
+            assert g.features.tobytes() == feats[o.ids].tobytes()
+            # size-independent properties: COO rows sorted = CSR, degree threshold of the hot set
+            for k in range(g.hops):
+                e0, e1 = g.edge_off[k], g.edge_off[k] + g.n_edges[k]
+                assert np.array_equal(np.bincount(g.agg_dst_off[e0:e1], minlength=g.n_nodes[k]),
+                                      np.diff(g.blk_indptr[k]))
+            deg = np.diff(indptr)[g.ids]
+            hit = g.cache_index >= 0
+            if hit.any() and (~hit).any():
+                assert deg[hit].min() >= deg[~hit].max()
+    finally:
+        srv.close()
+        info["feats"].free()
+
+
+def test_lru_workload_with_temporal_locality(lmi, oracle):
+    """paper100m-shaped graph at 1/100 of the node count, 3 hops [15,10,5], LRU cache; 80 % of the
+    seeds of a batch come from the frontiers of the previous 10 batches."""
+    srv, info, w, indptr, indices = build(lmi, "paper100m-lru", 0.01)
+    stream = lmi.stream_create()
+    feats = info["feats"].array
+    rb = feats.shape[1] * 4
+    host_rows = feats.view(np.uint8).reshape(feats.shape[0], rb)
+    ci = srv.cache_info()
+    lru = oracle.Lru(int(ci.n_sets), int(ci.ways), rb)
+    rng = np.random.default_rng(4)
+    B, recent, hits = 512, [], 0
+    try:
+        for it in range(14):
+            fresh = rng.choice(info["train"], B, replace=False)
+            if recent:
+                pool = np.unique(np.concatenate(recent[-10:]))
+                k = min(int(0.8 * B), len(pool))
+                seeds = np.concatenate([rng.choice(pool, k, replace=False), fresh[:B - k]])
+            else:
+                seeds = fresh
+            seeds = np.array(list(dict.fromkeys(seeds.tolist())), np.int32)
+            srv.run_once(seeds, rng_seed=70 + it, pipe=0, stream=stream)
+            g = srv.fetch(pipe=0, stream=stream)
+            o = oracle.sample_batch(indptr, indices, seeds, w["fanout"], 70 + it)
+            check_batch(g, o)
+            hit, fill, out = lru.access(o.ids, host_rows)
+            assert np.array_equal(g.cache_index, hit)
+            assert g.features.tobytes() == out.tobytes()
+            recent.append(o.ids)
+            hits += int((hit >= 0).sum())
+        keys, use = srv.cache_dump(int(ci.capacity_rows), with_aux=True)
+        okeys, ouse = lru.state()
+        assert np.array_equal(keys, okeys) and np.array_equal(use, ouse)
+        assert hits > 0
+    finally:
+        srv.close()
+        info["feats"].free()
+
+
+def test_int8_workload(lmi, oracle):
+    """MAG240M-shaped: 768-d fp16 rows, int8 cache with per-row scale, fan-out [25,15], at 1/500 of
+    the node count."""
+    srv, info, w, indptr, indices = build(lmi, "mag240m-int8", 0.002)
+    stream = lmi.stream_create()
+    feats = info["feats"].array
+    try:
+        slot_ref = oracle.static_cache_build(indptr, info["cache_rows"])
+        q, sc = oracle.quantize_rows(feats[np.flatnonzero(slot_ref >= 0)])
+        B = w["batch"]
+        for it in range(3):
+            srv.run_once(None, batch_counter=it, rng_seed=30 + it, pipe=it % 2, stream=stream)
+            g = srv.fetch(pipe=it % 2, stream=stream)
+            o = oracle.sample_batch(indptr, indices, info["train"][it * B:(it + 1) * B], w["fanout"], 30 + it)
+            check_batch(g, o)
+            assert np.array_equal(g.cache_index, slot_ref[o.ids])
+            ref = oracle.gather_rows_int8(o.ids, slot_ref[o.ids], q, sc, feats)
+            assert g.features.tobytes() == ref.tobytes()     # 0 ulp (north star allows 1)
+            hit = g.cache_index >= 0
+            assert hit.any() and (~hit).any()
+            # the codec is lossy but bounded: |y - x| <= scale / 2 (+ fp16 rounding of y)
+            x = feats[o.ids][hit].astype(np.float32)
+            y = g.features[hit].astype(np.float32)
+            bound = sc[slot_ref[o.ids][hit]][:, None] * 0.5 + np.abs(y) * 2.0 ** -10 + 1e-7
+            assert (np.abs(y - x) <= bound).all()
+    finally:
+        srv.close()
+        info["feats"].free()
