@@ -644,6 +644,7 @@ int lmi_tune(lmi_server *h, const char *key, int64_t value) {
   if (!s || !key) LMI_FAIL(LMI_ERR_ARG, "null argument");
   if (!strcmp(key, "gather_lanes_per_row")) s->gather_lpr = (int)value;
   else if (!strcmp(key, "gather_unroll")) s->gather_unroll = (int)value;
+  else if (!strcmp(key, "gather_vector_bytes")) s->gather_vec = (int)value;
   else if (!strcmp(key, "gather_blocks")) s->gather_blocks = (int)value;
   else if (!strcmp(key, "gather_nontemporal")) s->gather_nt = (int)value;
   else if (!strcmp(key, "lds_dedup")) s->lds_dedup = (int)value;

@@ -27,7 +27,9 @@ namespace lmi {
 // otherwise it is src_index[i] (or i).  The destination row is dst_index[i] (or
 // i); a negative source or destination skips the row.  LPR lanes cooperate on a
 // row, each moving sizeof(V) bytes per step, with U rows in flight per lane.
-template <typename V, int LPR, int U, bool NT>
+// HOSTLINK only names the instantiation that reads over the host link, so that
+// profiles list the HBM gather and the host-link gather as two kernels.
+template <typename V, int LPR, int U, bool NT, bool HOSTLINK>
 static __global__ __launch_bounds__(256) void move_rows_kernel(
     const int2 *list, const int32_t *first_ptr, const int32_t *n_ptr, const int32_t *src_index,
     const int32_t *dst_index, int src_from_list, const uint8_t *src, uint8_t *dst, int chunks,
@@ -84,6 +86,7 @@ struct MoveArgs {
   int src_from_list;
   int max_blocks;  // 0 = fill the device
   int unroll;      // 0 = the server's gather_unroll
+  int host_link;   // the source is pinned host memory read over the host link
   const uint8_t *src;
   uint8_t *dst;
   int64_t src_row_bytes, dst_row_bytes, row_bytes;  // row_bytes = bytes moved per row
@@ -93,12 +96,18 @@ struct MoveArgs {
 template <typename V, int LPR, int U>
 static void launch_move_vlu(hipStream_t st, const MoveArgs &a, int grid, bool nt) {
   const int chunks = (int)(a.row_bytes / sizeof(V));
-  if (nt)
-    hipLaunchKernelGGL((move_rows_kernel<V, LPR, U, true>), dim3(grid), dim3(256), 0, st, a.list, a.first_ptr, a.n_ptr,
-                       a.src_index, a.dst_index, a.src_from_list, a.src, a.dst, chunks, a.src_row_bytes, a.dst_row_bytes);
+  if (a.host_link)
+    hipLaunchKernelGGL((move_rows_kernel<V, LPR, U, true, true>), dim3(grid), dim3(256), 0, st, a.list, a.first_ptr,
+                       a.n_ptr, a.src_index, a.dst_index, a.src_from_list, a.src, a.dst, chunks, a.src_row_bytes,
+                       a.dst_row_bytes);
+  else if (nt)
+    hipLaunchKernelGGL((move_rows_kernel<V, LPR, U, true, false>), dim3(grid), dim3(256), 0, st, a.list, a.first_ptr,
+                       a.n_ptr, a.src_index, a.dst_index, a.src_from_list, a.src, a.dst, chunks, a.src_row_bytes,
+                       a.dst_row_bytes);
   else
-    hipLaunchKernelGGL((move_rows_kernel<V, LPR, U, false>), dim3(grid), dim3(256), 0, st, a.list, a.first_ptr, a.n_ptr,
-                       a.src_index, a.dst_index, a.src_from_list, a.src, a.dst, chunks, a.src_row_bytes, a.dst_row_bytes);
+    hipLaunchKernelGGL((move_rows_kernel<V, LPR, U, false, false>), dim3(grid), dim3(256), 0, st, a.list, a.first_ptr,
+                       a.n_ptr, a.src_index, a.dst_index, a.src_from_list, a.src, a.dst, chunks, a.src_row_bytes,
+                       a.dst_row_bytes);
 }
 
 template <typename V, int LPR>
@@ -114,6 +123,8 @@ static void launch_move_vl(hipStream_t st, const MoveArgs &a, int grid, bool nt,
 template <typename V>
 static void launch_move_v(hipStream_t st, const MoveArgs &a, int grid, bool nt, int unroll, int lpr) {
   switch (lpr) {
+    case 1: launch_move_vl<V, 1>(st, a, grid, nt, unroll); break;  // thread per row (measurement only)
+    case 4: launch_move_vl<V, 4>(st, a, grid, nt, unroll); break;
     case 8: launch_move_vl<V, 8>(st, a, grid, nt, unroll); break;
     case 16: launch_move_vl<V, 16>(st, a, grid, nt, unroll); break;
     case 32: launch_move_vl<V, 32>(st, a, grid, nt, unroll); break;
@@ -129,9 +140,10 @@ static int launch_move_rows(Server *s, hipStream_t st, const MoveArgs &a, bool n
                           (uintptr_t)a.dst_row_bytes | (uintptr_t)a.row_bytes;
   int vec = (align % 16 == 0) ? 16 : (align % 8 == 0) ? 8 : 4;
   if (align % 4 != 0) LMI_FAIL(LMI_ERR_ARG, "feature rows must be 4-byte aligned");
+  if (s->gather_vec == 4 || (s->gather_vec == 8 && vec == 16)) vec = s->gather_vec;  // narrower on request
   const int64_t chunks = a.row_bytes / vec;
   int lpr = s->gather_lpr;
-  if (lpr != 8 && lpr != 16 && lpr != 32 && lpr != 64) {
+  if (lpr != 1 && lpr != 4 && lpr != 8 && lpr != 16 && lpr != 32 && lpr != 64) {
     lpr = 8;
     while (lpr < chunks && lpr < 64) lpr <<= 1;
   }
@@ -438,6 +450,7 @@ int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last)
   if (s->feat_loc == LMI_LOC_HOST) {
     m.max_blocks = s->miss_blocks > 0 ? s->miss_blocks : s->n_cu;
     m.unroll = s->miss_unroll;
+    m.host_link = 1;
   }
   if (split) {
     prof_phase(s, st, -1);

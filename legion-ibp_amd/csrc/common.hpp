@@ -154,10 +154,11 @@ struct Server {
   std::vector<Pipe> pipes;
   // tuning
   int gather_lpr = 0;     // lanes per row (0 = auto)
-  int gather_unroll = 4;
+  int gather_vec = 0;     // bytes per lane access (0 = widest that fits: 16)
+  int gather_unroll = 1;  // rows in flight per lane (1 measured best: 62.5 % of HBM peak vs 60 % at 4)
   int gather_blocks = 0;  // 0 = auto
   int gather_nt = 1;      // non-temporal output stores
-  int lds_dedup = 1;
+  int lds_dedup = 0;      // 1: hop_sample stages its probes through an LDS hash table
   int split_miss = 1;     // 1: host-link gather on the pipe's side stream, after the HBM gather
   int use_graph = 1;      // lmi_run_once replays a captured HIP graph
   int miss_blocks = 32;   // grid of the host-link gather: enough reads in flight to fill the link, few enough

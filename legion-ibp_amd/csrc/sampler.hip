@@ -223,6 +223,85 @@ static __global__ __launch_bounds__(256) void hop_sample_kernel(HopArgs a) {
   }
 }
 
+// Variant with LDS-staged probes: the (up to 256) edges a block draws in one step are
+// first deduplicated in a 512-entry LDS hash table; only the lowest edge of each
+// distinct neighbour probes the HBM table, the other lanes copy its slot.  Same
+// results (the HBM table still sees the minimum edge index per key).
+template <int G>
+static __global__ __launch_bounds__(256) void hop_sample_lds_kernel(HopArgs a) {
+  constexpr int TAB = 512;
+  __shared__ int32_t lds_key[TAB];
+  __shared__ int32_t lds_min[TAB];
+  __shared__ int32_t lds_slot[TAB];
+  const DevState *st = a.st;
+  const int64_t flat = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  scan_chain_reset(a.chain_edges, a.max_tiles, flat, (int64_t)gridDim.x * blockDim.x);
+  const uint64_t seed = (uint64_t)st->rng_lo | ((uint64_t)st->rng_hi << 32);
+  const int n_prev = st->node_counter[9 + a.hop];
+  const int eoff = st->edge_counter[12 + a.hop + 1];
+  const int fanout = a.fanout;
+  const int lane = threadIdx.x & (G - 1);
+  const int group = (int)(flat / G);
+  const int n_groups = gridDim.x * blockDim.x / G;
+  const int groups_per_block = 256 / G;
+  // uniform trip count per block: the block's first group decides
+  for (int i0 = blockIdx.x * groups_per_block; i0 < n_prev; i0 += n_groups) {
+    const int i = i0 + (group - blockIdx.x * groups_per_block);
+    for (int t = threadIdx.x; t < TAB; t += 256) {
+      lds_key[t] = kEmptyKey;
+      lds_min[t] = kIntMax;
+    }
+    __syncthreads();
+    bool active = false;
+    int32_t nbr = -1;
+    int e = 0, h = 0;
+    if (i < n_prev) {
+      const int32_t v = a.ids[i];
+      if (v >= 0 && v < a.n_nodes) {
+        const int64_t beg = a.indptr[v];
+        const int64_t deg = a.indptr[v + 1] - beg;
+        const int base = a.row_ptr[i];
+        int64_t pick = lane;
+        int count;
+        if (deg <= (int64_t)fanout) {
+          count = (int)deg;
+        } else {
+          count = fanout;
+          const uint32_t j = (uint32_t)(deg - fanout) + (uint32_t)lane;
+          uint32_t t = 0xFFFFFFFFu;
+          if (lane < fanout) t = __umulhi(sample_draw(seed, (uint32_t)a.hop, (uint32_t)v, (uint32_t)lane), j + 1u);
+          bool dup = false;
+          for (int q = 0; q + 1 < fanout; ++q) {
+            const uint32_t mine = dup ? j : t;
+            const uint32_t p = __shfl(mine, q, G);
+            if (lane > q && t == p) dup = true;
+          }
+          pick = dup ? j : t;
+        }
+        if (lane < count) {
+          active = true;
+          nbr = a.indices[beg + pick];
+          e = base + lane;
+          a.agg_src_ids[eoff + e] = nbr;
+          a.agg_dst_off[eoff + e] = i;
+          h = (int)(((uint32_t)nbr * 0x9E3779B1u) >> 23);  // 9 bits
+          while (true) {
+            const int32_t k = atomicCAS(&lds_key[h], kEmptyKey, nbr);
+            if (k == kEmptyKey || k == nbr) break;
+            h = (h + 1) & (TAB - 1);
+          }
+          atomicMin(&lds_min[h], e);
+        }
+      }
+    }
+    __syncthreads();
+    if (active && lds_min[h] == e) lds_slot[h] = (int)table_insert_min(a.slots, a.log2cap, nbr, n_prev + e);
+    __syncthreads();
+    if (active) a.eslot[e] = lds_slot[h];
+    __syncthreads();
+  }
+}
+
 // ------------------------------------------------------------- hop, phase 3
 // firstv[e] = table value of the edge's source; an edge is the first occurrence
 // of a new node iff that value names the edge itself.  rank[e] = number of first
@@ -378,6 +457,15 @@ int launch_hop(Server *s, Pipe &p, hipStream_t st, int hop, bool stage_seeds) {
   int G = 4;
   while (G < f) G <<= 1;
   const int grid = (int)std::min<int64_t>(ceil_div(n_max * G, 256), 8192);
+  if (s->lds_dedup) {
+    switch (G) {
+      case 4: hipLaunchKernelGGL(hop_sample_lds_kernel<4>, dim3(grid), dim3(256), 0, st, a); break;
+      case 8: hipLaunchKernelGGL(hop_sample_lds_kernel<8>, dim3(grid), dim3(256), 0, st, a); break;
+      case 16: hipLaunchKernelGGL(hop_sample_lds_kernel<16>, dim3(grid), dim3(256), 0, st, a); break;
+      case 32: hipLaunchKernelGGL(hop_sample_lds_kernel<32>, dim3(grid), dim3(256), 0, st, a); break;
+      default: hipLaunchKernelGGL(hop_sample_lds_kernel<64>, dim3(grid), dim3(256), 0, st, a); break;
+    }
+  } else
   switch (G) {
     case 4: hipLaunchKernelGGL(hop_sample_kernel<4>, dim3(grid), dim3(256), 0, st, a); break;
     case 8: hipLaunchKernelGGL(hop_sample_kernel<8>, dim3(grid), dim3(256), 0, st, a); break;

@@ -58,6 +58,30 @@ def test_sample_batch_parity(lmi, oracle, fanout, n_nodes, mean_deg, batch):
         feats.free()
 
 
+@pytest.mark.parametrize("fanout", [[25, 10], [64, 3], [5, 4, 3]])
+def test_lds_staged_dedup_gives_the_same_batches(lmi, oracle, fanout):
+    rng = np.random.default_rng(sum(fanout))
+    n_nodes, batch = 2500, 120
+    indptr, indices = random_graph(rng, n_nodes, 25, hubs=8, hub_deg=900)   # hubs: many duplicate neighbours per tile
+    hot = rng.random(len(indices)) < 0.3
+    indices[hot] = rng.integers(0, 20, int(hot.sum()))    # 30 % of all edges point at 20 hot nodes
+    feats = make_features(lmi, rng, n_nodes, 8)
+    srv = lmi.Server(batch, fanout, 8)
+    stream = lmi.stream_create()
+    try:
+        srv.tune("lds_dedup", 1)
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        for it in range(4):
+            seeds = rng.choice(n_nodes, batch, replace=False).astype(np.int32)
+            st = stream if it % 2 else None          # graph replay and eager
+            srv.run_once(seeds, rng_seed=40 + it, stream=st)
+            assert_batch_equal(srv.fetch(stream=st), oracle.sample_batch(indptr, indices, seeds, fanout, 40 + it))
+    finally:
+        srv.close()
+        feats.free()
+
+
 def test_duplicate_seeds_and_isolated_nodes(lmi, oracle):
     rng = np.random.default_rng(5)
     indptr, indices = random_graph(rng, 300, 6, zero_frac=0.4)
