@@ -80,7 +80,9 @@ def build_workload(lmi, w, seed, pipes, host_budget_gb, table=2):
         # the feature table must fit in pinned host memory on this box
         scale = host_budget_gb / feat_gb
         n_nodes = int(n_nodes * scale)
-        note = "node count down-scaled x%.3f so the %.0f GB feature table fits pinned host memory" % (scale, feat_gb)
+        if w["cache"][0] in ("static", "lru", "int8"):
+            w = dict(w, cache=(w["cache"][0], w["cache"][1] * scale))   # keep the cached fraction
+        note = "node count and cache budget down-scaled x%.3f so the %.0f GB feature table fits pinned host memory" % (scale, feat_gb)
         log(note)
     t0 = time.time()
     if w["alpha"] is None:   # Erdos-Renyi-like: Poisson degrees, uniform neighbours
@@ -192,7 +194,7 @@ def main():
     ap.add_argument("--pipes", type=int, default=2)
     ap.add_argument("--seed", type=int, default=20260101)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget (0 = skip)")
-    ap.add_argument("--host-gb", type=float, default=200.0, help="pinned host memory budget for the feature table")
+    ap.add_argument("--host-gb", type=float, default=64.0, help="pinned host memory budget for the feature table")
     ap.add_argument("--table", default="rank", choices=["hash", "direct", "rank"], help="id->slot table layout")
     ap.add_argument("--tune", action="append", default=[], help="key=value passed to lmi_tune")
     args = ap.parse_args()
@@ -250,12 +252,12 @@ def main():
     achieved = hit_rows * hit_bytes / (hit_ms * 1e-3) / 1e9 if hit_ms > 0 else 0.0
     copy_ms = lmi.bench_copy(1 << 30, 10)
     copy_gbs = 2 * (1 << 30) / (copy_ms * 1e-3) / 1e9
-    roofline = dict(bound="hbm", kernel="move_rows_kernel (hit gather)", achieved=round(achieved, 1),
+    roofline = dict(bound="hbm", kernel="move_rows_kernel<u32x4,32,1,true,false> (HBM gather of cache hits)", achieved=round(achieved, 1),
                     peak=HBM_PEAK_GBS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBS, 4),
                     traffic=recorded_traffic(args.workload) if args.scale == 1.0 else None,
                     rows_per_launch=round(hit_rows, 1), bytes_per_row=hit_bytes, avg_launch_ms=round(hit_ms, 4),
                     measured_copy_gbs=round(copy_gbs, 1))
-    host_link = dict(bound="host-link", kernel="move_rows_kernel (miss gather)",
+    host_link = dict(bound="host-link", kernel="move_rows_kernel<u32x4,32,1,true,true> (host-link gather of misses)",
                      achieved=round(miss_rows * rb / (miss_ms * 1e-3) / 1e9, 2) if miss_ms > 0 else 0.0,
                      peak=HOST_LINK_PEAK_GBS, unit="GB/s", rows_per_launch=round(miss_rows, 1),
                      avg_launch_ms=round(miss_ms, 4))
