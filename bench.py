@@ -191,7 +191,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="paper100m", choices=sorted(WORKLOADS))
     ap.add_argument("--scale", type=float, default=1.0, help="shrink node/train counts (testing only)")
-    ap.add_argument("--pipes", type=int, default=2)
+    ap.add_argument("--pipes", type=int, default=2, help="output buffer sets in flight")
+    ap.add_argument("--streams", type=int, default=1, help="caller streams the pipes are spread over")
     ap.add_argument("--seed", type=int, default=20260101)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget (0 = skip)")
     ap.add_argument("--host-gb", type=float, default=64.0, help="pinned host memory budget for the feature table")
@@ -217,13 +218,15 @@ def main():
         k, v = kv.split("=")
         srv.tune(k, int(v))
     steps_per_epoch = -(-info["n_train"] // w["batch"])
-    stream = lmi.stream_create()
+    streams = [lmi.stream_create() for _ in range(max(1, args.streams))]
 
     def step(i):
-        # one caller stream; consecutive batches alternate output buffer sets (pipes), so the
-        # host-link part of batch i (on the server's side stream) overlaps the sampling of batch i+1
-        srv.run_once(None, batch_counter=i % steps_per_epoch, rng_seed=args.seed + i, pipe=i % args.pipes,
-                     stream=stream)
+        # consecutive batches alternate output buffer sets (pipes), so the host-link part of batch i
+        # (on the server's side stream) overlaps the sampling of batch i+1; a pipe always uses the
+        # same caller stream
+        p = i % args.pipes
+        srv.run_once(None, batch_counter=i % steps_per_epoch, rng_seed=args.seed + i, pipe=p,
+                     stream=streams[p % len(streams)])
 
     for i in range(args.warmup):
         step(i)
@@ -271,17 +274,15 @@ def main():
         "config": {"workload": args.workload, "nodes": info["n_nodes"], "edges": info["n_edges"],
                    "feat_dim": w["dim"], "batch": w["batch"], "fanout": w["fanout"],
                    "cache": "%s, %d rows, %s id->slot table" % (info["cache_kind"], info["cache_rows"], args.table),
-                   "pipes": args.pipes,
+                   "pipes": args.pipes, "streams": args.streams,
                    "graph": "Zipf-Mandelbrot degrees alpha=%s, degree-proportional neighbours" % w["alpha"],
                    "note": info["note"]},
         "feature_gather_gbs": round(achieved, 1),
         "feature_gather_frac_hbm_peak": round(achieved / HBM_PEAK_GBS, 4),
         "cache_hit_rate": round(prof.gather_hit_rows / total_rows, 4) if total_rows else None,
         "rows_per_batch": round(total_rows / max(args.steps, 1), 1),
-        "kernel_ms_per_batch": {"sample": round(prof.sample_ms / max(prof.sample_launches, 1), 4),
-                                "lookup": round(prof.lookup_ms / max(prof.lookup_launches, 1), 4),
-                                "gather_hit": round(hit_ms, 4), "gather_miss": round(miss_ms, 4),
-                                "batch": round(prof.batch_ms / max(prof.batches, 1), 4)},
+        "phase_ms_per_batch": {"sample_dedup_lookup": round(prof.sample_ms / max(prof.sample_launches, 1), 4),
+                               "gather_hit": round(hit_ms, 4), "gather_miss_side_stream": round(miss_ms, 4)},
         "roofline": roofline, "host_link": host_link,
     }
     if args.cpu_seconds > 0:

@@ -19,8 +19,6 @@ void set_error(const char *fmt, ...) {
 }
 
 // ------------------------------------------------------------ profiling
-constexpr int kProfRing = 8192;
-
 static hipEvent_t prof_event(Server *s) {
   if (!s->prof_free.empty()) {
     hipEvent_t e = s->prof_free.back();
@@ -48,26 +46,21 @@ int prof_end(Server *s, hipStream_t st, int handle) {
   return LMI_OK;
 }
 
-void prof_phase(Server *s, hipStream_t st, int next_kind) {
+void prof_phase(Server *s, hipStream_t st, int *open, int next_kind) {
   if (!s->prof_on) {
-    s->prof_open = -1;
+    *open = -1;
     return;
   }
-  if (s->prof_open < 0 && next_kind < 0) return;
+  if (*open < 0 && next_kind < 0) return;
   hipEvent_t e = prof_event(s);
   s->prof_used.push_back(e);
   (void)hipEventRecord(e, st);
-  if (s->prof_open >= 0) s->prof_events[s->prof_open].b = e;
-  s->prof_open = -1;
+  if (*open >= 0) s->prof_events[*open].b = e;
+  *open = -1;
   if (next_kind >= 0) {
     s->prof_events.push_back(EventPair{e, nullptr, next_kind});
-    s->prof_open = (int)s->prof_events.size() - 1;
+    *open = (int)s->prof_events.size() - 1;
   }
-}
-
-static void prof_snapshot(Server *s, Pipe &p, hipStream_t st) {
-  if (!s->prof_on || s->prof_ring_n >= kProfRing) return;
-  (void)hipMemcpyAsync(&s->prof_ring[s->prof_ring_n++], p.st, sizeof(DevState), hipMemcpyDeviceToHost, st);
 }
 
 static int check_pipe(Server *s, int pipe) {
@@ -91,7 +84,6 @@ static void pipe_free(Pipe &p) {
     if (q) (void)hipFree(q);
   if (p.graph_exec) (void)hipGraphExecDestroy(p.graph_exec);
   if (p.graph) (void)hipGraphDestroy(p.graph);
-  if (p.side) (void)hipStreamDestroy(p.side);
   if (p.fork) (void)hipEventDestroy(p.fork);
   if (p.join) (void)hipEventDestroy(p.join);
   p = Pipe{};
@@ -126,7 +118,6 @@ static int pipe_alloc(Server *s, Pipe &p) {
   LMI_TRY(dmalloc(&p.miss_list, s->max_nodes));
   LMI_TRY(dmalloc(&p.lru_fill, s->max_nodes));
   LMI_TRY(dmalloc(&p.seed_stage, s->cfg.batch_size));
-  LMI_HIP(hipStreamCreateWithFlags(&p.side, hipStreamNonBlocking));
   LMI_HIP(hipEventCreateWithFlags(&p.fork, hipEventDisableTiming));
   LMI_HIP(hipEventCreateWithFlags(&p.join, hipEventDisableTiming));
   return LMI_OK;
@@ -201,7 +192,8 @@ int lmi_server_create(const lmi_config *cfg, lmi_server **out) {
   for (auto &p : s->pipes)
     if ((rc = pipe_alloc(s, p)) != LMI_OK) break;
   if (rc == LMI_OK && hipMalloc(&s->d_scalar, 64) != hipSuccess) rc = LMI_ERR_HIP;
-  if (rc == LMI_OK && hipHostMalloc((void **)&s->prof_ring, sizeof(DevState) * kProfRing, hipHostMallocDefault) != hipSuccess)
+  if (rc == LMI_OK && hipStreamCreateWithFlags(&s->side, hipStreamNonBlocking) != hipSuccess) rc = LMI_ERR_HIP;
+  if (rc == LMI_OK && (hipMalloc(&s->d_prof_rows, 16) != hipSuccess || hipMemset(s->d_prof_rows, 0, 16) != hipSuccess))
     rc = LMI_ERR_HIP;
   if (rc != LMI_OK) {
     lmi_server_destroy(reinterpret_cast<lmi_server *>(s));
@@ -228,8 +220,9 @@ int lmi_server_destroy(lmi_server *h) {
   }
   for (auto &e : s->prof_used) (void)hipEventDestroy(e);
   for (auto &e : s->prof_free) (void)hipEventDestroy(e);
-  if (s->prof_ring) (void)hipHostFree(s->prof_ring);
+  if (s->d_prof_rows) (void)hipFree(s->d_prof_rows);
   if (s->d_scalar) (void)hipFree(s->d_scalar);
+  if (s->side) (void)hipStreamDestroy(s->side);
   delete s;
   return LMI_OK;
 }
@@ -451,9 +444,9 @@ int lmi_op_random_sample(lmi_server *h, int pipe, void *stream, int hop) {
   Pipe &p = s->pipes[pipe];
   if (hop != p.hops_done || hop >= s->cfg.hops) LMI_FAIL(LMI_ERR_ARG, "hop %d out of order (next is %d)", hop, p.hops_done);
   hipStream_t st = (hipStream_t)stream;
-  prof_phase(s, st, PROF_SAMPLE);
+  prof_phase(s, st, &s->prof_open, PROF_SAMPLE);
   LMI_TRY(launch_hop(s, p, st, hop, false));
-  prof_phase(s, st, -1);
+  prof_phase(s, st, &s->prof_open, -1);
   return LMI_OK;
 }
 
@@ -465,10 +458,10 @@ int lmi_op_cache_lookup(lmi_server *h, int pipe, void *stream, int segment) {
   if (segment < 0 || segment > p.hops_done) LMI_FAIL(LMI_ERR_ARG, "segment %d not sampled yet", segment);
   hipStream_t st = (hipStream_t)stream;
   LMI_TRY(pipe_join(p, st));
-  prof_phase(s, st, PROF_LOOKUP);
+  prof_phase(s, st, &s->prof_open, PROF_LOOKUP);
   LMI_TRY(launch_lookup(s, p, st, segment, segment));
   LMI_TRY(launch_gather_seg(s, p, st, segment, segment));
-  prof_phase(s, st, -1);
+  prof_phase(s, st, &s->prof_open, -1);
   return LMI_OK;
 }
 
@@ -484,7 +477,6 @@ int lmi_op_io_complete(lmi_server *h, int pipe, void *stream) {
   hipStream_t st = (hipStream_t)stream;
   LMI_TRY(pipe_join(p, st));
   LMI_TRY(launch_lru_insert(s, p, st, s->cfg.hops + 1));
-  prof_snapshot(s, p, st);
   return LMI_OK;
 }
 
@@ -531,7 +523,7 @@ int lmi_run_once(lmi_server *h, int pipe, void *stream, const int32_t *seeds, in
   BatchParams bp{};
   LMI_TRY(batch_params(s, p, st, seeds, n, seeds_location, batch_counter, mode, rng_seed, &bp));
   LMI_TRY(pipe_join(p, st));  // the previous batch of this pipe may still be gathering misses
-  prof_phase(s, st, PROF_SAMPLE);
+  prof_phase(s, st, &s->prof_open, PROF_SAMPLE);
   if (s->use_graph && st != nullptr) {  // the legacy default stream cannot be captured
     if (!p.graph_exec) LMI_TRY(capture_batch_graph(s, p, st, bp));
     LMI_TRY(graph_update_begin(s, p, bp));
@@ -543,8 +535,7 @@ int lmi_run_once(lmi_server *h, int pipe, void *stream, const int32_t *seeds, in
   }
   LMI_TRY(launch_gather_seg(s, p, st, 0, s->cfg.hops));
   LMI_TRY(launch_lru_insert(s, p, st, 1));
-  prof_phase(s, st, -1);
-  prof_snapshot(s, p, st);
+  prof_phase(s, st, &s->prof_open, -1);
   return LMI_OK;
 }
 
@@ -624,16 +615,13 @@ int lmi_profile_read(lmi_server *h, lmi_profile *out, int reset) {
   }
   for (auto &ev : s->prof_used) s->prof_free.push_back(ev);
   s->prof_used.clear();
-  s->prof_open = -1;
+  s->prof_open = s->prof_open_side = -1;
   s->prof_events.clear();
-  for (int i = 0; i < s->prof_ring_n; ++i) {
-    const DevState &d = s->prof_ring[i];
-    int64_t miss = 0;
-    for (int k = 0; k <= LMI_MAX_HOPS; ++k) miss += d.n_miss[k];
-    s->prof.gather_miss_rows += miss;
-    s->prof.gather_hit_rows += (int64_t)d.node_counter[7] - miss;
-  }
-  s->prof_ring_n = 0;
+  unsigned long long rows[2] = {0, 0};
+  LMI_HIP(hipMemcpy(rows, s->d_prof_rows, 16, hipMemcpyDeviceToHost));
+  LMI_HIP(hipMemset(s->d_prof_rows, 0, 16));
+  s->prof.gather_miss_rows += (int64_t)rows[1];
+  if (rows[0] > rows[1]) s->prof.gather_hit_rows += (int64_t)(rows[0] - rows[1]);
   *out = s->prof;
   if (reset) s->prof = lmi_profile{};
   return LMI_OK;

@@ -33,9 +33,11 @@ template <typename V, int LPR, int U, bool NT, bool HOSTLINK>
 static __global__ __launch_bounds__(256) void move_rows_kernel(
     const int2 *list, const int32_t *first_ptr, const int32_t *n_ptr, const int32_t *src_index,
     const int32_t *dst_index, int src_from_list, const uint8_t *src, uint8_t *dst, int chunks,
-    int64_t src_row_bytes, int64_t dst_row_bytes) {
+    int64_t src_row_bytes, int64_t dst_row_bytes, unsigned long long *row_counter) {
   const int n = *n_ptr;
   const int first = first_ptr ? *first_ptr : 0;
+  if (row_counter && blockIdx.x == 0 && threadIdx.x == 0 && n > first)
+    atomicAdd(row_counter, (unsigned long long)(n - first));  // work items offered to this launch (profiling)
   const int lane = threadIdx.x & (LPR - 1);
   const int group = (blockIdx.x * blockDim.x + threadIdx.x) / LPR;
   const int n_groups = gridDim.x * blockDim.x / LPR;
@@ -87,6 +89,7 @@ struct MoveArgs {
   int max_blocks;  // 0 = fill the device
   int unroll;      // 0 = the server's gather_unroll
   int host_link;   // the source is pinned host memory read over the host link
+  unsigned long long *row_counter;  // device counter that receives the number of work items, or null
   const uint8_t *src;
   uint8_t *dst;
   int64_t src_row_bytes, dst_row_bytes, row_bytes;  // row_bytes = bytes moved per row
@@ -99,15 +102,15 @@ static void launch_move_vlu(hipStream_t st, const MoveArgs &a, int grid, bool nt
   if (a.host_link)
     hipLaunchKernelGGL((move_rows_kernel<V, LPR, U, true, true>), dim3(grid), dim3(256), 0, st, a.list, a.first_ptr,
                        a.n_ptr, a.src_index, a.dst_index, a.src_from_list, a.src, a.dst, chunks, a.src_row_bytes,
-                       a.dst_row_bytes);
+                       a.dst_row_bytes, a.row_counter);
   else if (nt)
     hipLaunchKernelGGL((move_rows_kernel<V, LPR, U, true, false>), dim3(grid), dim3(256), 0, st, a.list, a.first_ptr,
                        a.n_ptr, a.src_index, a.dst_index, a.src_from_list, a.src, a.dst, chunks, a.src_row_bytes,
-                       a.dst_row_bytes);
+                       a.dst_row_bytes, a.row_counter);
   else
     hipLaunchKernelGGL((move_rows_kernel<V, LPR, U, false, false>), dim3(grid), dim3(256), 0, st, a.list, a.first_ptr,
                        a.n_ptr, a.src_index, a.dst_index, a.src_from_list, a.src, a.dst, chunks, a.src_row_bytes,
-                       a.dst_row_bytes);
+                       a.dst_row_bytes, a.row_counter);
 }
 
 template <typename V, int LPR>
@@ -195,9 +198,11 @@ static __global__ __launch_bounds__(256) void quantize_rows_kernel(
 template <typename OUT, int LPR>
 static __global__ __launch_bounds__(256) void gather_int8_kernel(
     const int32_t *first_ptr, const int32_t *n_ptr, const int32_t *cache_index, const int8_t *q,
-    const float *scale, OUT *out, int dim) {
+    const float *scale, OUT *out, int dim, unsigned long long *row_counter) {
   const int n = *n_ptr;
   const int first = first_ptr ? *first_ptr : 0;
+  if (row_counter && blockIdx.x == 0 && threadIdx.x == 0 && n > first)
+    atomicAdd(row_counter, (unsigned long long)(n - first));
   const int lane = threadIdx.x & (LPR - 1);
   const int group = (blockIdx.x * blockDim.x + threadIdx.x) / LPR;
   const int n_groups = gridDim.x * blockDim.x / LPR;
@@ -232,9 +237,11 @@ static __global__ __launch_bounds__(256) void gather_int8_kernel(
 template <typename OUT>
 static __global__ __launch_bounds__(256) void gather_int8_generic_kernel(
     const int32_t *first_ptr, const int32_t *n_ptr, const int32_t *cache_index, const int8_t *q,
-    const float *scale, OUT *out, int dim) {
+    const float *scale, OUT *out, int dim, unsigned long long *row_counter) {
   const int n = *n_ptr;
   const int first = first_ptr ? *first_ptr : 0;
+  if (row_counter && blockIdx.x == 0 && threadIdx.x == 0 && n > first)
+    atomicAdd(row_counter, (unsigned long long)(n - first));
   const int lane = threadIdx.x & (kWave - 1);
   const int wave = (blockIdx.x * blockDim.x + threadIdx.x) / kWave;
   const int n_waves = gridDim.x * blockDim.x / kWave;
@@ -379,94 +386,119 @@ int pipe_join(Pipe &p, hipStream_t st) {
   return LMI_OK;
 }
 
-// Gathers the rows [first, last) of a segment into the pipe's feature buffer.
-// Cache hits stream from HBM on `st`.  Misses come over the host link; with
-// split_miss they run on the pipe's side stream AFTER the HBM gather (host-link
-// reads in flight beside it cut its bandwidth by more than half) and the caller's
-// stream does not wait for them here: the next call on this pipe, or
-// lmi_batch_wait, joins.  The LRU cache joins at once (its insert copies the rows).
-int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last) {
-  const int64_t base = seg_list_base(s, seg);
+// HBM gather of the cache hits of rows [first, last) on stream `st`.
+static int launch_hits(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last) {
   const int64_t n_max = s->node_cap[seg_last];
-  const bool split = s->split_miss && s->feat_loc == LMI_LOC_HOST && s->cache_kind != LMI_CACHE_NONE;
-  hipStream_t ms = split ? p.side : st;
-  if (s->cache_kind != LMI_CACHE_NONE) {
-    prof_phase(s, st, PROF_GATHER_HIT);
-    if (s->cache_kind == LMI_CACHE_INT8) {
-      const int dim = s->cfg.feat_dim;
-      const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(n_max, 4), (int64_t)s->n_cu * 8));
-      const int32_t *first_ptr = seg == 0 ? nullptr : &p.st->node_counter[9 + seg - 1];
-      const int32_t *n_ptr = &p.st->node_counter[9 + seg_last];
-      const int8_t *q = (const int8_t *)s->cache_data;
-      if (dim % 16 == 0) {
-        const int chunks = dim / 16;
-        if (s->cfg.feat_dtype == LMI_F16) {
-          if (chunks <= 32)
-            hipLaunchKernelGGL((gather_int8_kernel<__half, 32>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
-                               p.cache_index, q, s->cache_scale, (__half *)p.features, dim);
-          else
-            hipLaunchKernelGGL((gather_int8_kernel<__half, 64>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
-                               p.cache_index, q, s->cache_scale, (__half *)p.features, dim);
-        } else {
-          if (chunks <= 32)
-            hipLaunchKernelGGL((gather_int8_kernel<float, 32>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
-                               p.cache_index, q, s->cache_scale, (float *)p.features, dim);
-          else
-            hipLaunchKernelGGL((gather_int8_kernel<float, 64>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
-                               p.cache_index, q, s->cache_scale, (float *)p.features, dim);
-        }
-      } else {
-        if (s->cfg.feat_dtype == LMI_F16)
-          hipLaunchKernelGGL((gather_int8_generic_kernel<__half>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
-                             p.cache_index, q, s->cache_scale, (__half *)p.features, dim);
+  if (s->cache_kind == LMI_CACHE_INT8) {
+    const int dim = s->cfg.feat_dim;
+    const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(n_max, 4), (int64_t)s->n_cu * 8));
+    const int32_t *first_ptr = seg == 0 ? nullptr : &p.st->node_counter[9 + seg - 1];
+    const int32_t *n_ptr = &p.st->node_counter[9 + seg_last];
+    const int8_t *q = (const int8_t *)s->cache_data;
+    unsigned long long *rc = s->prof_on ? s->d_prof_rows : nullptr;
+    if (dim % 16 == 0) {
+      const int chunks = dim / 16;
+      if (s->cfg.feat_dtype == LMI_F16) {
+        if (chunks <= 32)
+          hipLaunchKernelGGL((gather_int8_kernel<__half, 32>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
+                             p.cache_index, q, s->cache_scale, (__half *)p.features, dim, rc);
         else
-          hipLaunchKernelGGL((gather_int8_generic_kernel<float>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
-                             p.cache_index, q, s->cache_scale, (float *)p.features, dim);
+          hipLaunchKernelGGL((gather_int8_kernel<__half, 64>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
+                             p.cache_index, q, s->cache_scale, (__half *)p.features, dim, rc);
+      } else {
+        if (chunks <= 32)
+          hipLaunchKernelGGL((gather_int8_kernel<float, 32>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
+                             p.cache_index, q, s->cache_scale, (float *)p.features, dim, rc);
+        else
+          hipLaunchKernelGGL((gather_int8_kernel<float, 64>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
+                             p.cache_index, q, s->cache_scale, (float *)p.features, dim, rc);
       }
-      LMI_HIP(hipGetLastError());
     } else {
-      MoveArgs m{};
-      m.list = nullptr;  // rows [first, n) directly; cache_index < 0 (a miss) skips the row
-      m.first_ptr = seg == 0 ? nullptr : &p.st->node_counter[9 + seg - 1];
-      m.n_ptr = &p.st->node_counter[9 + seg_last];
-      m.src_index = p.cache_index;
-      m.src = s->cache_data;
-      m.dst = (uint8_t *)p.features;
-      m.src_row_bytes = m.dst_row_bytes = m.row_bytes = s->row_bytes;
-      m.n_max = n_max;
-      LMI_TRY(launch_move_rows(s, st, m, s->gather_nt != 0));
+      if (s->cfg.feat_dtype == LMI_F16)
+        hipLaunchKernelGGL((gather_int8_generic_kernel<__half>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
+                           p.cache_index, q, s->cache_scale, (__half *)p.features, dim, rc);
+      else
+        hipLaunchKernelGGL((gather_int8_generic_kernel<float>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
+                           p.cache_index, q, s->cache_scale, (float *)p.features, dim, rc);
     }
+    LMI_HIP(hipGetLastError());
+    return LMI_OK;
   }
-  // misses: raw rows from the feature table, on a small grid (the host link needs
-  // few bytes in flight)
   MoveArgs m{};
-  m.list = p.miss_list + base;
+  m.list = nullptr;  // rows [first, n) directly; cache_index < 0 (a miss) skips the row
+  m.first_ptr = seg == 0 ? nullptr : &p.st->node_counter[9 + seg - 1];
+  m.n_ptr = &p.st->node_counter[9 + seg_last];
+  m.src_index = p.cache_index;
+  m.src = s->cache_data;
+  m.dst = (uint8_t *)p.features;
+  m.src_row_bytes = m.dst_row_bytes = m.row_bytes = s->row_bytes;
+  m.n_max = n_max;
+  m.row_counter = s->prof_on ? s->d_prof_rows : nullptr;  // all rows of the segment: hits + misses
+  return launch_move_rows(s, st, m, s->gather_nt != 0);
+}
+
+// Gather of the rows on the segment's miss list from the feature table, on a
+// small grid when the table sits behind the host link (few bytes in flight fill it).
+static int launch_misses(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last) {
+  MoveArgs m{};
+  m.list = p.miss_list + seg_list_base(s, seg);
   m.n_ptr = &p.st->n_miss[seg];
   m.src_from_list = 1;
   m.src = s->feat;
   m.dst = (uint8_t *)p.features;
   m.src_row_bytes = m.dst_row_bytes = m.row_bytes = s->row_bytes;
-  m.n_max = n_max;
+  m.n_max = s->node_cap[seg_last];
   if (s->feat_loc == LMI_LOC_HOST) {
     m.max_blocks = s->miss_blocks > 0 ? s->miss_blocks : s->n_cu;
     m.unroll = s->miss_unroll;
     m.host_link = 1;
   }
-  if (split) {
-    prof_phase(s, st, -1);
-    LMI_HIP(hipEventRecord(p.fork, st));
-    LMI_HIP(hipStreamWaitEvent(p.side, p.fork, 0));
-    int h = prof_begin(s, ms, PROF_GATHER_MISS);
-    LMI_TRY(launch_move_rows(s, ms, m, s->gather_nt != 0));
-    prof_end(s, ms, h);
-    LMI_HIP(hipEventRecord(p.join, p.side));
-    p.side_pending = true;
-    if (s->cache_kind == LMI_CACHE_LRU) LMI_TRY(pipe_join(p, st));
-  } else {
-    prof_phase(s, st, PROF_GATHER_MISS);
-    LMI_TRY(launch_move_rows(s, ms, m, s->gather_nt != 0));
-    prof_phase(s, st, -1);
+  m.row_counter = s->prof_on ? s->d_prof_rows + 1 : nullptr;  // misses
+  return launch_move_rows(s, st, m, s->gather_nt != 0);
+}
+
+// Gathers the rows [first, last) of a segment into the pipe's feature buffer:
+// cache hits from HBM, misses over the host link.  Host-link reads in flight beside
+// the HBM gather cut its bandwidth by more than half, so the two never run
+// concurrently.  Schedules (tuning key "split_miss"):
+//   0  both on the caller's stream, one after the other;
+//   1  hits on the caller's stream, misses after them on the server's side stream,
+//      where they overlap the next batch's sampling;
+//   2  both on the side stream (a gather stage behind the sampling stage): the
+//      caller's stream is free for the next batch's sampling as soon as the lookup
+//      is done.
+// With 1 and 2 the caller's stream does not wait here: the next call on this pipe,
+// or lmi_batch_wait, joins.  The LRU cache joins at once (its insert copies the rows).
+int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last) {
+  const bool have_cache = s->cache_kind != LMI_CACHE_NONE;
+  int mode = (s->feat_loc == LMI_LOC_HOST && have_cache) ? s->split_miss : 0;
+  if (mode == 0) {
+    if (have_cache) {
+      prof_phase(s, st, &s->prof_open, PROF_GATHER_HIT);
+      LMI_TRY(launch_hits(s, p, st, seg, seg_last));
+    }
+    prof_phase(s, st, &s->prof_open, PROF_GATHER_MISS);
+    LMI_TRY(launch_misses(s, p, st, seg, seg_last));
+    prof_phase(s, st, &s->prof_open, -1);
+    return LMI_OK;
   }
+  if (mode == 1) {
+    prof_phase(s, st, &s->prof_open, PROF_GATHER_HIT);
+    LMI_TRY(launch_hits(s, p, st, seg, seg_last));
+  }
+  prof_phase(s, st, &s->prof_open, -1);
+  LMI_HIP(hipEventRecord(p.fork, st));
+  LMI_HIP(hipStreamWaitEvent(s->side, p.fork, 0));
+  if (mode == 2) {
+    prof_phase(s, s->side, &s->prof_open_side, PROF_GATHER_HIT);
+    LMI_TRY(launch_hits(s, p, s->side, seg, seg_last));
+  }
+  prof_phase(s, s->side, &s->prof_open_side, PROF_GATHER_MISS);
+  LMI_TRY(launch_misses(s, p, s->side, seg, seg_last));
+  prof_phase(s, s->side, &s->prof_open_side, -1);
+  LMI_HIP(hipEventRecord(p.join, s->side));
+  p.side_pending = true;
+  if (s->cache_kind == LMI_CACHE_LRU) LMI_TRY(pipe_join(p, st));
   return LMI_OK;
 }
 

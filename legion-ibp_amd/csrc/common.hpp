@@ -93,7 +93,6 @@ struct Pipe {
   int32_t max_tiles = 0;
   int2 *miss_list = nullptr;   // [max_nodes] (row, id) pairs of cache misses
   int32_t *lru_fill = nullptr;                        // [max_nodes] slot granted to a miss
-  hipStream_t side = nullptr;  // second stream for the host-link gather
   hipEvent_t fork = nullptr, join = nullptr;
   bool side_pending = false;   // the side stream still owes this pipe's miss rows (join not yet waited on)
   int32_t *seed_stage = nullptr;  // [batch_size] host seeds land here
@@ -152,6 +151,7 @@ struct Server {
   int32_t *lru_keys = nullptr, *lru_use = nullptr, *lru_claim[2] = {nullptr, nullptr};
   // pipes
   std::vector<Pipe> pipes;
+  hipStream_t side = nullptr;  // server-owned second stream for gathers that must not hold up the caller's stream
   // tuning
   int gather_lpr = 0;     // lanes per row (0 = auto)
   int gather_vec = 0;     // bytes per lane access (0 = widest that fits: 16)
@@ -159,7 +159,7 @@ struct Server {
   int gather_blocks = 0;  // 0 = auto
   int gather_nt = 1;      // non-temporal output stores
   int lds_dedup = 0;      // 1: hop_sample stages its probes through an LDS hash table
-  int split_miss = 1;     // 1: host-link gather on the pipe's side stream, after the HBM gather
+  int split_miss = 1;     // gather schedule, see launch_gather_seg
   int use_graph = 1;      // lmi_run_once replays a captured HIP graph
   int miss_blocks = 32;   // grid of the host-link gather: enough reads in flight to fill the link, few enough
                           // not to crowd HBM traffic out of the memory pipeline
@@ -170,8 +170,8 @@ struct Server {
   std::vector<hipEvent_t> prof_used;    // every event recorded since the last read (pairs may share one)
   std::vector<hipEvent_t> prof_free;    // recycled events
   int prof_open = -1;                   // pair still waiting for its end event on the caller's stream
-  DevState *prof_ring = nullptr;        // pinned host snapshots of finished batches
-  int prof_ring_n = 0;
+  int prof_open_side = -1;              // the same for the side stream
+  unsigned long long *d_prof_rows = nullptr;  // device counters: [0] rows offered to hit gathers, [1] miss rows
   lmi_profile prof{};
   int32_t *d_scalar = nullptr;          // small device scratch (counts for build-time launches)
   int n_cu = 256;
@@ -184,7 +184,7 @@ int prof_begin(Server *s, hipStream_t st, int kind);
 int prof_end(Server *s, hipStream_t st, int handle);
 // One event closes the pair left open on the caller's stream and opens the next
 // phase (next_kind < 0: only close), so a batch costs one event per phase boundary.
-void prof_phase(Server *s, hipStream_t st, int next_kind);
+void prof_phase(Server *s, hipStream_t st, int *open, int next_kind);
 
 // sampler.hip
 // stage_seeds: also run the seed-staging kernel now (otherwise hop 0 stages them itself)

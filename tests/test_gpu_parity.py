@@ -315,8 +315,9 @@ def test_synth_graph_matches_oracle(lmi, oracle):
     assert 8.0 < mean < 10.0
 
 
+@pytest.mark.parametrize("schedule", [0, 1, 2])
 @pytest.mark.parametrize("cache", ["static", "lru", "int8"])
-def test_graph_replay_matches_eager_and_oracle(lmi, oracle, cache):
+def test_graph_replay_matches_eager_and_oracle(lmi, oracle, cache, schedule):
     """lmi_run_once on a real stream replays a captured HIP graph; every replay is
     checked against the oracle, with eager batches and synchronisations in between."""
     rng = np.random.default_rng(21)
@@ -329,6 +330,7 @@ def test_graph_replay_matches_eager_and_oracle(lmi, oracle, cache):
     streams = [lmi.stream_create(), lmi.stream_create()]
     lru = oracle.Lru(128, 4, dim * 4)
     try:
+        srv.tune("split_miss", schedule)   # where the HBM and host-link gathers run (caller / side stream)
         srv.load_graph(indptr, indices)
         srv.attach_features(feats)
         srv.load_idset(lmi.MODE_TRAIN, train)
