@@ -8,7 +8,7 @@ the timed region starts.  One JSON line is printed on stdout.
 
     python bench.py [--gpus 1] [--steps 50] [--warmup 5] [--workload paper100m]
 
-Workloads (BASELINE.json `configs`): paper100m (default, the configuration the
+Workloads: paper100m (default, the configuration the
 metric is quoted on), products, paper100m-lru, mag240m-int8 (down-scaled node
 count, stated in the output), cora.  `--scale` shrinks node counts for quick runs.
 """
@@ -150,7 +150,8 @@ def cpu_baseline(lmi, srv, w, info, seed, budget_s):
     feats = info["feats"].array
     B = w["batch"]
     done, spent, parity_ok, rows = 0, 0.0, True, 0
-    while done < 20 and spent < budget_s:
+    max_batches = min(64, len(info["train"]) // B)
+    while done < max_batches and spent < budget_s:
         seeds = info["train"][done * B:(done + 1) * B]
         rs = seed + done
         t0 = time.time()
@@ -269,7 +270,7 @@ def main():
         "metric": "sampled mini-batches/sec", "value": round(args.steps / (t1 - t0), 2), "unit": "batches/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int32 ids / " + ("fp16" if w["dtype"] == "f16" else "fp32") + " rows (byte copy)",
+        "dtype": "int32", "feature_dtype": "fp16" if w["dtype"] == "f16" else "fp32",
         "data": "synthetic",
         "config": {"workload": args.workload, "nodes": info["n_nodes"], "edges": info["n_edges"],
                    "feat_dim": w["dim"], "batch": w["batch"], "fanout": w["fanout"],

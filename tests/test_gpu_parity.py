@@ -291,7 +291,7 @@ def test_int8_cache_parity(lmi, oracle, dim, dtype):
             assert_batch_equal(g, o)
             np.testing.assert_array_equal(g.cache_index, slot_ref[o.ids])
             ref = oracle.gather_rows_int8(o.ids, slot_ref[o.ids], q, sc, feats.array)
-            # tolerance: north-star allows 1 ulp on dequantised rows; both sides do one IEEE
+            # tolerance: the specification allows 1 ulp on dequantised rows; both sides do one IEEE
             # multiply (+ RNE to fp16), so the expected difference is 0
             assert g.features.tobytes() == ref.tobytes()
     finally:

@@ -1,4 +1,5 @@
-"""BASELINE.json's five configurations as parity cases: the synthetic workload
+"""The five target configurations (Cora-, products-, paper100m-, paper100m-LRU- and
+MAG240M-shaped) as parity cases: the synthetic workload
 builder of bench.py (graph generated on the GPU) at full size where that is
 cheap (cora, products) and at a stated fraction of the node count otherwise,
 compared with the CPU oracle batch by batch."""
@@ -123,7 +124,7 @@ def test_int8_workload(lmi, oracle):
             check_batch(g, o)
             assert np.array_equal(g.cache_index, slot_ref[o.ids])
             ref = oracle.gather_rows_int8(o.ids, slot_ref[o.ids], q, sc, feats)
-            assert g.features.tobytes() == ref.tobytes()     # 0 ulp (north star allows 1)
+            assert g.features.tobytes() == ref.tobytes()     # 0 ulp (the specification allows 1)
             hit = g.cache_index >= 0
             assert hit.any() and (~hit).any()
             # the codec is lossy but bounded: |y - x| <= scale / 2 (+ fp16 rounding of y)
