@@ -69,7 +69,7 @@ def log(msg):
     print("[bench] " + msg, file=sys.stderr, flush=True)
 
 
-def build_workload(lmi, w, seed, pipes, host_budget_gb, table=2):
+def build_workload(lmi, w, seed, pipes, host_budget_gb, table=2, policy="degree"):
     """Generate the graph, features, train set and cache; returns (server, info)."""
     np_dtype = np.float16 if w["dtype"] == "f16" else np.float32
     esz = np.dtype(np_dtype).itemsize
@@ -110,6 +110,13 @@ def build_workload(lmi, w, seed, pipes, host_budget_gb, table=2):
     n_train = min(w["train"], n_nodes)
     train = lmi.synth_trainset(seed + 2, n_nodes, n_train)
     srv.load_idset(lmi.MODE_TRAIN, train)
+    if policy == "presampled":
+        # the reference's policy: one presampling pass over the training set, rank by sampled frequency
+        t0 = time.time()
+        srv.presample(-(-n_train // w["batch"]))
+        srv.cache_policy(lmi.POLICY_PRESAMPLED)
+        lmi.check(lmi.lib().lmi_device_sync())
+        log("presampled one epoch (%.2f s)" % (time.time() - t0))
     t0 = time.time()
     kind, amount = w["cache"]
     row_bytes = w["dim"] * esz
@@ -198,6 +205,8 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget (0 = skip)")
     ap.add_argument("--host-gb", type=float, default=64.0, help="pinned host memory budget for the feature table")
     ap.add_argument("--table", default="rank", choices=["hash", "direct", "rank"], help="id->slot table layout")
+    ap.add_argument("--policy", default="degree", choices=["degree", "presampled"],
+                    help="ranking of the static hot set: out-degree (the configs' choice) or presampled frequency")
     ap.add_argument("--tune", action="append", default=[], help="key=value passed to lmi_tune")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -214,7 +223,7 @@ def main():
     if w["cache"][0] == "lru":
         args.pipes = 1   # the LRU state is batch-synchronous: batches may not overlap
     srv, info = build_workload(lmi, w, args.seed, args.pipes, args.host_gb,
-                               {"hash": 0, "direct": 1, "rank": 2}[args.table])
+                               {"hash": 0, "direct": 1, "rank": 2}[args.table], args.policy)
     for kv in args.tune:
         k, v = kv.split("=")
         srv.tune(k, int(v))
@@ -275,7 +284,7 @@ def main():
         "config": {"workload": args.workload, "nodes": info["n_nodes"], "edges": info["n_edges"],
                    "feat_dim": w["dim"], "batch": w["batch"], "fanout": w["fanout"],
                    "cache": "%s, %d rows, %s id->slot table" % (info["cache_kind"], info["cache_rows"], args.table),
-                   "pipes": args.pipes, "streams": args.streams,
+                   "pipes": args.pipes, "streams": args.streams, "cache_policy": args.policy,
                    "graph": "Zipf-Mandelbrot degrees alpha=%s, degree-proportional neighbours" % w["alpha"],
                    "note": info["note"]},
         "feature_gather_gbs": round(achieved, 1),

@@ -50,6 +50,9 @@ enum { LMI_MODE_TRAIN = 0, LMI_MODE_VALID = 1, LMI_MODE_TEST = 2 }; /* TRAINMODE
  * slot, load <= 0.5), direct map (4 B per node), or membership bitmap with a
  * running rank (16 B per 64 nodes; slot = rank of the node among cached nodes) */
 enum { LMI_TABLE_HASH = 0, LMI_TABLE_DIRECT = 1, LMI_TABLE_RANK = 2 };
+/* how the static / int8 hot set is ranked: by out-degree, or by how often presampling
+ * touched a node (the reference's policy, cache/cache.cu:354-447); ties by ascending id */
+enum { LMI_POLICY_DEGREE = 0, LMI_POLICY_PRESAMPLED = 1 };
 enum { LMI_CACHE_NONE = 0, LMI_CACHE_STATIC = 1, LMI_CACHE_LRU = 2, LMI_CACHE_INT8 = 3 };
 
 typedef struct lmi_server lmi_server;
@@ -141,9 +144,23 @@ int lmi_features_attach(lmi_server *s, const void *rows, int64_t n_rows, int loc
 int lmi_idset_load(lmi_server *s, int mode, const int32_t *ids, const int32_t *labels,
                    int64_t n, int location);
 
+/* ---- presampling (GPUServer::PreSc + PreSCCacheController, engine/server.cu:94-122,
+ *      cache/cache.cu:43-71) ------------------------------------------------------ */
+/* Samples batches first_batch .. first_batch+n_batches-1 of id set `mode` (no lookup, no
+ * gather) and adds one count per sampled id to the per-node hotness table.  Enqueued on
+ * `stream`; RNG seeds are the default per-batch seeds, so the same batches are served later. */
+int lmi_presample(lmi_server *s, int pipe, void *stream, int mode, int32_t first_batch, int32_t n_batches);
+/* HotnessMeasure for the batch currently in `pipe` (what IOComplete does while presampling,
+ * engine/operator_impl.cu:607-636). */
+int lmi_op_hotness(lmi_server *s, int pipe, void *stream);
+int lmi_presample_reset(lmi_server *s);                      /* forget the counts */
+int lmi_hotness_dump(lmi_server *s, uint32_t *counts, int64_t n);   /* synchronous read-back */
+/* Ranking used by the next lmi_cache_build_static / lmi_cache_build_int8. */
+int lmi_cache_policy(lmi_server *s, int policy);
+
 /* ---- caches (UnifiedCache::FillUp, cache/cache.cu:559-656) -------------- */
-/* Static hot-set cache: the capacity_rows nodes ranked first by (out-degree
- * descending, id ascending). */
+/* Static hot-set cache: the capacity_rows nodes ranked first by (key descending, id
+ * ascending); key = out-degree, or the presampling count under LMI_POLICY_PRESAMPLED. */
 int lmi_cache_build_static(lmi_server *s, int64_t capacity_rows, int table_kind);
 /* LRU dynamic cache, set-associative (comp_cache/static_cache.cu:20-113), starts empty. */
 int lmi_cache_build_lru(lmi_server *s, int64_t n_sets, int32_t ways);

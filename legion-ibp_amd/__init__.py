@@ -19,6 +19,7 @@ LOC_HOST, LOC_DEVICE = 0, 1
 MODE_TRAIN, MODE_VALID, MODE_TEST = 0, 1, 2
 TABLE_HASH, TABLE_DIRECT, TABLE_RANK = 0, 1, 2
 CACHE_NONE, CACHE_STATIC, CACHE_LRU, CACHE_INT8 = 0, 1, 2, 3
+POLICY_DEGREE, POLICY_PRESAMPLED = 0, 1
 
 # every symbol include/legion_mi.h declares
 ABI_SYMBOLS = [
@@ -26,7 +27,8 @@ ABI_SYMBOLS = [
     "lmi_host_alloc", "lmi_host_free", "lmi_device_alloc", "lmi_device_free",
     "lmi_copy_to_host", "lmi_copy_to_device", "lmi_stream_create", "lmi_stream_destroy",
     "lmi_stream_sync", "lmi_device_sync", "lmi_graph_load", "lmi_features_attach",
-    "lmi_idset_load", "lmi_cache_build_static", "lmi_cache_build_lru", "lmi_cache_build_int8",
+    "lmi_idset_load", "lmi_presample", "lmi_op_hotness", "lmi_presample_reset", "lmi_hotness_dump",
+    "lmi_cache_policy", "lmi_cache_build_static", "lmi_cache_build_lru", "lmi_cache_build_int8",
     "lmi_cache_info_get", "lmi_cache_dump", "lmi_op_batch_generate", "lmi_op_random_sample",
     "lmi_op_cache_lookup", "lmi_op_io_submit", "lmi_op_io_complete", "lmi_run_once",
     "lmi_batch_wait", "lmi_batch_view_get", "lmi_batch_counters", "lmi_steps_per_epoch", "lmi_profile_enable",
@@ -95,6 +97,11 @@ def lib():
         L.lmi_graph_load.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int]
         L.lmi_features_attach.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
         L.lmi_idset_load.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
+        L.lmi_presample.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int32, C.c_int32]
+        L.lmi_op_hotness.argtypes = [C.c_void_p, C.c_int, C.c_void_p]
+        L.lmi_presample_reset.argtypes = [C.c_void_p]
+        L.lmi_hotness_dump.argtypes = [C.c_void_p, C.c_void_p, C.c_int64]
+        L.lmi_cache_policy.argtypes = [C.c_void_p, C.c_int]
         L.lmi_cache_build_static.argtypes = [C.c_void_p, C.c_int64, C.c_int]
         L.lmi_cache_build_int8.argtypes = [C.c_void_p, C.c_int64, C.c_int]
         L.lmi_cache_build_lru.argtypes = [C.c_void_p, C.c_int64, C.c_int32]
@@ -205,6 +212,18 @@ class Server:
             labels = np.ascontiguousarray(labels, dtype=np.int32)
             lp = labels.ctypes.data
         check(lib().lmi_idset_load(self.h, mode, ids.ctypes.data, lp, len(ids), LOC_HOST))
+
+    # presampling -------------------------------------------------------------
+    def presample(self, n_batches, first_batch=0, mode=MODE_TRAIN, pipe=0, stream=None):
+        check(lib().lmi_presample(self.h, pipe, stream, mode, first_batch, n_batches))
+
+    def hotness(self, n_nodes):
+        out = np.empty(n_nodes, np.uint32)
+        check(lib().lmi_hotness_dump(self.h, out.ctypes.data, n_nodes))
+        return out
+
+    def cache_policy(self, policy):
+        check(lib().lmi_cache_policy(self.h, policy))
 
     # caches ------------------------------------------------------------------
     def build_static_cache(self, rows, table=TABLE_HASH):

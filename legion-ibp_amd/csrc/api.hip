@@ -222,6 +222,7 @@ int lmi_server_destroy(lmi_server *h) {
   for (auto &e : s->prof_free) (void)hipEventDestroy(e);
   if (s->d_prof_rows) (void)hipFree(s->d_prof_rows);
   if (s->d_scalar) (void)hipFree(s->d_scalar);
+  if (s->hot) (void)hipFree(s->hot);
   if (s->side) (void)hipStreamDestroy(s->side);
   delete s;
   return LMI_OK;
@@ -285,6 +286,10 @@ int lmi_graph_load(lmi_server *h, const int64_t *indptr, const int32_t *indices,
     (void)hipFree((void *)s->indptr);
     (void)hipFree((void *)s->indices);
     s->own_graph = false;
+  }
+  if (s->hot) {  // counts belong to the previous graph
+    (void)hipFree(s->hot);
+    s->hot = nullptr;
   }
   if (location == LMI_LOC_DEVICE) {
     s->indptr = indptr;
@@ -390,6 +395,31 @@ int lmi_cache_dump(lmi_server *h, int32_t *slot_of, int64_t n, int32_t *aux) {
   return cache_dump(s, slot_of, n, aux);
 }
 
+// -------------------------------------------------------------- presampling
+int lmi_cache_policy(lmi_server *h, int policy) {
+  Server *s = reinterpret_cast<Server *>(h);
+  if (!s || (policy != LMI_POLICY_DEGREE && policy != LMI_POLICY_PRESAMPLED)) LMI_FAIL(LMI_ERR_ARG, "bad policy");
+  s->policy = policy;
+  return LMI_OK;
+}
+
+int lmi_presample_reset(lmi_server *h) {
+  Server *s = reinterpret_cast<Server *>(h);
+  if (!s) LMI_FAIL(LMI_ERR_ARG, "null server");
+  LMI_HIP(hipDeviceSynchronize());
+  if (s->hot) LMI_HIP(hipMemset(s->hot, 0, (size_t)s->n_nodes * 4));
+  return LMI_OK;
+}
+
+int lmi_hotness_dump(lmi_server *h, uint32_t *counts, int64_t n) {
+  Server *s = reinterpret_cast<Server *>(h);
+  if (!s || !counts || n != s->n_nodes) LMI_FAIL(LMI_ERR_ARG, "hotness dump needs n == n_nodes");
+  if (!s->hot) LMI_FAIL(LMI_ERR_STATE, "nothing presampled yet");
+  LMI_HIP(hipDeviceSynchronize());
+  LMI_HIP(hipMemcpy(counts, s->hot, (size_t)n * 4, hipMemcpyDeviceToHost));
+  return LMI_OK;
+}
+
 // ---------------------------------------------------------------- operators
 static int ready(Server *s) {
   if (!s->indptr) LMI_FAIL(LMI_ERR_STATE, "no graph loaded");
@@ -462,6 +492,32 @@ int lmi_op_cache_lookup(lmi_server *h, int pipe, void *stream, int segment) {
   LMI_TRY(launch_lookup(s, p, st, segment, segment));
   LMI_TRY(launch_gather_seg(s, p, st, segment, segment));
   prof_phase(s, st, &s->prof_open, -1);
+  return LMI_OK;
+}
+
+int lmi_op_hotness(lmi_server *h, int pipe, void *stream) {
+  Server *s = reinterpret_cast<Server *>(h);
+  LMI_TRY(check_pipe(s, pipe));
+  LMI_TRY(ready(s));
+  return launch_hotness(s, s->pipes[pipe], (hipStream_t)stream);
+}
+
+int lmi_presample(lmi_server *h, int pipe, void *stream, int mode, int32_t first_batch, int32_t n_batches) {
+  Server *s = reinterpret_cast<Server *>(h);
+  LMI_TRY(check_pipe(s, pipe));
+  if (n_batches < 0) LMI_FAIL(LMI_ERR_ARG, "negative batch count");
+  Pipe &p = s->pipes[pipe];
+  hipStream_t st = (hipStream_t)stream;
+  for (int32_t b = first_batch; b < first_batch + n_batches; ++b) {
+    BatchParams bp{};
+    LMI_TRY(pipe_join(p, st));
+    const int tick = s->lru_tick;
+    LMI_TRY(batch_params(s, p, st, nullptr, 0, LMI_LOC_DEVICE, b, mode, 0, &bp));
+    s->lru_tick = tick;  // presampling does not age the LRU cache
+    LMI_TRY(launch_batch_generate(s, p, st, bp, false));
+    for (int k = 0; k < s->cfg.hops; ++k) LMI_TRY(launch_hop(s, p, st, k, true));
+    LMI_TRY(launch_hotness(s, p, st));
+  }
   return LMI_OK;
 }
 

@@ -601,12 +601,40 @@ int launch_lru_insert(Server *s, Pipe &p, hipStream_t st, int n_lists) {
 }
 
 // -------------------------------------------------------- static cache build
-static __global__ __launch_bounds__(256) void degree_stats_kernel(const int64_t *indptr, int64_t n,
-                                                                  int64_t thr, unsigned long long *count_ge,
+// Ranking key of a node: its out-degree, or how often presampling touched it.
+__device__ __forceinline__ int64_t rank_key(const int64_t *indptr, const uint32_t *hot, int64_t v) {
+  return hot ? (int64_t)hot[v] : indptr[v + 1] - indptr[v];
+}
+
+// Presampling hotness (reference: HotnessMeasure, cache/cache_impl.cuh:190-198): one
+// count per appearance of a node among a batch's sampled ids.
+static __global__ __launch_bounds__(256) void hotness_kernel(const int32_t *ids, const DevState *st, int64_t n_nodes,
+                                                             uint32_t *hot) {
+  const int n = st->node_counter[7];
+  for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < n; i += gridDim.x * blockDim.x) {
+    const int32_t v = ids[i];
+    if (v >= 0 && v < n_nodes) atomicAdd(&hot[v], 1u);
+  }
+}
+
+int launch_hotness(Server *s, Pipe &p, hipStream_t st) {
+  if (!s->hot) {
+    LMI_HIP(hipMalloc(&s->hot, (size_t)s->n_nodes * 4));
+    LMI_HIP(hipMemsetAsync(s->hot, 0, (size_t)s->n_nodes * 4, st));
+  }
+  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(s->max_nodes, 256), (int64_t)s->n_cu * 4));
+  hipLaunchKernelGGL(hotness_kernel, dim3(grid), dim3(256), 0, st, p.ids, p.st, s->n_nodes, s->hot);
+  LMI_HIP(hipGetLastError());
+  return LMI_OK;
+}
+
+static __global__ __launch_bounds__(256) void degree_stats_kernel(const int64_t *indptr, const uint32_t *hot,
+                                                                  int64_t n, int64_t thr,
+                                                                  unsigned long long *count_ge,
                                                                   unsigned long long *max_deg) {
   unsigned long long c = 0, m = 0;
   for (int64_t v = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; v < n; v += (int64_t)gridDim.x * blockDim.x) {
-    const unsigned long long d = (unsigned long long)(indptr[v + 1] - indptr[v]);
+    const unsigned long long d = (unsigned long long)rank_key(indptr, hot, v);
     c += (d >= (unsigned long long)thr) ? 1 : 0;
     m = d > m ? d : m;
   }
@@ -624,8 +652,8 @@ static __global__ __launch_bounds__(256) void degree_stats_kernel(const int64_t 
 
 // mode 0: cnt[v] = (deg == thr);  mode 1: cnt[v] = member flag using tie ranks.
 static __global__ __launch_bounds__(kScanBlock) void member_flag_kernel(
-    const int64_t *indptr, const int32_t *n_ptr, int64_t thr, int mode, const int32_t *tie_rank,
-    int64_t ties_taken, int32_t *cnt, int32_t *tile_sums) {
+    const int64_t *indptr, const uint32_t *hot, const int32_t *n_ptr, int64_t thr, int mode,
+    const int32_t *tie_rank, int64_t ties_taken, int32_t *cnt, int32_t *tile_sums) {
   __shared__ int lds[kScanBlock / kWave];
   const int n = *n_ptr;
   const int n_tiles = (n + kScanTile - 1) / kScanTile;
@@ -636,7 +664,7 @@ static __global__ __launch_bounds__(kScanBlock) void member_flag_kernel(
     for (int j = 0; j < kScanItems; ++j) {
       const int v = base + j;
       if (v < n) {
-        const int64_t d = indptr[v + 1] - indptr[v];
+        const int64_t d = rank_key(indptr, hot, v);
         int f;
         if (mode == 0) f = (d == thr);
         else f = (d > thr) || (d == thr && (int64_t)tie_rank[v] < ties_taken);
@@ -718,8 +746,8 @@ void cache_free(Server *s) {
 
 static int count_ge(const Server *s, int64_t thr, unsigned long long *d_pair, int64_t *count, int64_t *max_deg) {
   LMI_HIP(hipMemset(d_pair, 0, 16));
-  hipLaunchKernelGGL(degree_stats_kernel, dim3(s->n_cu * 8), dim3(256), 0, 0, s->indptr, s->n_nodes, thr, d_pair,
-                     d_pair + 1);
+  hipLaunchKernelGGL(degree_stats_kernel, dim3(s->n_cu * 8), dim3(256), 0, 0, s->indptr,
+                     s->policy == LMI_POLICY_PRESAMPLED ? s->hot : nullptr, s->n_nodes, thr, d_pair, d_pair + 1);
   unsigned long long h[2];
   LMI_HIP(hipMemcpy(h, d_pair, 16, hipMemcpyDeviceToHost));
   *count = (int64_t)h[0];
@@ -741,6 +769,9 @@ int cache_build_static(Server *s, int64_t capacity_rows, int table_kind, bool in
   s->table_kind = table_kind;
   s->cache_row_bytes = int8 ? s->cfg.feat_dim : s->row_bytes;
   if (cap == 0) LMI_FAIL(LMI_ERR_ARG, "cache capacity must be at least one row");
+  if (s->policy == LMI_POLICY_PRESAMPLED && !s->hot)
+    LMI_FAIL(LMI_ERR_STATE, "the presampled policy needs lmi_presample (or presampling operators) first");
+  const uint32_t *hot_key = s->policy == LMI_POLICY_PRESAMPLED ? s->hot : nullptr;
 
   unsigned long long *d_pair = nullptr;
   int32_t *d_cnt = nullptr, *d_tie = nullptr, *d_slot = nullptr, *d_tiles = nullptr, *d_n = nullptr,
@@ -769,10 +800,10 @@ int cache_build_static(Server *s, int64_t capacity_rows, int table_kind, bool in
   const int64_t ties_taken = cap - cnt;
 
   const int grid = scan_grid(N);
-  hipLaunchKernelGGL(member_flag_kernel, dim3(grid), dim3(kScanBlock), 0, 0, s->indptr, d_n, thr, 0, nullptr,
+  hipLaunchKernelGGL(member_flag_kernel, dim3(grid), dim3(kScanBlock), 0, 0, s->indptr, hot_key, d_n, thr, 0, nullptr,
                      (int64_t)0, d_cnt, d_tiles);
   LMI_TRY(launch_scan_phases(0, d_cnt, d_tie, d_tiles, d_n, N, SCAN_EPI_NONE, nullptr, 0, d_n + 1));
-  hipLaunchKernelGGL(member_flag_kernel, dim3(grid), dim3(kScanBlock), 0, 0, s->indptr, d_n, thr, 1, d_tie,
+  hipLaunchKernelGGL(member_flag_kernel, dim3(grid), dim3(kScanBlock), 0, 0, s->indptr, hot_key, d_n, thr, 1, d_tie,
                      ties_taken, d_cnt, d_tiles);
   LMI_TRY(launch_scan_phases(0, d_cnt, d_slot, d_tiles, d_n, N, SCAN_EPI_NONE, nullptr, 0, d_n + 1));
   int32_t total = 0;

@@ -136,6 +136,8 @@ struct Server {
   int32_t *set_labels[3] = {nullptr, nullptr, nullptr};
   int64_t set_n[3] = {0, 0, 0};
   // cache
+  int policy = LMI_POLICY_DEGREE;    // ranking key of the static / int8 hot set
+  uint32_t *hot = nullptr;           // [n_nodes] presampling appearance counts
   int cache_kind = LMI_CACHE_NONE;
   int table_kind = LMI_TABLE_HASH;
   int64_t cache_rows = 0;
@@ -200,6 +202,7 @@ int cache_build_static(Server *s, int64_t capacity_rows, int table_kind, bool in
 int cache_build_lru(Server *s, int64_t n_sets, int32_t ways);
 void cache_free(Server *s);
 int launch_lookup(Server *s, Pipe &p, hipStream_t st, int seg_first, int seg_last);
+int launch_hotness(Server *s, Pipe &p, hipStream_t st);
 int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last);
 int launch_lru_insert(Server *s, Pipe &p, hipStream_t st, int n_lists);
 int pipe_join(Pipe &p, hipStream_t st);  // make `st` wait for the pipe's side-stream work

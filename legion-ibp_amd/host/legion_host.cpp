@@ -100,7 +100,13 @@ class SSDIOSubmitOP : public Operator {
 class SSDIOCompleteOP : public Operator {
  public:
   explicit SSDIOCompleteOP(int id) : op_id_(id) {}
-  void run(OpParams *p) override { LMI_MUST(lmi_op_io_complete((lmi_server *)p->env, p->pipe, p->stream)); }
+  void run(OpParams *p) override {
+    if (p->is_presc) {  // CacheProfiling: count the batch's sampled ids (engine/operator_impl.cu:607-636)
+      LMI_MUST(lmi_op_hotness((lmi_server *)p->env, p->pipe, p->stream));
+      return;
+    }
+    LMI_MUST(lmi_op_io_complete((lmi_server *)p->env, p->pipe, p->stream));
+  }
  private:
   int op_id_;
 };
@@ -249,6 +255,18 @@ class GPUServer : public Server {
       std::exit(EXIT_FAILURE);
     }
     const int64_t row_bytes = (int64_t)meta_.feature_dim * 4;
+    if (std::getenv("LEGION_MI_PRESAMPLE")) {
+      // the reference's policy: one presampling pass over the training set through the
+      // operator table, then rank by how often each node was sampled (engine/server.cu:31-37,94-122)
+      int32_t steps = 0;
+      LMI_MUST(lmi_steps_per_epoch(h_, LMI_MODE_TRAIN, &steps));
+      for (int i = 0; i < steps; ++i) {
+        params_.global_batch_id = i;
+        runner_->RunPreSc(&params_);
+      }
+      runner_->InitializeFeaturesBuffer(&params_);
+      LMI_MUST(lmi_cache_policy(h_, LMI_POLICY_PRESAMPLED));
+    }
     if (dyn_cache_ & LEGION_DYN_COMP) {
       const int64_t rows = std::max<int64_t>(1, meta_.cache_memory / (meta_.feature_dim + 4));
       LMI_MUST(lmi_cache_build_int8(h_, rows, LMI_TABLE_RANK));

@@ -55,7 +55,8 @@ class Server {
   virtual ~Server() {}
   // Reads ./meta_config and the dataset it names, creates the per-GPU server.
   virtual void Initialize(int global_shard_count, std::vector<int> fanout, int in_memory_mode, int dyn_cache) = 0;
-  // Builds the feature cache (the reference presamples here; this build ranks by degree).
+  // Builds the feature cache: ranked by degree, or (LEGION_MI_PRESAMPLE set) by one presampling
+  // pass over the training set, which is what the reference does here.
   virtual void PreSc(int cache_agg_mode) = 0;
   // epoch x steps mini-batches through the runner.
   virtual void Run() = 0;

@@ -135,6 +135,14 @@ def static_cache_build(indptr, cap_rows):
     return slot_of
 
 
+def static_cache_build_keys(keys, cap_rows):
+    keys = np.ascontiguousarray(keys, dtype=np.int64)
+    slot_of = np.empty(len(keys), np.int32)
+    lib().orc_static_cache_build_keys(_ptr(keys, C.c_int64), C.c_int64(len(keys)), C.c_int64(cap_rows),
+                                      _ptr(slot_of, C.c_int32))
+    return slot_of
+
+
 class Lru:
     def __init__(self, n_sets, ways, row_bytes):
         self.n_sets, self.ways, self.row_bytes = n_sets, ways, row_bytes

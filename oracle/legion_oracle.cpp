@@ -257,11 +257,19 @@ int orc_sample_batch(const int64_t *indptr, const int32_t *indices, int64_t n_no
  * is undefined. */
 void orc_static_cache_build(const int64_t *indptr, int64_t n_nodes, int64_t cap_rows,
                             int32_t *slot_of) {
+  std::vector<int64_t> deg((size_t)n_nodes);
+  for (int64_t v = 0; v < n_nodes; ++v) deg[v] = indptr[v + 1] - indptr[v];
+  orc_static_cache_build_keys(deg.data(), n_nodes, cap_rows, slot_of);
+}
+
+/* The same selection for any ranking key (key descending, id ascending); with
+ * key = presampling appearance counts this is the reference's hot-set policy
+ * (cache/cache.cu:354-447) with its undefined tie order made definite. */
+void orc_static_cache_build_keys(const int64_t *keys, int64_t n_nodes, int64_t cap_rows,
+                                 int32_t *slot_of) {
   std::vector<int32_t> order((size_t)n_nodes);
   std::iota(order.begin(), order.end(), 0);
-  std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) {
-    return (indptr[a + 1] - indptr[a]) > (indptr[b + 1] - indptr[b]);
-  });
+  std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return keys[a] > keys[b]; });
   for (int64_t v = 0; v < n_nodes; ++v) slot_of[v] = -1;
   const int64_t cap = std::min(std::max<int64_t>(cap_rows, 0), n_nodes);
   for (int64_t r = 0; r < cap; ++r) slot_of[order[r]] = 0;

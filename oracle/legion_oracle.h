@@ -69,6 +69,10 @@ int orc_sample_batch(const int64_t *indptr, const int32_t *indices, int64_t n_no
 void orc_static_cache_build(const int64_t *indptr, int64_t n_nodes, int64_t cap_rows,
                             int32_t *slot_of);
 
+/* the same with an arbitrary ranking key per node (e.g. presampling counts) */
+void orc_static_cache_build_keys(const int64_t *keys, int64_t n_nodes, int64_t cap_rows,
+                                 int32_t *slot_of);
+
 /* ---- LRU dynamic cache ---------------------------------------------- */
 void *orc_lru_create(int64_t n_sets, int32_t ways, int64_t row_bytes);
 void  orc_lru_destroy(void *lru);

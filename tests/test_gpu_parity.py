@@ -370,3 +370,51 @@ def test_graph_replay_matches_eager_and_oracle(lmi, oracle, cache, schedule):
     finally:
         srv.close()
         feats.free()
+
+
+@pytest.mark.parametrize("int8", [False, True])
+def test_presampled_hot_set_policy(lmi, oracle, int8):
+    """The reference's own cache policy: presample the training batches, count how often every
+    node is sampled, cache the most frequently sampled rows (ties by id)."""
+    rng = np.random.default_rng(17)
+    n_nodes, batch, fanout, dim, n_train = 4000, 80, [10, 5], 32, 400
+    indptr, indices = random_graph(rng, n_nodes, 9, hubs=6, hub_deg=500)
+    feats = make_features(lmi, rng, n_nodes, dim)
+    train = rng.permutation(n_nodes)[:n_train].astype(np.int32)
+    srv = lmi.Server(batch, fanout, dim, seed=23)
+    stream = lmi.stream_create()
+    try:
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        srv.load_idset(lmi.MODE_TRAIN, train)
+        with pytest.raises(lmi.LegionError):
+            srv.cache_policy(lmi.POLICY_PRESAMPLED)
+            srv.build_static_cache(500)            # nothing presampled yet
+        srv.presample(3, first_batch=0, stream=stream)
+        srv.presample(2, first_batch=3, stream=stream)
+        counts = np.zeros(n_nodes, np.int64)
+        for b in range(5):
+            o = oracle.sample_batch(indptr, indices, train[b * batch:(b + 1) * batch], fanout, 23 + b)
+            counts += np.bincount(o.ids, minlength=n_nodes)
+        assert np.array_equal(srv.hotness(n_nodes).astype(np.int64), counts)
+        cap = 700
+        slot_ref = oracle.static_cache_build_keys(counts, cap)
+        if int8:
+            srv.build_int8_cache(cap, lmi.TABLE_RANK)
+            q, sc = oracle.quantize_rows(feats.array[np.flatnonzero(slot_ref >= 0)])
+        else:
+            srv.build_static_cache(cap, lmi.TABLE_HASH)
+        assert np.array_equal(srv.cache_dump(n_nodes), slot_ref)
+        assert not np.array_equal(slot_ref >= 0, oracle.static_cache_build(indptr, cap) >= 0)  # differs from degree order
+        srv.run_once(None, batch_counter=1, stream=stream)
+        g = srv.fetch(stream=stream)
+        o = oracle.sample_batch(indptr, indices, train[batch:2 * batch], fanout, 24)
+        assert_batch_equal(g, o)
+        assert np.array_equal(g.cache_index, slot_ref[o.ids])
+        ref = oracle.gather_rows_int8(o.ids, slot_ref[o.ids], q, sc, feats.array) if int8 else feats.array[o.ids]
+        assert g.features.tobytes() == ref.tobytes()
+        # a served batch of the presampled set hits more often than under degree order would guarantee
+        assert (g.cache_index >= 0).mean() > cap / n_nodes
+    finally:
+        srv.close()
+        feats.free()

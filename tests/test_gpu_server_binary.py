@@ -44,8 +44,9 @@ def read_dump(path, dim):
     return nc, ec, ids, src, dst, feat
 
 
-@pytest.mark.parametrize("dyn_cache,table_mode", [(0, False), (0, True), (1, False), (1, True), (8, False)])
-def test_sampling_server_binary(tmp_path, oracle, dyn_cache, table_mode):
+@pytest.mark.parametrize("dyn_cache,table_mode,presample", [(0, False, False), (0, True, False), (1, False, False),
+                                                             (1, True, False), (8, False, False), (0, True, True)])
+def test_sampling_server_binary(tmp_path, oracle, dyn_cache, table_mode, presample):
     assert os.path.exists(BIN), "build the host shim first (make -C legion-ibp_amd)"
     rng = np.random.default_rng(dyn_cache * 2 + table_mode)
     n_nodes, dim, batch, n_train, fanout = 5000, 64, 100, 350, [25, 10]
@@ -60,6 +61,8 @@ def test_sampling_server_binary(tmp_path, oracle, dyn_cache, table_mode):
     env = dict(os.environ, LEGION_MI_DUMP=str(dump), LEGION_MI_DUMP_BATCHES="4")
     if table_mode:
         env["LEGION_MI_OPERATOR_TABLE"] = "1"
+    if presample:
+        env["LEGION_MI_PRESAMPLE"] = "1"   # rank the hot set by a presampling pass, as the reference does
     out = subprocess.run([BIN, "1", "0", str(dyn_cache), "25,10"], cwd=str(tmp_path), env=env, timeout=100,
                          capture_output=True, text=True)
     assert out.returncode == 0, out.stdout + out.stderr

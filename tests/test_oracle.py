@@ -184,6 +184,16 @@ def test_static_cache_is_top_by_degree_then_id(oracle, cap):
     assert np.array_equal(slot[members], np.arange(cap))       # slot = rank among cached ids
 
 
+def test_static_cache_by_arbitrary_keys(oracle):
+    rng = np.random.default_rng(9)
+    keys = rng.integers(0, 6, 800)                    # presampling counts: few distinct values, many ties
+    for cap in (0, 1, 250, 800):
+        slot = oracle.static_cache_build_keys(keys, cap)
+        members = np.sort(np.lexsort((np.arange(800), -keys))[:cap])
+        assert np.array_equal(np.flatnonzero(slot >= 0), members)
+        assert np.array_equal(slot[members], np.arange(cap))
+
+
 # ---------------------------------------------------------------------- LRU
 class PyLru:
     """Independent model: a list of [key, last_use] per set, plain loops."""
