@@ -63,6 +63,22 @@ void prof_phase(Server *s, hipStream_t st, int *open, int next_kind) {
   }
 }
 
+// The captured batch graphs hold the graph, cache-table and tuning state by value:
+// anything that changes those must drop them (they are captured again on next use).
+static void invalidate_graphs(Server *s) {
+  bool any = false;
+  for (auto &p : s->pipes) any = any || p.graph_exec;
+  if (!any) return;
+  (void)hipDeviceSynchronize();
+  for (auto &p : s->pipes) {
+    if (p.graph_exec) (void)hipGraphExecDestroy(p.graph_exec);
+    if (p.graph) (void)hipGraphDestroy(p.graph);
+    p.graph_exec = nullptr;
+    p.graph = nullptr;
+    p.begin_node = nullptr;
+  }
+}
+
 static int check_pipe(Server *s, int pipe) {
   if (!s) LMI_FAIL(LMI_ERR_ARG, "null server");
   if (pipe < 0 || pipe >= (int)s->pipes.size()) LMI_FAIL(LMI_ERR_ARG, "pipe %d out of range", pipe);
@@ -282,6 +298,7 @@ int lmi_graph_load(lmi_server *h, const int64_t *indptr, const int32_t *indices,
   if (!s || !indptr || (!indices && n_edges > 0)) LMI_FAIL(LMI_ERR_ARG, "null argument");
   if (n_nodes < 1 || n_nodes >= (int64_t(1) << 31) - 4096 || n_edges < 0) LMI_FAIL(LMI_ERR_ARG, "bad graph size");
   LMI_HIP(hipSetDevice(s->cfg.device_id));
+  invalidate_graphs(s);
   if (s->own_graph) {
     (void)hipFree((void *)s->indptr);
     (void)hipFree((void *)s->indices);
@@ -357,18 +374,21 @@ int lmi_cache_build_static(lmi_server *h, int64_t capacity_rows, int table_kind)
   Server *s = reinterpret_cast<Server *>(h);
   if (!s) LMI_FAIL(LMI_ERR_ARG, "null server");
   LMI_HIP(hipSetDevice(s->cfg.device_id));
+  invalidate_graphs(s);
   return cache_build_static(s, capacity_rows, table_kind, false);
 }
 int lmi_cache_build_int8(lmi_server *h, int64_t capacity_rows, int table_kind) {
   Server *s = reinterpret_cast<Server *>(h);
   if (!s) LMI_FAIL(LMI_ERR_ARG, "null server");
   LMI_HIP(hipSetDevice(s->cfg.device_id));
+  invalidate_graphs(s);
   return cache_build_static(s, capacity_rows, table_kind, true);
 }
 int lmi_cache_build_lru(lmi_server *h, int64_t n_sets, int32_t ways) {
   Server *s = reinterpret_cast<Server *>(h);
   if (!s) LMI_FAIL(LMI_ERR_ARG, "null server");
   LMI_HIP(hipSetDevice(s->cfg.device_id));
+  invalidate_graphs(s);
   return cache_build_lru(s, n_sets, ways);
 }
 int lmi_cache_info_get(lmi_server *h, lmi_cache_info *out) {
@@ -686,6 +706,7 @@ int lmi_profile_read(lmi_server *h, lmi_profile *out, int reset) {
 int lmi_tune(lmi_server *h, const char *key, int64_t value) {
   Server *s = reinterpret_cast<Server *>(h);
   if (!s || !key) LMI_FAIL(LMI_ERR_ARG, "null argument");
+  invalidate_graphs(s);
   if (!strcmp(key, "gather_lanes_per_row")) s->gather_lpr = (int)value;
   else if (!strcmp(key, "gather_unroll")) s->gather_unroll = (int)value;
   else if (!strcmp(key, "gather_vector_bytes")) s->gather_vec = (int)value;

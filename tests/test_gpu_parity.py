@@ -418,3 +418,36 @@ def test_presampled_hot_set_policy(lmi, oracle, int8):
     finally:
         srv.close()
         feats.free()
+
+
+def test_rebuilding_cache_or_graph_after_graph_capture(lmi, oracle):
+    """The captured batch graph holds table pointers and graph pointers; rebuilding either
+    afterwards must take effect on the next batch."""
+    rng = np.random.default_rng(31)
+    n_nodes, batch, fanout, dim = 3000, 64, [8, 4], 16
+    indptr, indices = random_graph(rng, n_nodes, 8, hubs=4, hub_deg=200)
+    indptr2, indices2 = random_graph(rng, n_nodes, 5, hubs=2, hub_deg=400)
+    feats = make_features(lmi, rng, n_nodes, dim)
+    srv = lmi.Server(batch, fanout, dim)
+    stream = lmi.stream_create()
+    seeds = rng.choice(n_nodes, batch, replace=False).astype(np.int32)
+    try:
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        for step, (cap, table, gp, gi) in enumerate([(500, lmi.TABLE_HASH, indptr, indices),
+                                                     (1500, lmi.TABLE_RANK, indptr, indices),
+                                                     (900, lmi.TABLE_DIRECT, indptr2, indices2)]):
+            if step == 2:
+                srv.load_graph(gp, gi)
+            srv.build_static_cache(cap, table)
+            slot_ref = oracle.static_cache_build(gp, cap)
+            for rep in range(2):
+                srv.run_once(seeds, rng_seed=5 + rep, stream=stream)
+                g = srv.fetch(stream=stream)
+                o = oracle.sample_batch(gp, gi, seeds, fanout, 5 + rep)
+                assert_batch_equal(g, o)
+                assert np.array_equal(g.cache_index, slot_ref[o.ids])
+                assert g.features.tobytes() == feats.array[o.ids].tobytes()
+    finally:
+        srv.close()
+        feats.free()
