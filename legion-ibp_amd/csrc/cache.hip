@@ -15,6 +15,7 @@
 // scale instead of the un-vendored lossless codec; one lane moves 16 bytes and
 // several rows are in flight per lane instead of one float per thread.
 #include <algorithm>
+#include <vector>
 
 #include "scan.hpp"
 
@@ -773,16 +774,28 @@ int cache_build_static(Server *s, int64_t capacity_rows, int table_kind, bool in
     LMI_FAIL(LMI_ERR_STATE, "the presampled policy needs lmi_presample (or presampling operators) first");
   const uint32_t *hot_key = s->policy == LMI_POLICY_PRESAMPLED ? s->hot : nullptr;
 
+  // build-time scratch, released on every return path
+  struct Scratch {
+    std::vector<void *> ptrs;
+    ~Scratch() {
+      for (void *q : ptrs) (void)hipFree(q);
+    }
+    hipError_t get(void **p, size_t bytes) {
+      const hipError_t e = hipMalloc(p, bytes ? bytes : 1);
+      if (e == hipSuccess) ptrs.push_back(*p);
+      return e;
+    }
+  } scratch;
   unsigned long long *d_pair = nullptr;
   int32_t *d_cnt = nullptr, *d_tie = nullptr, *d_slot = nullptr, *d_tiles = nullptr, *d_n = nullptr,
           *d_cached = nullptr;
-  LMI_HIP(hipMalloc(&d_pair, 16));
-  LMI_HIP(hipMalloc(&d_cnt, (N + 1) * 4));
-  LMI_HIP(hipMalloc(&d_tie, (N + 1) * 4));
-  LMI_HIP(hipMalloc(&d_slot, (N + 1) * 4));
-  LMI_HIP(hipMalloc(&d_tiles, (ceil_div(N, kScanTile) + 1) * 4));
-  LMI_HIP(hipMalloc(&d_n, 8));
-  LMI_HIP(hipMalloc(&d_cached, cap * 4));
+  LMI_HIP(scratch.get((void **)&d_pair, 16));
+  LMI_HIP(scratch.get((void **)&d_cnt, (N + 1) * 4));
+  LMI_HIP(scratch.get((void **)&d_tie, (N + 1) * 4));
+  LMI_HIP(scratch.get((void **)&d_slot, (N + 1) * 4));
+  LMI_HIP(scratch.get((void **)&d_tiles, (ceil_div(N, kScanTile) + 1) * 4));
+  LMI_HIP(scratch.get((void **)&d_n, 8));
+  LMI_HIP(scratch.get((void **)&d_cached, cap * 4));
   const int32_t n32[2] = {(int32_t)N, 0};
   LMI_HIP(hipMemcpy(d_n, n32, 8, hipMemcpyHostToDevice));
 
@@ -849,8 +862,6 @@ int cache_build_static(Server *s, int64_t capacity_rows, int table_kind, bool in
     LMI_TRY(launch_move_rows(s, 0, m, false));
   }
   LMI_HIP(hipDeviceSynchronize());
-  (void)hipFree(d_pair); (void)hipFree(d_cnt); (void)hipFree(d_tie); (void)hipFree(d_slot);
-  (void)hipFree(d_tiles); (void)hipFree(d_n); (void)hipFree(d_cached);
   s->cache_rows = cap;
   s->cache_kind = int8 ? LMI_CACHE_INT8 : LMI_CACHE_STATIC;
   return LMI_OK;
