@@ -157,7 +157,7 @@ def cpu_baseline(lmi, srv, w, info, seed, budget_s):
     feats = info["feats"].array
     B = w["batch"]
     done, spent, parity_ok, rows = 0, 0.0, True, 0
-    max_batches = min(64, len(info["train"]) // B)
+    max_batches = min(256, len(info["train"]) // B)
     while done < max_batches and spent < budget_s:
         seeds = info["train"][done * B:(done + 1) * B]
         rs = seed + done
