@@ -191,8 +191,9 @@ int lmi_op_io_submit(lmi_server *s, int pipe, void *stream);
  * misses into the LRU cache. */
 int lmi_op_io_complete(lmi_server *s, int pipe, void *stream);
 /* Runner::RunOnce (engine/server.cu:330-400): the whole operator chain with one
- * gather over all rows.  On a non-default stream the sampling part replays a HIP
- * graph captured on first use.  Returns with the host-link part of the gather
+ * gather over all rows.  With lmi_tune("use_graph", 1) and a non-default stream the
+ * sampling part replays a HIP graph captured on first use instead of launching its
+ * kernels one by one.  Returns with the host-link part of the gather
  * possibly still running on the server's side stream: see lmi_batch_wait. */
 int lmi_run_once(lmi_server *s, int pipe, void *stream, const int32_t *seeds, int32_t n,
                  int seeds_location, int32_t batch_counter, int mode, uint64_t rng_seed);
@@ -212,7 +213,10 @@ int lmi_batch_counters(lmi_server *s, int pipe, void *stream, int32_t node_count
 int lmi_steps_per_epoch(lmi_server *s, int mode, int32_t *steps);
 
 /* ---- measurement ------------------------------------------------------- */
-int lmi_profile_enable(lmi_server *s, int on);   /* on: record HIP events around kernels */
+/* level 0: off; 1: HIP events bracket every phase of a batch (sampling, lookup, both
+ * gathers); 2: only the two gather kernels are bracketed, the sampling kernels run back
+ * to back as without profiling.  Rows per gather are counted on the device at any level. */
+int lmi_profile_enable(lmi_server *s, int level);
 int lmi_profile_read(lmi_server *s, lmi_profile *out, int reset);  /* synchronises the device */
 /* Tuning knobs by name (e.g. "gather_lanes_per_row", "gather_unroll", "lds_dedup"). */
 int lmi_tune(lmi_server *s, const char *key, int64_t value);

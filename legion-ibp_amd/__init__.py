@@ -312,8 +312,9 @@ class Server:
         return b
 
     # measurement -------------------------------------------------------------
-    def profile_enable(self, on=True):
-        check(lib().lmi_profile_enable(self.h, int(on)))
+    def profile_enable(self, level=1):
+        """0 / False: off; 1 / True: events around every phase; 2: around the gather kernels only."""
+        check(lib().lmi_profile_enable(self.h, int(level)))
 
     def profile_read(self, reset=True):
         p = Profile()

@@ -46,12 +46,17 @@ int prof_end(Server *s, hipStream_t st, int handle) {
   return LMI_OK;
 }
 
-void prof_phase(Server *s, hipStream_t st, int *open, int next_kind) {
+// Ends the open bracket of a stream and starts one of kind `next_kind` (-1: none) with a
+// single event record; returns that event, or nullptr when nothing was recorded.  Level 2
+// brackets only the gather kernels, so the sampling kernels run back to back as they do
+// without profiling.
+hipEvent_t prof_phase(Server *s, hipStream_t st, int *open, int next_kind) {
   if (!s->prof_on) {
     *open = -1;
-    return;
+    return nullptr;
   }
-  if (*open < 0 && next_kind < 0) return;
+  if (s->prof_level == 2 && (next_kind == PROF_SAMPLE || next_kind == PROF_LOOKUP)) next_kind = -1;
+  if (*open < 0 && next_kind < 0) return nullptr;
   hipEvent_t e = prof_event(s);
   s->prof_used.push_back(e);
   (void)hipEventRecord(e, st);
@@ -61,6 +66,7 @@ void prof_phase(Server *s, hipStream_t st, int *open, int next_kind) {
     s->prof_events.push_back(EventPair{e, nullptr, next_kind});
     *open = (int)s->prof_events.size() - 1;
   }
+  return e;
 }
 
 // The captured batch graphs hold the graph, cache-table and tuning state by value:
@@ -128,7 +134,15 @@ static int pipe_alloc(Server *s, Pipe &p) {
   LMI_TRY(dmalloc(&p.cnt, scan_n + 1));
   LMI_TRY(dmalloc(&p.rank, s->max_edges_hop + 1));
   LMI_TRY(dmalloc(&p.tile_sums, ceil_div(scan_n, 2048) + 1));
-  p.max_tiles = (int32_t)ceil_div(scan_n, 256) + 1;  // the finest tiling any scan kernel uses
+  // the finest tiling any scan kernel uses: 256 items per tile over nodes or edges, or the
+  // node tiles of the fused count-and-sample kernel
+  int64_t tiles = ceil_div(scan_n, 256);
+  for (int k = 0; k < s->cfg.hops; ++k) {
+    int G = 4;
+    while (G < s->cfg.fanout[k]) G <<= 1;
+    tiles = std::max(tiles, ceil_div(s->node_cap[k], (int64_t)hop_tile_nodes(s->node_cap[k], G)));
+  }
+  p.max_tiles = (int32_t)tiles + 1;
   LMI_TRY(dmalloc(&p.chain_status[0], p.max_tiles));
   LMI_TRY(dmalloc(&p.chain_status[1], p.max_tiles));
   LMI_TRY(dmalloc(&p.miss_list, s->max_nodes));
@@ -668,7 +682,9 @@ int lmi_steps_per_epoch(lmi_server *h, int mode, int32_t *steps) {
 int lmi_profile_enable(lmi_server *h, int on) {
   Server *s = reinterpret_cast<Server *>(h);
   if (!s) LMI_FAIL(LMI_ERR_ARG, "null server");
+  if (on < 0 || on > 2) LMI_FAIL(LMI_ERR_ARG, "profile level must be 0, 1 or 2");
   s->prof_on = on != 0;
+  s->prof_level = on;
   return LMI_OK;
 }
 
@@ -713,6 +729,7 @@ int lmi_tune(lmi_server *h, const char *key, int64_t value) {
   else if (!strcmp(key, "gather_blocks")) s->gather_blocks = (int)value;
   else if (!strcmp(key, "gather_nontemporal")) s->gather_nt = (int)value;
   else if (!strcmp(key, "lds_dedup")) s->lds_dedup = (int)value;
+  else if (!strcmp(key, "fuse_count")) s->fuse_count = (int)value;
   else if (!strcmp(key, "split_miss")) s->split_miss = (int)value;
   else if (!strcmp(key, "use_graph")) s->use_graph = (int)value;
   else if (!strcmp(key, "miss_blocks")) s->miss_blocks = (int)value;

@@ -379,9 +379,16 @@ int launch_lookup(Server *s, Pipe &p, hipStream_t st, int seg_first, int seg_las
   return LMI_OK;
 }
 
+// Orders `st` behind the pipe's work on the side stream.  A wait on another queue's
+// event holds a stream up for about 10 us even when the event fired long ago, so the
+// wait is only queued when the host cannot already see the event as complete.
 int pipe_join(Pipe &p, hipStream_t st) {
   if (p.side_pending) {
-    LMI_HIP(hipStreamWaitEvent(st, p.join, 0));
+    const hipError_t q = hipEventQuery(p.join);
+    if (q != hipSuccess) {
+      (void)hipGetLastError();  // "not ready" is an answer, not a failure
+      LMI_HIP(hipStreamWaitEvent(st, p.join, 0));
+    }
     p.side_pending = false;
   }
   return LMI_OK;
@@ -487,9 +494,13 @@ int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last)
     prof_phase(s, st, &s->prof_open, PROF_GATHER_HIT);
     LMI_TRY(launch_hits(s, p, st, seg, seg_last));
   }
-  prof_phase(s, st, &s->prof_open, -1);
-  LMI_HIP(hipEventRecord(p.fork, st));
-  LMI_HIP(hipStreamWaitEvent(s->side, p.fork, 0));
+  // the event that closes the profiling bracket, when there is one, also serves as the fork
+  hipEvent_t fork = prof_phase(s, st, &s->prof_open, -1);
+  if (!fork) {
+    fork = p.fork;
+    LMI_HIP(hipEventRecord(fork, st));
+  }
+  LMI_HIP(hipStreamWaitEvent(s->side, fork, 0));
   if (mode == 2) {
     prof_phase(s, s->side, &s->prof_open_side, PROF_GATHER_HIT);
     LMI_TRY(launch_hits(s, p, s->side, seg, seg_last));

@@ -160,14 +160,18 @@ struct Server {
   int gather_unroll = 1;  // rows in flight per lane (1 measured best: 62.5 % of HBM peak vs 60 % at 4)
   int gather_blocks = 0;  // 0 = auto
   int gather_nt = 1;      // non-temporal output stores
+  int fuse_count = 1;     // 1: row counts, their scan and the sampling of a hop share one launch
   int lds_dedup = 0;      // 1: hop_sample stages its probes through an LDS hash table
   int split_miss = 1;     // gather schedule, see launch_gather_seg
-  int use_graph = 1;      // lmi_run_once replays a captured HIP graph
+  int use_graph = 0;      // 1: lmi_run_once replays a captured HIP graph of the sampling kernels (measured
+                          // 2-3 % slower than plain launches here: the host enqueues a batch in 85 us,
+                          // well inside its 205 us of device time, and a graph's end costs 9 us)
   int miss_blocks = 32;   // grid of the host-link gather: enough reads in flight to fill the link, few enough
                           // not to crowd HBM traffic out of the memory pipeline
   int miss_unroll = 1;    // rows in flight per lane in the host-link gather
   // profiling
-  bool prof_on = false;
+  bool prof_on = false;                 // any level: device row counters are kept
+  int prof_level = 0;                   // 0 off, 1 every phase bracketed, 2 only the gather kernels
   std::vector<EventPair> prof_events;   // recorded, not yet resolved
   std::vector<hipEvent_t> prof_used;    // every event recorded since the last read (pairs may share one)
   std::vector<hipEvent_t> prof_free;    // recycled events
@@ -186,7 +190,7 @@ int prof_begin(Server *s, hipStream_t st, int kind);
 int prof_end(Server *s, hipStream_t st, int handle);
 // One event closes the pair left open on the caller's stream and opens the next
 // phase (next_kind < 0: only close), so a batch costs one event per phase boundary.
-void prof_phase(Server *s, hipStream_t st, int *open, int next_kind);
+hipEvent_t prof_phase(Server *s, hipStream_t st, int *open, int next_kind);
 
 // sampler.hip
 // stage_seeds: also run the seed-staging kernel now (otherwise hop 0 stages them itself)
@@ -209,5 +213,13 @@ int pipe_join(Pipe &p, hipStream_t st);  // make `st` wait for the pipe's side-s
 int cache_dump(Server *s, int32_t *slot_of, int64_t n, int32_t *aux);
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
+
+// Nodes per block of the fused count-and-sample kernel for a hop of at most n_max nodes
+// sampled G lanes per node: a small hop takes one node per lane group (more, smaller tiles
+// keep every CU busy), a large one a full wavefront of nodes.
+inline int hop_tile_nodes(int64_t n_max, int G) {
+  const int per_pass = 256 / G;
+  return (n_max <= 32768 && per_pass < 64) ? per_pass : 64;
+}
 
 }  // namespace lmi

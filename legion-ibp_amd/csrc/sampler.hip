@@ -302,6 +302,116 @@ static __global__ __launch_bounds__(256) void hop_sample_lds_kernel(HopArgs a) {
   }
 }
 
+// ------------------------------------------------- hop, phases 1 and 2 in one launch
+// One tile of NPB nodes per block.  Wavefront 0 loads the tile's row pointers, scans
+// min(deg, fanout) across its lanes and obtains the tile's edge offset by look-back
+// over the earlier tiles; then the whole block samples the tile's nodes, G lanes per
+// node, from the row bounds kept in LDS.  Same outputs as hop_count_scan_kernel
+// followed by hop_sample_kernel, one launch and one row-pointer read less.
+template <int G, int NPB>
+static __global__ __launch_bounds__(256) void hop_count_sample_kernel(HopArgs a) {
+  static_assert(NPB <= kWave && NPB >= 256 / G, "tile = one wavefront of nodes at most, one pass at least");
+  __shared__ int32_t s_id[NPB];
+  __shared__ int64_t s_beg[NPB], s_deg[NPB];
+  __shared__ int s_row[NPB];
+  __shared__ int s_prefix;
+  DevState *st = a.st;
+  const int64_t flat = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  scan_chain_reset(a.chain_edges, a.max_tiles, flat, (int64_t)gridDim.x * blockDim.x);
+  const int n_prev = st->node_counter[9 + a.hop];
+  const int n_tiles = (n_prev + NPB - 1) / NPB;
+  if (n_tiles == 0) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+      a.row_ptr[0] = 0;
+      scan_epilogue(SCAN_EPI_HOP_EDGES, st, a.hop, 0);
+    }
+    return;
+  }
+  const int tile = blockIdx.x;
+  if (tile >= n_tiles) return;
+  // ---- counts, tile scan (wavefront 0)
+  const int t = threadIdx.x;
+  const int my = tile * NPB + t;
+  int cnt = 0, ex = 0, total = 0;
+  int32_t id = -1;
+  int64_t lo = 0, hi = 0;
+  if (t < kWave) {
+    if (t < NPB && my < n_prev) {
+      if (a.stage_seeds) {
+        id = st->seeds[my];
+        a.ids[my] = id;
+        a.labels[my] = st->labels_in ? st->labels_in[my] : -1;
+      } else {
+        id = a.ids[my];
+      }
+      if (id < 0 || id >= a.n_nodes) {
+        if (a.stage_seeds) st->bad_id = 1;
+        id = -1;
+      }
+    }
+    if (id >= 0) {
+      lo = a.indptr[id];
+      hi = a.indptr[id + 1];
+      if (a.stage_seeds) table_insert_min(a.slots, a.log2cap, id, my);
+    }
+    const int64_t deg = hi - lo;
+    cnt = (int)(deg < (int64_t)a.fanout ? deg : (int64_t)a.fanout);
+    const int inc = wave_inclusive_scan(cnt);
+    ex = inc - cnt;
+    total = __shfl(inc, kWave - 1, kWave);
+  }
+  const int prefix = scan_tile_prefix(a.chain_nodes, tile, total, &s_prefix, &st->scan_fault);
+  if (t < NPB) {
+    s_id[t] = id;
+    s_beg[t] = lo;
+    s_deg[t] = hi - lo;
+    s_row[t] = prefix + ex;
+    if (my < n_prev) a.row_ptr[my] = prefix + ex;
+  }
+  if (tile == n_tiles - 1 && t == 0) {
+    a.row_ptr[n_prev] = prefix + total;
+    scan_epilogue(SCAN_EPI_HOP_EDGES, st, a.hop, prefix + total);
+  }
+  __syncthreads();
+  // ---- sampling: the edge offset of the hop is fixed by the hops before it
+  const uint64_t seed = (uint64_t)st->rng_lo | ((uint64_t)st->rng_hi << 32);
+  const int eoff = (a.hop == 0) ? 0 : st->edge_counter[12 + a.hop] + st->edge_counter[9 + a.hop];
+  const int fanout = a.fanout;
+  const int lane = t & (G - 1);
+  for (int q = t / G; q < NPB; q += 256 / G) {
+    const int i = tile * NPB + q;
+    if (i >= n_prev) break;
+    const int32_t v = s_id[q];
+    if (v < 0) continue;
+    const int64_t beg = s_beg[q], deg = s_deg[q];
+    const int base = s_row[q];
+    int64_t pick = lane;
+    int count;
+    if (deg <= (int64_t)fanout) {
+      count = (int)deg;
+    } else {
+      count = fanout;
+      const uint32_t j = (uint32_t)(deg - fanout) + (uint32_t)lane;
+      uint32_t d = 0xFFFFFFFFu;
+      if (lane < fanout) d = __umulhi(sample_draw(seed, (uint32_t)a.hop, (uint32_t)v, (uint32_t)lane), j + 1u);
+      bool dup = false;
+      for (int r = 0; r + 1 < fanout; ++r) {
+        const uint32_t mine = dup ? j : d;
+        const uint32_t p = __shfl(mine, r, G);
+        if (lane > r && d == p) dup = true;
+      }
+      pick = dup ? j : d;
+    }
+    if (lane < count) {
+      const int32_t nbr = a.indices[beg + pick];
+      const int e = base + lane;
+      a.agg_src_ids[eoff + e] = nbr;
+      a.agg_dst_off[eoff + e] = i;
+      a.eslot[e] = (int)table_insert_min(a.slots, a.log2cap, nbr, n_prev + e);
+    }
+  }
+}
+
 // ------------------------------------------------------------- hop, phase 3
 // firstv[e] = table value of the edge's source; an edge is the first occurrence
 // of a new node iff that value names the edge itself.  rank[e] = number of first
@@ -442,6 +552,27 @@ int launch_hop(Server *s, Pipe &p, hipStream_t st, int hop, bool stage_seeds) {
   a.chain_edges = chain_of(p, 1);
   a.max_tiles = p.max_tiles;
   a.stage_seeds = (hop == 0 && stage_seeds) ? 1 : 0;
+  int G = 4;
+  while (G < f) G <<= 1;
+  const bool fused = s->fuse_count && !s->lds_dedup;
+  if (fused) {
+    // counts, scan and sampling in one launch, one tile of nodes per block
+    const int npb = hop_tile_nodes(n_max, G);
+    const int grid = (int)ceil_div(std::max<int64_t>(n_max, 1), npb);
+#define LMI_FUSED(GG)                                                                                   \
+  if (npb == 64)                                                                                        \
+    hipLaunchKernelGGL((hop_count_sample_kernel<GG, 64>), dim3(grid), dim3(256), 0, st, a);             \
+  else                                                                                                  \
+    hipLaunchKernelGGL((hop_count_sample_kernel<GG, (256 / GG)>), dim3(grid), dim3(256), 0, st, a);
+    switch (G) {
+      case 4: LMI_FUSED(4) break;
+      case 8: LMI_FUSED(8) break;
+      case 16: LMI_FUSED(16) break;
+      case 32: LMI_FUSED(32) break;
+      default: LMI_FUSED(64) break;
+    }
+#undef LMI_FUSED
+  } else {
   // one tile per block (blocks past the real item count leave at once); few items per
   // thread while that keeps the tile count near a thousand: the row-pointer reads are
   // dependent random accesses, so parallelism matters more than per-thread work
@@ -454,8 +585,6 @@ int launch_hop(Server *s, Pipe &p, hipStream_t st, int hop, bool stage_seeds) {
     hipLaunchKernelGGL(hop_count_scan_kernel<4>, dim3((int)ceil_div(nm, kScanBlock * 4)), dim3(kScanBlock), 0, st, a);
   else
     hipLaunchKernelGGL(hop_count_scan_kernel<8>, dim3((int)ceil_div(nm, kScanBlock * 8)), dim3(kScanBlock), 0, st, a);
-  int G = 4;
-  while (G < f) G <<= 1;
   const int grid = (int)std::min<int64_t>(ceil_div(n_max * G, 256), 8192);
   if (s->lds_dedup) {
     switch (G) {
@@ -472,6 +601,7 @@ int launch_hop(Server *s, Pipe &p, hipStream_t st, int hop, bool stage_seeds) {
     case 16: hipLaunchKernelGGL(hop_sample_kernel<16>, dim3(grid), dim3(256), 0, st, a); break;
     case 32: hipLaunchKernelGGL(hop_sample_kernel<32>, dim3(grid), dim3(256), 0, st, a); break;
     default: hipLaunchKernelGGL(hop_sample_kernel<64>, dim3(grid), dim3(256), 0, st, a); break;
+  }
   }
   const int64_t em = std::max<int64_t>(e_max, 1);
   if (em <= 1024 * 1024)

@@ -70,6 +70,7 @@ def test_lds_staged_dedup_gives_the_same_batches(lmi, oracle, fanout):
     stream = lmi.stream_create()
     try:
         srv.tune("lds_dedup", 1)
+        srv.tune("use_graph", 1)
         srv.load_graph(indptr, indices)
         srv.attach_features(feats)
         for it in range(4):
@@ -77,6 +78,32 @@ def test_lds_staged_dedup_gives_the_same_batches(lmi, oracle, fanout):
             st = stream if it % 2 else None          # graph replay and eager
             srv.run_once(seeds, rng_seed=40 + it, stream=st)
             assert_batch_equal(srv.fetch(stream=st), oracle.sample_batch(indptr, indices, seeds, fanout, 40 + it))
+    finally:
+        srv.close()
+        feats.free()
+
+
+@pytest.mark.parametrize("fused", [1, 0])
+@pytest.mark.parametrize("batch,fanout", [(96, [25, 10]), (1800, [20, 5]), (700, [64, 2]), (300, [3, 4, 3])])
+def test_count_and_sample_in_one_launch_or_two(lmi, oracle, batch, fanout, fused):
+    """Both launch shapes of a hop (row counts + scan + sampling fused, or two launches), with
+    small tiles (one node per lane group) and full 64-node tiles, against the oracle."""
+    rng = np.random.default_rng(batch + fused)
+    n_nodes = 6000
+    indptr, indices = random_graph(rng, n_nodes, 18, zero_frac=0.1, hubs=6, hub_deg=700)
+    feats = make_features(lmi, rng, n_nodes, 4)
+    srv = lmi.Server(batch, fanout, 4)
+    stream = lmi.stream_create()
+    try:
+        srv.tune("fuse_count", fused)
+        srv.tune("use_graph", 1)
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        for it in range(3):
+            seeds = rng.choice(n_nodes, batch if it < 2 else batch // 3, replace=False).astype(np.int32)
+            st = stream if it % 2 else None          # graph replay and eager
+            srv.run_once(seeds, rng_seed=7 + it, stream=st)
+            assert_batch_equal(srv.fetch(stream=st), oracle.sample_batch(indptr, indices, seeds, fanout, 7 + it))
     finally:
         srv.close()
         feats.free()
@@ -331,6 +358,7 @@ def test_graph_replay_matches_eager_and_oracle(lmi, oracle, cache, schedule):
     lru = oracle.Lru(128, 4, dim * 4)
     try:
         srv.tune("split_miss", schedule)   # where the HBM and host-link gathers run (caller / side stream)
+        srv.tune("use_graph", 1)           # batches on a real stream replay a captured graph
         srv.load_graph(indptr, indices)
         srv.attach_features(feats)
         srv.load_idset(lmi.MODE_TRAIN, train)
@@ -432,6 +460,7 @@ def test_rebuilding_cache_or_graph_after_graph_capture(lmi, oracle):
     stream = lmi.stream_create()
     seeds = rng.choice(n_nodes, batch, replace=False).astype(np.int32)
     try:
+        srv.tune("use_graph", 1)
         srv.load_graph(indptr, indices)
         srv.attach_features(feats)
         for step, (cap, table, gp, gi) in enumerate([(500, lmi.TABLE_HASH, indptr, indices),
