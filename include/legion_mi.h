@@ -143,6 +143,10 @@ int lmi_features_attach(lmi_server *s, const void *rows, int64_t n_rows, int loc
  * labels may be NULL.  Always copied into HBM. */
 int lmi_idset_load(lmi_server *s, int mode, const int32_t *ids, const int32_t *labels,
                    int64_t n, int location);
+/* Ids per batch of id set `mode` when batches are sliced from the set (1 .. batch_size;
+ * default batch_size).  The reference serves validation and test batches of their own
+ * size (GetCurrentBatchsize, engine/ipc_service.cu:228-236). */
+int lmi_idset_batch(lmi_server *s, int mode, int32_t ids_per_batch);
 
 /* ---- presampling (GPUServer::PreSc + PreSCCacheController, engine/server.cu:94-122,
  *      cache/cache.cu:43-71) ------------------------------------------------------ */
@@ -209,7 +213,9 @@ int lmi_batch_view_get(lmi_server *s, int pipe, lmi_batch_view *out);
 /* Synchronises `stream`, copies both headers to the host, reports a bad seed id. */
 int lmi_batch_counters(lmi_server *s, int pipe, void *stream, int32_t node_counter[16],
                        int32_t edge_counter[16]);
-/* Steps per epoch of an id set: ceil(size / batch_size) (engine/ipc_service.cu:60-128). */
+/* Batches an id set holds: ceil(size / ids per batch).  The reference's own step counts
+ * (Coordinate, engine/ipc_service.cu:60-128: it drops the training set's last batch)
+ * are computed by the host layer above this ABI. */
 int lmi_steps_per_epoch(lmi_server *s, int mode, int32_t *steps);
 
 /* ---- measurement ------------------------------------------------------- */

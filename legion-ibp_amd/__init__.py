@@ -27,7 +27,7 @@ ABI_SYMBOLS = [
     "lmi_host_alloc", "lmi_host_free", "lmi_device_alloc", "lmi_device_free",
     "lmi_copy_to_host", "lmi_copy_to_device", "lmi_stream_create", "lmi_stream_destroy",
     "lmi_stream_sync", "lmi_device_sync", "lmi_graph_load", "lmi_features_attach",
-    "lmi_idset_load", "lmi_presample", "lmi_op_hotness", "lmi_presample_reset", "lmi_hotness_dump",
+    "lmi_idset_load", "lmi_idset_batch", "lmi_presample", "lmi_op_hotness", "lmi_presample_reset", "lmi_hotness_dump",
     "lmi_cache_policy", "lmi_cache_build_static", "lmi_cache_build_lru", "lmi_cache_build_int8",
     "lmi_cache_info_get", "lmi_cache_dump", "lmi_op_batch_generate", "lmi_op_random_sample",
     "lmi_op_cache_lookup", "lmi_op_io_submit", "lmi_op_io_complete", "lmi_run_once",
@@ -97,6 +97,7 @@ def lib():
         L.lmi_graph_load.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int]
         L.lmi_features_attach.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
         L.lmi_idset_load.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
+        L.lmi_idset_batch.argtypes = [C.c_void_p, C.c_int, C.c_int32]
         L.lmi_presample.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_int, C.c_int32, C.c_int32]
         L.lmi_op_hotness.argtypes = [C.c_void_p, C.c_int, C.c_void_p]
         L.lmi_presample_reset.argtypes = [C.c_void_p]
@@ -212,6 +213,10 @@ class Server:
             labels = np.ascontiguousarray(labels, dtype=np.int32)
             lp = labels.ctypes.data
         check(lib().lmi_idset_load(self.h, mode, ids.ctypes.data, lp, len(ids), LOC_HOST))
+
+    def idset_batch(self, mode, ids_per_batch):
+        """Ids per sliced batch of id set `mode` (default: the server's batch size)."""
+        check(lib().lmi_idset_batch(self.h, mode, ids_per_batch))
 
     # presampling -------------------------------------------------------------
     def presample(self, n_batches, first_batch=0, mode=MODE_TRAIN, pipe=0, stream=None):

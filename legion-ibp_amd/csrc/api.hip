@@ -140,7 +140,7 @@ static int pipe_alloc(Server *s, Pipe &p) {
   for (int k = 0; k < s->cfg.hops; ++k) {
     int G = 4;
     while (G < s->cfg.fanout[k]) G <<= 1;
-    tiles = std::max(tiles, ceil_div(s->node_cap[k], (int64_t)hop_tile_nodes(s->node_cap[k], G)));
+    tiles = std::max(tiles, ceil_div(s->node_cap[k], (int64_t)std::min(64, 256 / G)));  // smallest tile
   }
   p.max_tiles = (int32_t)tiles + 1;
   LMI_TRY(dmalloc(&p.chain_status[0], p.max_tiles));
@@ -476,9 +476,10 @@ static int batch_params(Server *s, Pipe &p, hipStream_t st, const int32_t *seeds
     // slice `batch_counter` of the id set (batch_generate, operator_impl.cu:40-53); a short last
     // batch is shortened rather than padded with -1
     if (mode < 0 || mode > 2 || !s->set_ids[mode]) LMI_FAIL(LMI_ERR_STATE, "id set %d not loaded", mode);
-    const int64_t off = (int64_t)batch_counter * s->cfg.batch_size;
+    const int32_t per = s->set_batch[mode] ? s->set_batch[mode] : s->cfg.batch_size;
+    const int64_t off = (int64_t)batch_counter * per;
     if (batch_counter < 0 || off >= s->set_n[mode]) LMI_FAIL(LMI_ERR_ARG, "batch %d is past the end of id set %d", batch_counter, mode);
-    n = (int32_t)std::min<int64_t>(s->cfg.batch_size, s->set_n[mode] - off);
+    n = (int32_t)std::min<int64_t>(per, s->set_n[mode] - off);
     bp->seeds = s->set_ids[mode] + off;
     if (s->set_labels[mode]) bp->labels = s->set_labels[mode] + off;
   }
@@ -671,10 +672,19 @@ int lmi_batch_counters(lmi_server *h, int pipe, void *stream, int32_t node_count
   return LMI_OK;
 }
 
+int lmi_idset_batch(lmi_server *h, int mode, int32_t ids_per_batch) {
+  Server *s = reinterpret_cast<Server *>(h);
+  if (!s || mode < 0 || mode > 2) LMI_FAIL(LMI_ERR_ARG, "bad argument");
+  if (ids_per_batch < 1 || ids_per_batch > s->cfg.batch_size)
+    LMI_FAIL(LMI_ERR_CAPACITY, "%d ids per batch outside 1..%d", ids_per_batch, s->cfg.batch_size);
+  s->set_batch[mode] = ids_per_batch;
+  return LMI_OK;
+}
+
 int lmi_steps_per_epoch(lmi_server *h, int mode, int32_t *steps) {
   Server *s = reinterpret_cast<Server *>(h);
   if (!s || !steps || mode < 0 || mode > 2) LMI_FAIL(LMI_ERR_ARG, "bad argument");
-  *steps = (int32_t)ceil_div(s->set_n[mode], s->cfg.batch_size);
+  *steps = (int32_t)ceil_div(s->set_n[mode], s->set_batch[mode] ? s->set_batch[mode] : s->cfg.batch_size);
   return LMI_OK;
 }
 
@@ -730,6 +740,7 @@ int lmi_tune(lmi_server *h, const char *key, int64_t value) {
   else if (!strcmp(key, "gather_nontemporal")) s->gather_nt = (int)value;
   else if (!strcmp(key, "lds_dedup")) s->lds_dedup = (int)value;
   else if (!strcmp(key, "fuse_count")) s->fuse_count = (int)value;
+  else if (!strcmp(key, "fuse_small_max")) s->fuse_small_max = value;
   else if (!strcmp(key, "split_miss")) s->split_miss = (int)value;
   else if (!strcmp(key, "use_graph")) s->use_graph = (int)value;
   else if (!strcmp(key, "miss_blocks")) s->miss_blocks = (int)value;

@@ -135,6 +135,7 @@ struct Server {
   int32_t *set_ids[3] = {nullptr, nullptr, nullptr};
   int32_t *set_labels[3] = {nullptr, nullptr, nullptr};
   int64_t set_n[3] = {0, 0, 0};
+  int32_t set_batch[3] = {0, 0, 0};  // ids per sliced batch; 0 = cfg.batch_size
   // cache
   int policy = LMI_POLICY_DEGREE;    // ranking key of the static / int8 hot set
   uint32_t *hot = nullptr;           // [n_nodes] presampling appearance counts
@@ -160,6 +161,7 @@ struct Server {
   int gather_unroll = 1;  // rows in flight per lane (1 measured best: 62.5 % of HBM peak vs 60 % at 4)
   int gather_blocks = 0;  // 0 = auto
   int gather_nt = 1;      // non-temporal output stores
+  int64_t fuse_small_max = 32768;  // hops of at most this many nodes use the small tile of hop_tile_nodes
   int fuse_count = 1;     // 1: row counts, their scan and the sampling of a hop share one launch
   int lds_dedup = 0;      // 1: hop_sample stages its probes through an LDS hash table
   int split_miss = 1;     // gather schedule, see launch_gather_seg
@@ -217,9 +219,9 @@ inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }
 // Nodes per block of the fused count-and-sample kernel for a hop of at most n_max nodes
 // sampled G lanes per node: a small hop takes one node per lane group (more, smaller tiles
 // keep every CU busy), a large one a full wavefront of nodes.
-inline int hop_tile_nodes(int64_t n_max, int G) {
+inline int hop_tile_nodes(int64_t n_max, int G, int64_t small_max = 32768) {
   const int per_pass = 256 / G;
-  return (n_max <= 32768 && per_pass < 64) ? per_pass : 64;
+  return (n_max <= small_max && per_pass < 64) ? per_pass : 64;
 }
 
 }  // namespace lmi

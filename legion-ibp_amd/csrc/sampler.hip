@@ -557,7 +557,7 @@ int launch_hop(Server *s, Pipe &p, hipStream_t st, int hop, bool stage_seeds) {
   const bool fused = s->fuse_count && !s->lds_dedup;
   if (fused) {
     // counts, scan and sampling in one launch, one tile of nodes per block
-    const int npb = hop_tile_nodes(n_max, G);
+    const int npb = hop_tile_nodes(n_max, G, s->fuse_small_max);
     const int grid = (int)ceil_div(std::max<int64_t>(n_max, 1), npb);
 #define LMI_FUSED(GG)                                                                                   \
   if (npb == 64)                                                                                        \

@@ -7,6 +7,7 @@
 //   engine/operator.cu:10-150   operator classes forwarding to the extern "C" layer
 //   storage/storage_management.cu:33-279   ./meta_config + dataset files
 #include "legion_host.hpp"
+#include "ipc_service.hpp"
 
 #include <sys/mman.h>
 #include <sys/stat.h>
@@ -14,6 +15,9 @@
 #include <unistd.h>
 
 #include <chrono>
+#include <condition_variable>
+#include <mutex>
+#include <thread>
 #include <cstdio>
 #include <cstdlib>
 #include <cstring>
@@ -116,7 +120,13 @@ class GPURunner : public Runner {
  public:
   void Initialize(RunnerParams *params) override {
     hops_ = (int)params->fanout.size();
+    device_ = params->device_id;
     LMI_MUST(lmi_stream_create(&stream_));
+    if (IPCEnv *ipc = (IPCEnv *)params->ipc) {  // engine/server.cu:256
+      lmi_batch_view v;
+      LMI_MUST(lmi_batch_view_get((lmi_server *)params->env, 0, &v));
+      ipc->InitializeSamplesBuffer(ipc->GetRawBatchsize(), (int32_t)v.max_nodes, 0, device_, LEGION_INTERBATCH_CON);
+    }
     // slot table: [BatchGen, Lookup, IOSubmit, (Sample, Lookup, IOSubmit) x hops, IOComplete]
     ops_.push_back(NewBatchGenerateOP(0));
     ops_.push_back(NewCacheLookupOP(1));
@@ -141,19 +151,39 @@ class GPURunner : public Runner {
       o.neighbor_count = (i % 3 == 0 && hop >= 0 && hop < hops_) ? params->fanout[hop] : 0;
     }
   }
-  void InitializeFeaturesBuffer(RunnerParams *) override {}
-  void RunPreSc(RunnerParams *params) override { run_table(params, true); }
-  void RunOnce(RunnerParams *params) override {
+  void InitializeFeaturesBuffer(RunnerParams *params) override {  // engine/server.cu:303-308
+    if (IPCEnv *ipc = (IPCEnv *)params->ipc) {
+      lmi_batch_view v;
+      LMI_MUST(lmi_batch_view_get((lmi_server *)params->env, 0, &v));
+      ipc->InitializeFeaturesBuffer(0, (int32_t)v.max_nodes, params->feature_dim, device_, LEGION_INTERBATCH_CON);
+    }
+  }
+  void RunPreSc(RunnerParams *params) override { run_table(params, params->global_batch_id, LMI_MODE_TRAIN, true); }
+  void RunOnce(RunnerParams *params) override {  // engine/server.cu:330-400
+    IPCEnv *ipc = (IPCEnv *)params->ipc;
+    int mode = params->mode, local = params->global_batch_id;
+    if (ipc) {
+      mode = ipc->GetCurrentMode(params->global_batch_id);
+      local = ipc->GetLocalBatchId(params->global_batch_id);
+    }
     pipe_ ^= 1;  // two output buffer sets, as INTERBATCH_CON = 2
+    ran_ = true;
+    if (ipc) ipc->IPCWait(device_, pipe_);  // until the trainer has released this buffer set
     if (params->fused) {
-      LMI_MUST(lmi_run_once((lmi_server *)params->env, pipe_, stream_, nullptr, 0, LMI_LOC_DEVICE,
-                            params->global_batch_id, params->mode, 0));
+      LMI_MUST(lmi_run_once((lmi_server *)params->env, pipe_, stream_, nullptr, 0, LMI_LOC_DEVICE, local, mode, 0));
     } else {
-      run_table(params, false);
+      run_table(params, local, mode, false);
     }
     LMI_MUST(lmi_batch_wait((lmi_server *)params->env, pipe_, stream_));
+    if (ipc && ipc->HandoffEnabled()) {
+      LMI_MUST(lmi_stream_sync(stream_));  // the batch is complete before the trainer is told
+      ipc->IPCPost(device_, pipe_);
+    }
   }
-  void Finalize(RunnerParams *) override {
+  void Finalize(RunnerParams *params) override {
+    // the trainer must have released the last batch before its buffers go away
+    if (IPCEnv *ipc = (IPCEnv *)params->ipc)
+      if (ran_) ipc->IPCWait(device_, pipe_);
     if (stream_) {
       LMI_MUST(lmi_stream_sync(stream_));
       LMI_MUST(lmi_stream_destroy(stream_));
@@ -166,17 +196,18 @@ class GPURunner : public Runner {
   void *Stream() const override { return stream_; }
 
  private:
-  void run_table(RunnerParams *params, bool presc) {
+  void run_table(RunnerParams *, int local_batch_id, int mode, bool presc) {
     for (size_t i = 0; i < ops_.size(); ++i) {
       OpParams &o = op_params_[i];
       o.pipe = pipe_;
-      o.global_batch_id = params->global_batch_id;
-      o.mode = params->mode;
+      o.global_batch_id = local_batch_id;
+      o.mode = mode;
       o.is_presc = presc;
       ops_[i]->run(&o);
     }
   }
-  int hops_ = 0, pipe_ = 1;
+  int hops_ = 0, pipe_ = 1, device_ = 0;
+  bool ran_ = false;
   void *stream_ = nullptr;
   std::vector<Operator *> ops_;
   std::vector<OpParams> op_params_;
@@ -191,7 +222,8 @@ class GPUServer : public Server {
       std::exit(EXIT_FAILURE);
     }
     std::string err;
-    if (!LegionReadMetaConfig("./meta_config", &meta_, &err)) {
+    const char *meta_path = std::getenv("LEGION_MI_META_CONFIG");
+    if (!LegionReadMetaConfig(meta_path ? meta_path : "./meta_config", &meta_, &err)) {
       std::fprintf(stderr, "%s\n", err.c_str());
       std::exit(EXIT_FAILURE);
     }
@@ -236,7 +268,24 @@ class GPUServer : public Server {
           if (ids[i] >= 0 && ids[i] < meta_.node_num) lab[i] = labels[ids[i]];
       LMI_MUST(lmi_idset_load(h_, m, ids.data(), have_labels ? lab.data() : nullptr, counts[m], LMI_LOC_HOST));
     }
+    // schedule and hand-off (storage_management.cu builds the IPCEnv and calls Coordinate)
+    ipc_ = NewIPCEnv(1);
+    ipc_->EnableHandoff(handoff_ || std::getenv("LEGION_MI_HANDOFF") != nullptr);
+    ipc_->SetWaitSeconds(wait_seconds_);
+    BuildInfo info;
+    info.partition_count = 1;
+    info.training_set_num = {(int32_t)meta_.training_set_num};
+    info.validation_set_num = {(int32_t)meta_.validation_set_num};
+    info.testing_set_num = {(int32_t)meta_.testing_set_num};
+    info.epoch = meta_.epoch;
+    info.raw_batch_size = meta_.batch_size;
+    ipc_->Coordinate(&info);
+    for (int m = LMI_MODE_VALID; m <= LMI_MODE_TEST; ++m)
+      if (ipc_->GetCurrentBatchsize(0, m) > 0) LMI_MUST(lmi_idset_batch(h_, m, ipc_->GetCurrentBatchsize(0, m)));
+    ipc_->BindServer(0, h_);
     runner_ = NewGPURunner();
+    params_.ipc = ipc_;
+    params_.feature_dim = meta_.feature_dim;
     params_.device_id = 0;
     params_.fanout = fanout;
     params_.cache = params_.graph = params_.feature = nullptr;
@@ -264,9 +313,9 @@ class GPUServer : public Server {
         params_.global_batch_id = i;
         runner_->RunPreSc(&params_);
       }
-      runner_->InitializeFeaturesBuffer(&params_);
       LMI_MUST(lmi_cache_policy(h_, LMI_POLICY_PRESAMPLED));
     }
+    runner_->InitializeFeaturesBuffer(&params_);  // engine/server.cu:36
     if (dyn_cache_ & LEGION_DYN_COMP) {
       const int64_t rows = std::max<int64_t>(1, meta_.cache_memory / (meta_.feature_dim + 4));
       LMI_MUST(lmi_cache_build_int8(h_, rows, LMI_TABLE_RANK));
@@ -284,22 +333,19 @@ class GPUServer : public Server {
     std::cout << "System is ready for serving\n";  // the line the reference's scripts wait for
   }
 
-  void Run() override {
-    int32_t steps = 0;
-    LMI_MUST(lmi_steps_per_epoch(h_, LMI_MODE_TRAIN, &steps));
+  void Run() override {  // engine/server.cu:124-135
+    const int32_t max_step = ipc_->GetMaxStep();
     const auto t0 = std::chrono::steady_clock::now();
     int64_t batches = 0;
-    for (int e = 0; e < meta_.epoch; ++e) {
-      for (int i = 0; i < steps; ++i) {
-        params_.global_batch_id = i;
-        runner_->RunOnce(&params_);
-        if (sink_) {
-          lmi_batch_view v;
-          LMI_MUST(lmi_batch_view_get(h_, runner_->CurrentPipe(), &v));
-          sink_(&v, 0, runner_->CurrentPipe(), runner_->Stream(), sink_user_);
-        }
-        ++batches;
+    for (int32_t batch_id = 0; batch_id < max_step; ++batch_id) {
+      params_.global_batch_id = batch_id;
+      runner_->RunOnce(&params_);
+      if (sink_) {
+        lmi_batch_view v;
+        LMI_MUST(lmi_batch_view_get(h_, runner_->CurrentPipe(), &v));
+        sink_(&v, 0, runner_->CurrentPipe(), runner_->Stream(), sink_user_);
       }
+      ++batches;
     }
     LMI_MUST(lmi_stream_sync(runner_->Stream()));
     const double sec = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
@@ -313,6 +359,11 @@ class GPUServer : public Server {
       delete runner_;
       runner_ = nullptr;
     }
+    if (ipc_) {
+      ipc_->Finalize();
+      delete ipc_;
+      ipc_ = nullptr;
+    }
     if (h_) LMI_MUST(lmi_server_destroy(h_));
     h_ = nullptr;
     if (host_features_) LMI_MUST(lmi_host_free(host_features_));
@@ -323,6 +374,10 @@ class GPUServer : public Server {
     sink_ = sink;
     sink_user_ = user;
   }
+  void EnableHandoff(bool on, double wait_seconds) override {
+    handoff_ = on;
+    wait_seconds_ = wait_seconds;
+  }
   lmi_server *Handle(int) override { return h_; }
 
  private:
@@ -332,6 +387,9 @@ class GPUServer : public Server {
   lmi_server *h_ = nullptr;
   void *host_features_ = nullptr;
   Runner *runner_ = nullptr;
+  IPCEnv *ipc_ = nullptr;
+  bool handoff_ = false;
+  double wait_seconds_ = 600.0;
   RunnerParams params_{};
   LegionBatchSink sink_ = nullptr;
   void *sink_user_ = nullptr;
@@ -372,3 +430,47 @@ Operator *NewRandomSampleOP(int op_id) { return new RandomSampleOP(op_id); }
 Operator *NewCacheLookupOP(int op_id) { return new CacheLookupOP(op_id); }
 Operator *NewSSDIOSubmitOP(int op_id) { return new SSDIOSubmitOP(op_id); }
 Operator *NewSSDIOCompleteOP(int op_id) { return new SSDIOCompleteOP(op_id); }
+
+// ------------------------------------------------- server on a background thread
+namespace {
+struct Background {
+  std::thread thread;
+  std::mutex mu;
+  std::condition_variable cv;
+  bool ready = false;
+  bool started = false;
+};
+Background g_bg;
+}  // namespace
+
+extern "C" int legion_server_start(int gpu_number, int cache_agg_mode, int dyn_cache, const int32_t *fanout,
+                                   int hops, int handoff, double wait_seconds) {
+  if (g_bg.started || !fanout || hops < 1) return -1;
+  std::vector<int> fan(fanout, fanout + hops);
+  g_bg.ready = false;
+  g_bg.started = true;
+  g_bg.thread = std::thread([=]() {
+    Server *server = NewGPUServer();
+    server->EnableHandoff(handoff != 0, wait_seconds);
+    server->Initialize(gpu_number, fan, 1, dyn_cache);
+    server->PreSc(cache_agg_mode);
+    {
+      std::lock_guard<std::mutex> lock(g_bg.mu);
+      g_bg.ready = true;
+    }
+    g_bg.cv.notify_all();
+    server->Run();
+    server->Finalize();
+    delete server;
+  });
+  std::unique_lock<std::mutex> lock(g_bg.mu);
+  g_bg.cv.wait(lock, [] { return g_bg.ready; });
+  return 0;
+}
+
+extern "C" int legion_server_join(void) {
+  if (!g_bg.started) return -1;
+  g_bg.thread.join();
+  g_bg.started = false;
+  return 0;
+}

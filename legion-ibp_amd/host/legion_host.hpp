@@ -18,8 +18,13 @@
 //   * `dyn_cache` keeps the reference's bit meaning where a counterpart exists:
 //     0 = static hot-set cache, DYN_ENABLE (1) = LRU dynamic cache,
 //     DYN_COMP (8) = compressed (int8) cache; other bits are ignored;
-//   * the hand-off to a trainer is a callback (SetBatchSink) instead of CUDA IPC +
-//     POSIX semaphores; the buffers it receives are the reference's output contract.
+//   * Run() serves the reference's schedule (per epoch the training steps, then the
+//     validation steps; the test steps after the last epoch; engine/server.cu:124-135,
+//     engine/ipc_service.cu:60-128,212-260);
+//   * the hand-off to a trainer is a callback (SetBatchSink) and, once EnableHandoff(true)
+//     was called, the reference's shared-memory slab + two named semaphores per output
+//     buffer set (ipc_service.hpp) towards a consumer in the same process; the buffers
+//     either receives are the reference's output contract.
 #pragma once
 
 #include <cstdint>
@@ -44,6 +49,11 @@ struct RunnerParams {
   // additions (defaulted, so reference-style aggregate use still works)
   bool fused = false;  // true: RunOnce calls lmi_run_once instead of the operator table
   int mode = LMI_MODE_TRAIN;
+  int feature_dim = 0;
+  void *ipc = nullptr;  // IPCEnv* (ipc_service.hpp; the reference passes it in `env`).  When set,
+                        // global_batch_id counts over the whole schedule and the mode and the
+                        // batch's place in its id set come from it; when null, global_batch_id
+                        // is the place in id set `mode`.
 };
 
 // Called once per finished batch with the pipe's device buffers; the stream has
@@ -63,6 +73,9 @@ class Server {
   virtual void Finalize() = 0;
   // additions
   virtual void SetBatchSink(LegionBatchSink sink, void *user) = 0;
+  // Before Initialize: serve batches through the semaphore handshake of ipc_service.hpp,
+  // waiting at most wait_seconds for the trainer to release a buffer set.
+  virtual void EnableHandoff(bool on, double wait_seconds) = 0;
   virtual lmi_server *Handle(int device_id) = 0;
 };
 Server *NewGPUServer();
@@ -128,3 +141,11 @@ struct LegionMetaConfig {
   std::string feature_path;  // optional alternative directory for features / labels
 };
 bool LegionReadMetaConfig(const std::string &path, LegionMetaConfig *out, std::string *error);
+
+// A sampling server on a thread of the calling process, for a trainer that lives in the
+// same process (trainer_ipc.hpp): Initialize + PreSc run before the call returns, Run and
+// Finalize go on in the background.  The meta config is ./meta_config, or the file the
+// environment variable LEGION_MI_META_CONFIG names.  One server per process at a time.
+extern "C" int legion_server_start(int gpu_number, int cache_agg_mode, int dyn_cache, const int32_t *fanout,
+                                   int hops, int handoff, double wait_seconds);
+extern "C" int legion_server_join(void);  // waits for Run + Finalize; 0, or -1 if none was started

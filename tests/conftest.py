@@ -47,3 +47,16 @@ def random_graph(rng, n_nodes, mean_deg, hubs=0, hub_deg=0, zero_frac=0.1):
     indptr = np.concatenate([[0], np.cumsum(deg)]).astype(np.int64)
     indices = rng.integers(0, n_nodes, int(indptr[-1])).astype(np.int32)
     return indptr, indices
+
+
+def load_ipc_service():
+    """Import the trainer-side consumer module of the product package."""
+    name = "legion_ibp_amd_ipc_service"
+    if name in sys.modules:
+        return sys.modules[name]
+    path = os.path.join(ROOT, "legion-ibp_amd", "ipc_service.py")
+    spec = importlib.util.spec_from_file_location(name, path)
+    mod = importlib.util.module_from_spec(spec)
+    sys.modules[name] = mod
+    spec.loader.exec_module(mod)
+    return mod

@@ -216,6 +216,37 @@ def test_operator_chain_matches_run_once(lmi, oracle):
         feats.free()
 
 
+def test_id_set_sliced_at_its_own_batch_size(lmi, oracle):
+    """Validation / test sets are served in batches of their own size (the reference's
+    GetCurrentBatchsize): 130 ids at 40 a batch -> 40, 40, 40, 10."""
+    rng = np.random.default_rng(12)
+    n_nodes, batch, fanout, dim = 2000, 64, [5, 3], 8
+    indptr, indices = random_graph(rng, n_nodes, 8)
+    feats = make_features(lmi, rng, n_nodes, dim)
+    valid = rng.permutation(n_nodes)[:130].astype(np.int32)
+    labels = (valid % 5).astype(np.int32)
+    srv = lmi.Server(batch, fanout, dim, seed=3)
+    try:
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        srv.load_idset(lmi.MODE_VALID, valid, labels)
+        with pytest.raises(lmi.LegionError):
+            srv.idset_batch(lmi.MODE_VALID, batch + 1)   # more than the output buffers hold
+        with pytest.raises(lmi.LegionError):
+            srv.idset_batch(lmi.MODE_VALID, 0)
+        srv.idset_batch(lmi.MODE_VALID, 40)
+        for it in range(4):
+            srv.run_once(None, batch_counter=it, mode=lmi.MODE_VALID)
+            g = srv.fetch()
+            assert_batch_equal(g, oracle.sample_batch(indptr, indices, valid[it * 40:(it + 1) * 40], fanout, 3 + it))
+            np.testing.assert_array_equal(g.labels, labels[it * 40:(it + 1) * 40])
+        with pytest.raises(lmi.LegionError):
+            srv.run_once(None, batch_counter=4, mode=lmi.MODE_VALID)
+    finally:
+        srv.close()
+        feats.free()
+
+
 @pytest.mark.parametrize("n_sets,ways", [(64, 8), (16, 4), (1, 32), (500, 2)])
 def test_lru_cache_parity(lmi, oracle, n_sets, ways):
     """Reference-shaped toy workload (comp_cache/tests/test_cache.cu:4-9,48-53):

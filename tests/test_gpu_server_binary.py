@@ -30,6 +30,10 @@ def write_dataset(d, rng, n_nodes, dim, n_train):
     return indptr, indices, feats, train
 
 
+def read_sets(d):
+    return [np.fromfile(os.path.join(d, n), np.int32) for n in ("trainingset", "validationset", "testingset")]
+
+
 def read_dump(path, dim):
     raw = np.fromfile(path, np.int32)
     nc, ec = raw[:16], raw[16:32]
@@ -66,13 +70,17 @@ def test_sampling_server_binary(tmp_path, oracle, dyn_cache, table_mode, presamp
     out = subprocess.run([BIN, "1", "0", str(dyn_cache), "25,10"], cwd=str(tmp_path), env=env, timeout=100,
                          capture_output=True, text=True)
     assert out.returncode == 0, out.stdout + out.stderr
-    assert "System is ready for serving" in out.stdout and "batches: 8" in out.stdout
+    # the reference's schedule: (350-1)/100 = 3 training steps and 1 validation step per epoch,
+    # 1 test step after the last epoch
+    assert "System is ready for serving" in out.stdout and "batches: 9" in out.stdout
     if dyn_cache == 8:
         slot = oracle.static_cache_build(indptr, cache_bytes // (dim + 4))
         q, sc = oracle.quantize_rows(feats[np.flatnonzero(slot >= 0)])
-    for i in range(4):   # 350 ids / 100 -> batches of 100,100,100,50
+    valid = read_sets(str(data))[1]
+    for i in range(4):   # three training batches of 100, then the validation batch of 50
         nc, ec, ids, src, dst, feat = read_dump(str(dump / ("batch_%d.bin" % i)), dim)
-        o = oracle.sample_batch(indptr, indices, train[i * batch:(i + 1) * batch], fanout, 1 + i)
+        seeds, local = (train[i * batch:(i + 1) * batch], i) if i < 3 else (valid, 0)
+        o = oracle.sample_batch(indptr, indices, seeds, fanout, 1 + local)
         assert list(nc) == list(o.node_counter) and list(ec) == list(o.edge_counter)
         assert np.array_equal(ids, o.ids) and np.array_equal(src, o.agg_src_off) and np.array_equal(dst, o.agg_dst_off)
         if dyn_cache == 8:
