@@ -99,8 +99,8 @@ static int dmalloc(T **p, int64_t count) {
 
 static void pipe_free(Pipe &p) {
   void *ptrs[] = {p.ids, p.features, p.labels, p.agg_src_ids, p.agg_src_off, p.agg_dst_off, p.blk_indptr[0],
-                  p.blk_indptr[1], p.blk_indptr[2], p.cache_index, p.st, p.dedup.slots, p.eslot, p.firstv,
-                  p.cnt, p.rank, p.tile_sums, p.miss_list, p.lru_fill, p.seed_stage,
+                  p.blk_indptr[1], p.blk_indptr[2], p.cache_index, p.st, p.dedup.slots, p.eslot[0], p.eslot[1],
+                  p.miss_list, p.lru_fill, p.seed_stage,
                   p.chain_status[0], p.chain_status[1]};
   for (void *q : ptrs)
     if (q) (void)hipFree(q);
@@ -128,12 +128,9 @@ static int pipe_alloc(Server *s, Pipe &p) {
   while ((int64_t(1) << lg) * 2 < 3 * s->max_nodes) ++lg;
   p.dedup.log2cap = lg;
   LMI_HIP(hipMalloc(&p.dedup.slots, size_t(8) << lg));
-  LMI_TRY(dmalloc(&p.eslot, s->max_edges_hop));
-  LMI_TRY(dmalloc(&p.firstv, s->max_edges_hop));
+  LMI_TRY(dmalloc(&p.eslot[0], s->max_edges_hop));
+  LMI_TRY(dmalloc(&p.eslot[1], s->max_edges_hop));
   const int64_t scan_n = std::max(s->max_nodes, s->max_edges_hop);
-  LMI_TRY(dmalloc(&p.cnt, scan_n + 1));
-  LMI_TRY(dmalloc(&p.rank, s->max_edges_hop + 1));
-  LMI_TRY(dmalloc(&p.tile_sums, ceil_div(scan_n, 2048) + 1));
   // the finest tiling any scan kernel uses: 256 items per tile over nodes or edges, or the
   // node tiles of the fused count-and-sample kernel
   int64_t tiles = ceil_div(scan_n, 256);
@@ -510,7 +507,7 @@ int lmi_op_random_sample(lmi_server *h, int pipe, void *stream, int hop) {
   if (hop != p.hops_done || hop >= s->cfg.hops) LMI_FAIL(LMI_ERR_ARG, "hop %d out of order (next is %d)", hop, p.hops_done);
   hipStream_t st = (hipStream_t)stream;
   prof_phase(s, st, &s->prof_open, PROF_SAMPLE);
-  LMI_TRY(launch_hop(s, p, st, hop, false));
+  LMI_TRY(launch_hop(s, p, st, hop, false, false));
   prof_phase(s, st, &s->prof_open, -1);
   return LMI_OK;
 }
@@ -550,7 +547,8 @@ int lmi_presample(lmi_server *h, int pipe, void *stream, int mode, int32_t first
     LMI_TRY(batch_params(s, p, st, nullptr, 0, LMI_LOC_DEVICE, b, mode, 0, &bp));
     s->lru_tick = tick;  // presampling does not age the LRU cache
     LMI_TRY(launch_batch_generate(s, p, st, bp, false));
-    for (int k = 0; k < s->cfg.hops; ++k) LMI_TRY(launch_hop(s, p, st, k, true));
+    for (int k = 0; k < s->cfg.hops; ++k) LMI_TRY(launch_hop(s, p, st, k, true, true));
+    LMI_TRY(launch_fill(s, p, st));
     LMI_TRY(launch_hotness(s, p, st));
   }
   return LMI_OK;
@@ -579,7 +577,7 @@ static int capture_batch_graph(Server *s, Pipe &p, hipStream_t st, const BatchPa
   s->prof_on = false;  // no event records inside the capture
   LMI_HIP(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
   int rc = launch_batch_generate(s, p, st, bp, false);
-  for (int k = 0; rc == LMI_OK && k < s->cfg.hops; ++k) rc = launch_hop(s, p, st, k, true);
+  for (int k = 0; rc == LMI_OK && k < s->cfg.hops; ++k) rc = launch_hop(s, p, st, k, true, true);
   if (rc == LMI_OK) rc = launch_lookup(s, p, st, 0, s->cfg.hops);
   hipGraph_t g = nullptr;
   const hipError_t e = hipStreamEndCapture(st, &g);
@@ -621,7 +619,7 @@ int lmi_run_once(lmi_server *h, int pipe, void *stream, const int32_t *seeds, in
     LMI_HIP(hipGraphLaunch(p.graph_exec, st));
   } else {
     LMI_TRY(launch_batch_generate(s, p, st, bp, false));
-    for (int k = 0; k < s->cfg.hops; ++k) LMI_TRY(launch_hop(s, p, st, k, true));
+    for (int k = 0; k < s->cfg.hops; ++k) LMI_TRY(launch_hop(s, p, st, k, true, true));
     LMI_TRY(launch_lookup(s, p, st, 0, s->cfg.hops));
   }
   LMI_TRY(launch_gather_seg(s, p, st, 0, s->cfg.hops));

@@ -275,6 +275,8 @@ struct LookupArgs {
   int2 *miss_list;
   DevState *st;
   int seg_first, seg_last, seg;
+  int lookup_blocks;  // blocks [0, lookup_blocks) look rows up, the rest carry `fill`
+  FillArgs fill;      // last step of the hop sampled just before (hop -1: none)
 };
 
 // Bitmap + rank table: the slot of a cached node is the number of cached nodes
@@ -304,10 +306,15 @@ constexpr int kLookupBlock = 1024;
 static __global__ __launch_bounds__(kLookupBlock) void lookup_kernel(LookupArgs a) {
   __shared__ int wave_cnt[kLookupBlock / kWave];
   __shared__ int block_base;
+  if ((int)blockIdx.x >= a.lookup_blocks) {
+    fill_local_ids(a.fill, (int64_t)(blockIdx.x - a.lookup_blocks) * blockDim.x + threadIdx.x,
+                   (int64_t)(gridDim.x - a.lookup_blocks) * blockDim.x);
+    return;
+  }
   const int first = (a.seg_first == 0) ? 0 : a.st->node_counter[9 + a.seg_first - 1];
   const int last = a.st->node_counter[9 + a.seg_last];
   const int lane = threadIdx.x & (kWave - 1), wid = threadIdx.x / kWave;
-  const int stride = gridDim.x * blockDim.x;
+  const int stride = a.lookup_blocks * blockDim.x;
   for (int b = first + blockIdx.x * blockDim.x; b < last; b += stride) {
     const int i = b + threadIdx.x;
     bool miss = false;
@@ -373,7 +380,14 @@ int launch_lookup(Server *s, Pipe &p, hipStream_t st, int seg_first, int seg_las
   a.seg_last = seg_last;
   a.seg = seg_first;
   const int64_t n_max = s->node_cap[seg_last];
-  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(n_max, kLookupBlock), (int64_t)s->n_cu * 2));
+  int grid = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(n_max, kLookupBlock), (int64_t)s->n_cu * 2));
+  a.lookup_blocks = grid;
+  a.fill.hop = -1;
+  if (p.fill_pending >= 0) {  // the hop sampled last left its local ids to this kernel
+    a.fill = fill_args(p, p.fill_pending);
+    grid += fill_blocks(s->edge_cap[p.fill_pending], kLookupBlock);
+    p.fill_pending = -1;
+  }
   hipLaunchKernelGGL(lookup_kernel, dim3(grid), dim3(kLookupBlock), 0, st, a);
   LMI_HIP(hipGetLastError());
   return LMI_OK;

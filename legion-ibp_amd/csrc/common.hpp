@@ -84,11 +84,9 @@ struct Pipe {
   DevState *st = nullptr;
   // scratch
   Table dedup;                 // global id -> local id (per batch)
-  int32_t *eslot = nullptr;    // [max_edges_hop] table slot of each edge's source
-  int32_t *firstv = nullptr;   // [max_edges_hop] table value seen by each edge
-  int32_t *cnt = nullptr;      // [max(max_nodes, max_edges_hop)] scan input
-  int32_t *rank = nullptr;     // [max_edges_hop + 1] scan output
-  int32_t *tile_sums = nullptr;
+  int32_t *eslot[2] = {nullptr, nullptr};  // [max_edges_hop] table slot of each edge's source; hops alternate
+                                           // so that a hop's slots survive into the next hop's first kernel
+  int fill_pending = -1;       // hop whose edge sources still wait for their local ids (launch_fill)
   unsigned long long *chain_status[2] = {nullptr, nullptr};  // look-back scan state: [0] node scans, [1] edge scans
   int32_t max_tiles = 0;
   int2 *miss_list = nullptr;   // [max_nodes] (row, id) pairs of cache misses
@@ -198,7 +196,14 @@ hipEvent_t prof_phase(Server *s, hipStream_t st, int *open, int next_kind);
 // stage_seeds: also run the seed-staging kernel now (otherwise hop 0 stages them itself)
 int launch_batch_generate(Server *s, Pipe &p, hipStream_t st, const BatchParams &bp, bool stage_seeds);
 int graph_update_begin(Server *s, Pipe &p, const BatchParams &bp);
-int launch_hop(Server *s, Pipe &p, hipStream_t st, int hop, bool stage_seeds);
+// defer_fill: leave the last step of the hop (local ids of the edge sources) to the next
+// kernel of the batch -- the next hop's first kernel or the lookup -- which carries it in
+// extra blocks; otherwise a kernel of its own finishes the hop.
+int launch_hop(Server *s, Pipe &p, hipStream_t st, int hop, bool stage_seeds, bool defer_fill);
+int launch_fill(Server *s, Pipe &p, hipStream_t st);  // finishes a hop left pending, if any
+struct FillArgs;
+FillArgs fill_args(const Pipe &p, int hop);
+int fill_blocks(int64_t e_max, int block);  // grid share of a fill over at most e_max edges
 int launch_table_clear(Table &t, hipStream_t st);
 
 enum { SCAN_EPI_NONE = 0, SCAN_EPI_HOP_EDGES = 1, SCAN_EPI_HOP_NODES = 2 };
@@ -207,6 +212,8 @@ enum { SCAN_EPI_NONE = 0, SCAN_EPI_HOP_EDGES = 1, SCAN_EPI_HOP_NODES = 2 };
 int cache_build_static(Server *s, int64_t capacity_rows, int table_kind, bool int8);
 int cache_build_lru(Server *s, int64_t n_sets, int32_t ways);
 void cache_free(Server *s);
+// Extra blocks of the lookup finish a hop left pending (launch_hop, defer_fill).  (Finishing
+// it on the side stream instead, ahead of the host-link gather, measured 2 % slower.)
 int launch_lookup(Server *s, Pipe &p, hipStream_t st, int seg_first, int seg_last);
 int launch_hotness(Server *s, Pipe &p, hipStream_t st);
 int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last);

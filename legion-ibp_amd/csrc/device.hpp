@@ -77,6 +77,24 @@ __device__ __forceinline__ int32_t table_find(const HashSlot *slots, int log2cap
   }
 }
 
+// Last step of a hop: the local id of every edge source is the value its table slot
+// holds once the hop's first occurrences have published theirs.  Strided over the
+// `n_threads` threads that take part, `tid` being this thread's place among them.
+struct FillArgs {
+  const DevState *st;
+  const HashSlot *slots;
+  const int32_t *eslot;  // table slot per edge of hop `hop`
+  int32_t *agg_src_off;
+  int hop;               // -1: nothing to fill
+};
+
+__device__ __forceinline__ void fill_local_ids(const FillArgs &f, int64_t tid, int64_t n_threads) {
+  if (f.hop < 0) return;
+  const int n = f.st->edge_counter[9 + f.hop + 1];
+  const int eoff = f.st->edge_counter[12 + f.hop + 1];
+  for (int64_t e = tid; e < n; e += n_threads) f.agg_src_off[eoff + e] = f.slots[f.eslot[e]].val;
+}
+
 // ------------------------------------------------------------------- scans
 __device__ __forceinline__ int wave_inclusive_scan(int v) {
   const int lane = threadIdx.x & (kWave - 1);

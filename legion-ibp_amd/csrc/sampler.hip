@@ -13,12 +13,17 @@
 // plus an N-entry position map; scans instead of atomics for placement, so the
 // edge order is (node, slot) and local ids follow first occurrence in that order.
 //
-// A hop is four kernels:
-//   1. hop_count_scan   per-node output counts -> block-CSR row pointers (single-pass
-//                       scan); for hop 0 it also stages the seeds
-//   2. hop_sample       draw positions, write edges, insert sources into the dedup table
-//   3. hop_flag_scan    first-occurrence flags -> ranks (single-pass scan), new node count
-//   4. hop_relabel      local ids of edge sources, append new nodes to ids[]
+// A hop is three steps:
+//   1. hop_count_sample per-node output counts -> block-CSR row pointers (single-pass
+//                       scan), draw positions, write edges, insert sources into the dedup
+//                       table; for hop 0 it also stages the seeds.  (Also available as
+//                       two kernels, hop_count_scan + hop_sample.)
+//   2. hop_flag_scan    first-occurrence flags -> ranks (single-pass scan); first
+//                       occurrences append their node to ids[] and publish its local id
+//                       in the table; new node count
+//   3. fill             local id of every edge source = its table slot's value.  Inside a
+//                       batch this rides in extra blocks of the next kernel (the next
+//                       hop's step 1, or the cache lookup); hop_fill_kernel does it alone.
 #include <algorithm>
 
 #include "scan.hpp"
@@ -38,10 +43,12 @@ struct HopArgs {
   int32_t *agg_src_ids, *agg_src_off, *agg_dst_off;
   HashSlot *slots;
   int log2cap;
-  int32_t *eslot, *firstv, *rank;
+  int32_t *eslot;   // table slot per edge of this hop
   ScanChain chain_nodes, chain_edges;
   int max_tiles;
   int stage_seeds;  // hop 0 only: the seeds have not been staged by batch_generate_kernel yet
+  int tile_blocks;  // hop_count_sample: blocks [0, tile_blocks) own node tiles, the rest fill
+  FillArgs fill;    // the previous hop's last step, carried by hop_count_sample (hop -1: none)
 };
 
 // ------------------------------------------------------------ batch start
@@ -318,6 +325,11 @@ static __global__ __launch_bounds__(256) void hop_count_sample_kernel(HopArgs a)
   DevState *st = a.st;
   const int64_t flat = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   scan_chain_reset(a.chain_edges, a.max_tiles, flat, (int64_t)gridDim.x * blockDim.x);
+  if ((int)blockIdx.x >= a.tile_blocks) {  // extra blocks: the previous hop's local ids
+    fill_local_ids(a.fill, (int64_t)(blockIdx.x - a.tile_blocks) * blockDim.x + threadIdx.x,
+                   (int64_t)(gridDim.x - a.tile_blocks) * blockDim.x);
+    return;
+  }
   const int n_prev = st->node_counter[9 + a.hop];
   const int n_tiles = (n_prev + NPB - 1) / NPB;
   if (n_tiles == 0) {
@@ -412,18 +424,23 @@ static __global__ __launch_bounds__(256) void hop_count_sample_kernel(HopArgs a)
   }
 }
 
-// ------------------------------------------------------------- hop, phase 3
-// firstv[e] = table value of the edge's source; an edge is the first occurrence
-// of a new node iff that value names the edge itself.  rank[e] = number of first
-// occurrences before e; the total is the number of new nodes.
+// ------------------------------------------------------------- hop, step 2
+// An edge is the first occurrence of a new node iff the table value of its source names
+// the edge itself (n_prev + e).  Its rank among first occurrences (single-pass scan) is the
+// node's place after the n_prev known nodes: the edge appends the node to ids[] and
+// publishes the local id in the table.  Publishing while other tiles still read is safe: a
+// later edge of the same node compares the value with its own, larger, index either way.
 template <int ITEMS>
 static __global__ __launch_bounds__(kScanBlock) void hop_flag_scan_kernel(HopArgs a) {
   constexpr int TILE = kScanBlock * ITEMS;
   __shared__ int lds[kScanBlock / kWave + 1];
   __shared__ int s_prefix;
   DevState *st = a.st;
+  const int64_t flat = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  scan_chain_reset(a.chain_nodes, a.max_tiles, flat, (int64_t)gridDim.x * blockDim.x);  // for the next hop
   const int n_prev = st->node_counter[9 + a.hop];
   const int n = st->edge_counter[9 + a.hop + 1];
+  const int eoff = st->edge_counter[12 + a.hop + 1];
   const int n_tiles = (n + TILE - 1) / TILE;
   if (n_tiles == 0) {
     if (blockIdx.x == 0 && threadIdx.x == 0) scan_epilogue(SCAN_EPI_HOP_NODES, st, a.hop, 0);
@@ -432,15 +449,15 @@ static __global__ __launch_bounds__(kScanBlock) void hop_flag_scan_kernel(HopArg
   const int tile = blockIdx.x;
   if (tile < n_tiles) {
     const int base = tile * TILE + threadIdx.x * ITEMS;
-    int v[ITEMS], sum = 0;
+    int v[ITEMS], slot[ITEMS], sum = 0;
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {
       const int e = base + j;
       int flag = 0;
+      slot[j] = 0;
       if (e < n) {
-        const int32_t val = a.slots[a.eslot[e]].val;
-        a.firstv[e] = val;
-        flag = (val == n_prev + e) ? 1 : 0;
+        slot[j] = a.eslot[e];
+        flag = (a.slots[slot[j]].val == n_prev + e) ? 1 : 0;
       }
       v[j] = flag;
       sum += flag;
@@ -451,36 +468,20 @@ static __global__ __launch_bounds__(kScanBlock) void hop_flag_scan_kernel(HopArg
     int run = prefix + ex;
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {
-      if (base + j < n) a.rank[base + j] = run;
+      if (v[j]) {
+        const int local = n_prev + run;
+        a.ids[local] = a.agg_src_ids[eoff + base + j];
+        a.slots[slot[j]].val = local;
+      }
       run += v[j];
     }
     if (tile == n_tiles - 1 && threadIdx.x == 0) scan_epilogue(SCAN_EPI_HOP_NODES, st, a.hop, prefix + total);
   }
 }
 
-// ------------------------------------------------------------- hop, phase 4
-// local id of an edge source: an old node keeps its id; a new node gets
-// n_prev + (rank of its first edge among first edges).  First edges also
-// append the node to ids[] and publish the final id in the table.
-static __global__ __launch_bounds__(256) void hop_relabel_kernel(HopArgs a) {
-  const DevState *st = a.st;
-  const int64_t flat = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  scan_chain_reset(a.chain_nodes, a.max_tiles, flat, (int64_t)gridDim.x * blockDim.x);  // for the next hop
-  const int n_prev = st->node_counter[9 + a.hop];
-  const int n = st->edge_counter[9 + a.hop + 1];
-  const int eoff = st->edge_counter[12 + a.hop + 1];
-  for (int e = (int)flat; e < n; e += gridDim.x * blockDim.x) {
-    const int32_t val = a.firstv[e];
-    int32_t local = val;
-    if (val >= n_prev) {
-      local = n_prev + a.rank[val - n_prev];
-      if (val == n_prev + e) {
-        a.ids[local] = a.agg_src_ids[eoff + e];
-        a.slots[a.eslot[e]].val = local;
-      }
-    }
-    a.agg_src_off[eoff + e] = local;
-  }
+// ------------------------------------------------------------- hop, step 3
+static __global__ __launch_bounds__(256) void hop_fill_kernel(FillArgs f) {
+  fill_local_ids(f, (int64_t)blockIdx.x * blockDim.x + threadIdx.x, (int64_t)gridDim.x * blockDim.x);
 }
 
 // ---------------------------------------------------------------- launchers
@@ -527,7 +528,7 @@ int graph_update_begin(Server *s, Pipe &p, const BatchParams &bp) {
   return LMI_OK;
 }
 
-int launch_hop(Server *s, Pipe &p, hipStream_t st, int hop, bool stage_seeds) {
+int launch_hop(Server *s, Pipe &p, hipStream_t st, int hop, bool stage_seeds, bool defer_fill) {
   const int f = s->cfg.fanout[hop];
   const int64_t n_max = s->node_cap[hop], e_max = s->edge_cap[hop];
   HopArgs a{};
@@ -545,9 +546,7 @@ int launch_hop(Server *s, Pipe &p, hipStream_t st, int hop, bool stage_seeds) {
   a.agg_dst_off = p.agg_dst_off;
   a.slots = p.dedup.slots;
   a.log2cap = p.dedup.log2cap;
-  a.eslot = p.eslot;
-  a.firstv = p.firstv;
-  a.rank = p.rank;
+  a.eslot = p.eslot[hop & 1];
   a.chain_nodes = chain_of(p, 0);
   a.chain_edges = chain_of(p, 1);
   a.max_tiles = p.max_tiles;
@@ -555,10 +554,19 @@ int launch_hop(Server *s, Pipe &p, hipStream_t st, int hop, bool stage_seeds) {
   int G = 4;
   while (G < f) G <<= 1;
   const bool fused = s->fuse_count && !s->lds_dedup;
+  a.fill.hop = -1;
+  if (!fused) LMI_TRY(launch_fill(s, p, st));
   if (fused) {
-    // counts, scan and sampling in one launch, one tile of nodes per block
+    // counts, scan and sampling in one launch, one tile of nodes per block; a hop left
+    // pending gets its local ids filled in by extra blocks behind the tile blocks
     const int npb = hop_tile_nodes(n_max, G, s->fuse_small_max);
-    const int grid = (int)ceil_div(std::max<int64_t>(n_max, 1), npb);
+    a.tile_blocks = (int)ceil_div(std::max<int64_t>(n_max, 1), npb);
+    int grid = a.tile_blocks;
+    if (p.fill_pending >= 0) {
+      a.fill = fill_args(p, p.fill_pending);
+      grid += fill_blocks(s->edge_cap[p.fill_pending], 256);
+      p.fill_pending = -1;
+    }
 #define LMI_FUSED(GG)                                                                                   \
   if (npb == 64)                                                                                        \
     hipLaunchKernelGGL((hop_count_sample_kernel<GG, 64>), dim3(grid), dim3(256), 0, st, a);             \
@@ -610,10 +618,33 @@ int launch_hop(Server *s, Pipe &p, hipStream_t st, int hop, bool stage_seeds) {
     hipLaunchKernelGGL(hop_flag_scan_kernel<4>, dim3((int)ceil_div(em, kScanBlock * 4)), dim3(kScanBlock), 0, st, a);
   else
     hipLaunchKernelGGL(hop_flag_scan_kernel<8>, dim3((int)ceil_div(em, kScanBlock * 8)), dim3(kScanBlock), 0, st, a);
-  const int rgrid = (int)std::min<int64_t>(ceil_div(e_max, 256), 4096);
-  hipLaunchKernelGGL(hop_relabel_kernel, dim3(rgrid), dim3(256), 0, st, a);
   LMI_HIP(hipGetLastError());
+  p.fill_pending = hop;
+  if (!defer_fill) LMI_TRY(launch_fill(s, p, st));
   p.hops_done = hop + 1;
+  return LMI_OK;
+}
+
+FillArgs fill_args(const Pipe &p, int hop) {
+  FillArgs f{};
+  f.st = p.st;
+  f.slots = p.dedup.slots;
+  f.eslot = p.eslot[hop & 1];
+  f.agg_src_off = p.agg_src_off;
+  f.hop = hop;
+  return f;
+}
+
+int fill_blocks(int64_t e_max, int block) {
+  return (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(e_max, block), 1024));
+}
+
+int launch_fill(Server *s, Pipe &p, hipStream_t st) {
+  if (p.fill_pending < 0) return LMI_OK;
+  hipLaunchKernelGGL(hop_fill_kernel, dim3(fill_blocks(s->edge_cap[p.fill_pending], 256)), dim3(256), 0, st,
+                     fill_args(p, p.fill_pending));
+  LMI_HIP(hipGetLastError());
+  p.fill_pending = -1;
   return LMI_OK;
 }
 
