@@ -219,9 +219,10 @@ int lmi_batch_counters(lmi_server *s, int pipe, void *stream, int32_t node_count
 int lmi_steps_per_epoch(lmi_server *s, int mode, int32_t *steps);
 
 /* ---- measurement ------------------------------------------------------- */
-/* level 0: off; 1: HIP events bracket every phase of a batch (sampling, lookup, both
- * gathers); 2: only the two gather kernels are bracketed, the sampling kernels run back
- * to back as without profiling.  Rows per gather are counted on the device at any level. */
+/* level 0: off; 1: HIP events bracket the sampling phase and the lookup of a batch and each
+ * gather kernel carries a start / stop event pair of its own; 2: only the gather kernels
+ * are timed, nothing is queued between kernels.  Rows per gather are counted on the device
+ * for the same batches.  lmi_tune("profile_every", n) profiles one batch in n. */
 int lmi_profile_enable(lmi_server *s, int level);
 int lmi_profile_read(lmi_server *s, lmi_profile *out, int reset);  /* synchronises the device */
 /* Tuning knobs by name (e.g. "gather_lanes_per_row", "gather_unroll", "lds_dedup"). */

@@ -69,6 +69,22 @@ hipEvent_t prof_phase(Server *s, hipStream_t st, int *open, int next_kind) {
   return e;
 }
 
+// Start of a batch: decides whether this one is profiled.
+static void prof_batch(Server *s) {
+  s->prof_on = s->prof_level != 0 && (s->prof_seq++ % std::max(1, s->prof_every)) == 0;
+}
+
+void prof_kernel_events(Server *s, int kind, hipEvent_t *start, hipEvent_t *stop) {
+  *start = *stop = nullptr;
+  if (!s->prof_on) return;
+  EventPair p{prof_event(s), prof_event(s), kind};
+  s->prof_used.push_back(p.a);
+  s->prof_used.push_back(p.b);
+  s->prof_events.push_back(p);
+  *start = p.a;
+  *stop = p.b;
+}
+
 // The captured batch graphs hold the graph, cache-table and tuning state by value:
 // anything that changes those must drop them (they are captured again on next use).
 static void invalidate_graphs(Server *s) {
@@ -494,6 +510,7 @@ int lmi_op_batch_generate(lmi_server *h, int pipe, void *stream, const int32_t *
   Pipe &p = s->pipes[pipe];
   hipStream_t st = (hipStream_t)stream;
   BatchParams bp{};
+  prof_batch(s);
   LMI_TRY(pipe_join(p, st));
   LMI_TRY(batch_params(s, p, st, seeds, n, seeds_location, batch_counter, mode, rng_seed, &bp));
   return launch_batch_generate(s, p, st, bp, true);
@@ -610,6 +627,7 @@ int lmi_run_once(lmi_server *h, int pipe, void *stream, const int32_t *seeds, in
   Pipe &p = s->pipes[pipe];
   hipStream_t st = (hipStream_t)stream;
   BatchParams bp{};
+  prof_batch(s);
   LMI_TRY(batch_params(s, p, st, seeds, n, seeds_location, batch_counter, mode, rng_seed, &bp));
   LMI_TRY(pipe_join(p, st));  // the previous batch of this pipe may still be gathering misses
   prof_phase(s, st, &s->prof_open, PROF_SAMPLE);
@@ -693,6 +711,7 @@ int lmi_profile_enable(lmi_server *h, int on) {
   if (on < 0 || on > 2) LMI_FAIL(LMI_ERR_ARG, "profile level must be 0, 1 or 2");
   s->prof_on = on != 0;
   s->prof_level = on;
+  s->prof_seq = 0;
   return LMI_OK;
 }
 
@@ -738,6 +757,7 @@ int lmi_tune(lmi_server *h, const char *key, int64_t value) {
   else if (!strcmp(key, "gather_nontemporal")) s->gather_nt = (int)value;
   else if (!strcmp(key, "lds_dedup")) s->lds_dedup = (int)value;
   else if (!strcmp(key, "fuse_count")) s->fuse_count = (int)value;
+  else if (!strcmp(key, "profile_every")) s->prof_every = (int)std::max<int64_t>(1, value);
   else if (!strcmp(key, "fuse_small_max")) s->fuse_small_max = value;
   else if (!strcmp(key, "split_miss")) s->split_miss = (int)value;
   else if (!strcmp(key, "use_graph")) s->use_graph = (int)value;

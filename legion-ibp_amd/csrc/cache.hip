@@ -17,6 +17,8 @@
 #include <algorithm>
 #include <vector>
 
+#include <hip/hip_ext.h>
+
 #include "scan.hpp"
 
 namespace lmi {
@@ -91,6 +93,7 @@ struct MoveArgs {
   int unroll;      // 0 = the server's gather_unroll
   int host_link;   // the source is pinned host memory read over the host link
   unsigned long long *row_counter;  // device counter that receives the number of work items, or null
+  hipEvent_t ev_start, ev_stop;     // stamped with the kernel's begin and end when not null (profiling)
   const uint8_t *src;
   uint8_t *dst;
   int64_t src_row_bytes, dst_row_bytes, row_bytes;  // row_bytes = bytes moved per row
@@ -100,18 +103,25 @@ struct MoveArgs {
 template <typename V, int LPR, int U>
 static void launch_move_vlu(hipStream_t st, const MoveArgs &a, int grid, bool nt) {
   const int chunks = (int)(a.row_bytes / sizeof(V));
-  if (a.host_link)
-    hipLaunchKernelGGL((move_rows_kernel<V, LPR, U, true, true>), dim3(grid), dim3(256), 0, st, a.list, a.first_ptr,
-                       a.n_ptr, a.src_index, a.dst_index, a.src_from_list, a.src, a.dst, chunks, a.src_row_bytes,
-                       a.dst_row_bytes, a.row_counter);
-  else if (nt)
-    hipLaunchKernelGGL((move_rows_kernel<V, LPR, U, true, false>), dim3(grid), dim3(256), 0, st, a.list, a.first_ptr,
-                       a.n_ptr, a.src_index, a.dst_index, a.src_from_list, a.src, a.dst, chunks, a.src_row_bytes,
-                       a.dst_row_bytes, a.row_counter);
-  else
-    hipLaunchKernelGGL((move_rows_kernel<V, LPR, U, false, false>), dim3(grid), dim3(256), 0, st, a.list, a.first_ptr,
-                       a.n_ptr, a.src_index, a.dst_index, a.src_from_list, a.src, a.dst, chunks, a.src_row_bytes,
-                       a.dst_row_bytes, a.row_counter);
+  // with profiling on, the launch carries its own start / stop events
+#define LMI_MOVE(NT_, HL_)                                                                                      \
+  if (a.ev_start)                                                                                               \
+    hipExtLaunchKernelGGL((move_rows_kernel<V, LPR, U, NT_, HL_>), dim3(grid), dim3(256), 0, st, a.ev_start,     \
+                          a.ev_stop, 0, a.list, a.first_ptr, a.n_ptr, a.src_index, a.dst_index,                  \
+                          a.src_from_list, a.src, a.dst, chunks, a.src_row_bytes, a.dst_row_bytes,               \
+                          a.row_counter);                                                                        \
+  else                                                                                                          \
+    hipLaunchKernelGGL((move_rows_kernel<V, LPR, U, NT_, HL_>), dim3(grid), dim3(256), 0, st, a.list,            \
+                       a.first_ptr, a.n_ptr, a.src_index, a.dst_index, a.src_from_list, a.src, a.dst, chunks,    \
+                       a.src_row_bytes, a.dst_row_bytes, a.row_counter)
+  if (a.host_link) {
+    LMI_MOVE(true, true);
+  } else if (nt) {
+    LMI_MOVE(true, false);
+  } else {
+    LMI_MOVE(false, false);
+  }
+#undef LMI_MOVE
 }
 
 template <typename V, int LPR>
@@ -418,31 +428,33 @@ static int launch_hits(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last
     const int32_t *n_ptr = &p.st->node_counter[9 + seg_last];
     const int8_t *q = (const int8_t *)s->cache_data;
     unsigned long long *rc = s->prof_on ? s->d_prof_rows : nullptr;
+    hipEvent_t e0, e1;
+    prof_kernel_events(s, PROF_GATHER_HIT, &e0, &e1);
+#define LMI_INT8(KERN, OUT_T)                                                                                   \
+  if (e0)                                                                                                       \
+    hipExtLaunchKernelGGL((KERN), dim3(grid), dim3(256), 0, st, e0, e1, 0, first_ptr, n_ptr, p.cache_index, q,   \
+                          s->cache_scale, (OUT_T *)p.features, dim, rc);                                         \
+  else                                                                                                          \
+    hipLaunchKernelGGL((KERN), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr, p.cache_index, q, s->cache_scale, \
+                       (OUT_T *)p.features, dim, rc)
+    const bool half = s->cfg.feat_dtype == LMI_F16;
     if (dim % 16 == 0) {
-      const int chunks = dim / 16;
-      if (s->cfg.feat_dtype == LMI_F16) {
-        if (chunks <= 32)
-          hipLaunchKernelGGL((gather_int8_kernel<__half, 32>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
-                             p.cache_index, q, s->cache_scale, (__half *)p.features, dim, rc);
-        else
-          hipLaunchKernelGGL((gather_int8_kernel<__half, 64>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
-                             p.cache_index, q, s->cache_scale, (__half *)p.features, dim, rc);
+      const bool narrow = dim / 16 <= 32;
+      if (half && narrow) {
+        LMI_INT8((gather_int8_kernel<__half, 32>), __half);
+      } else if (half) {
+        LMI_INT8((gather_int8_kernel<__half, 64>), __half);
+      } else if (narrow) {
+        LMI_INT8((gather_int8_kernel<float, 32>), float);
       } else {
-        if (chunks <= 32)
-          hipLaunchKernelGGL((gather_int8_kernel<float, 32>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
-                             p.cache_index, q, s->cache_scale, (float *)p.features, dim, rc);
-        else
-          hipLaunchKernelGGL((gather_int8_kernel<float, 64>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
-                             p.cache_index, q, s->cache_scale, (float *)p.features, dim, rc);
+        LMI_INT8((gather_int8_kernel<float, 64>), float);
       }
+    } else if (half) {
+      LMI_INT8((gather_int8_generic_kernel<__half>), __half);
     } else {
-      if (s->cfg.feat_dtype == LMI_F16)
-        hipLaunchKernelGGL((gather_int8_generic_kernel<__half>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
-                           p.cache_index, q, s->cache_scale, (__half *)p.features, dim, rc);
-      else
-        hipLaunchKernelGGL((gather_int8_generic_kernel<float>), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr,
-                           p.cache_index, q, s->cache_scale, (float *)p.features, dim, rc);
+      LMI_INT8((gather_int8_generic_kernel<float>), float);
     }
+#undef LMI_INT8
     LMI_HIP(hipGetLastError());
     return LMI_OK;
   }
@@ -456,6 +468,7 @@ static int launch_hits(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last
   m.src_row_bytes = m.dst_row_bytes = m.row_bytes = s->row_bytes;
   m.n_max = n_max;
   m.row_counter = s->prof_on ? s->d_prof_rows : nullptr;  // all rows of the segment: hits + misses
+  prof_kernel_events(s, PROF_GATHER_HIT, &m.ev_start, &m.ev_stop);
   return launch_move_rows(s, st, m, s->gather_nt != 0);
 }
 
@@ -476,6 +489,7 @@ static int launch_misses(Server *s, Pipe &p, hipStream_t st, int seg, int seg_la
     m.host_link = 1;
   }
   m.row_counter = s->prof_on ? s->d_prof_rows + 1 : nullptr;  // misses
+  prof_kernel_events(s, PROF_GATHER_MISS, &m.ev_start, &m.ev_stop);
   return launch_move_rows(s, st, m, s->gather_nt != 0);
 }
 
@@ -494,34 +508,26 @@ static int launch_misses(Server *s, Pipe &p, hipStream_t st, int seg, int seg_la
 int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last) {
   const bool have_cache = s->cache_kind != LMI_CACHE_NONE;
   int mode = (s->feat_loc == LMI_LOC_HOST && have_cache) ? s->split_miss : 0;
+  // The gather kernels carry their own profiling events (prof_kernel_events); a bracket
+  // left open by the sampling phase ends here.
+  hipEvent_t closing = prof_phase(s, st, &s->prof_open, -1);
   if (mode == 0) {
-    if (have_cache) {
-      prof_phase(s, st, &s->prof_open, PROF_GATHER_HIT);
-      LMI_TRY(launch_hits(s, p, st, seg, seg_last));
-    }
-    prof_phase(s, st, &s->prof_open, PROF_GATHER_MISS);
+    if (have_cache) LMI_TRY(launch_hits(s, p, st, seg, seg_last));
     LMI_TRY(launch_misses(s, p, st, seg, seg_last));
-    prof_phase(s, st, &s->prof_open, -1);
     return LMI_OK;
   }
+  hipEvent_t fork = closing;  // when mode 2 forks right here, the closing event doubles as the fork
   if (mode == 1) {
-    prof_phase(s, st, &s->prof_open, PROF_GATHER_HIT);
     LMI_TRY(launch_hits(s, p, st, seg, seg_last));
+    fork = nullptr;
   }
-  // the event that closes the profiling bracket, when there is one, also serves as the fork
-  hipEvent_t fork = prof_phase(s, st, &s->prof_open, -1);
   if (!fork) {
     fork = p.fork;
     LMI_HIP(hipEventRecord(fork, st));
   }
   LMI_HIP(hipStreamWaitEvent(s->side, fork, 0));
-  if (mode == 2) {
-    prof_phase(s, s->side, &s->prof_open_side, PROF_GATHER_HIT);
-    LMI_TRY(launch_hits(s, p, s->side, seg, seg_last));
-  }
-  prof_phase(s, s->side, &s->prof_open_side, PROF_GATHER_MISS);
+  if (mode == 2) LMI_TRY(launch_hits(s, p, s->side, seg, seg_last));
   LMI_TRY(launch_misses(s, p, s->side, seg, seg_last));
-  prof_phase(s, s->side, &s->prof_open_side, -1);
   LMI_HIP(hipEventRecord(p.join, s->side));
   p.side_pending = true;
   if (s->cache_kind == LMI_CACHE_LRU) LMI_TRY(pipe_join(p, st));

@@ -170,8 +170,10 @@ struct Server {
                           // not to crowd HBM traffic out of the memory pipeline
   int miss_unroll = 1;    // rows in flight per lane in the host-link gather
   // profiling
-  bool prof_on = false;                 // any level: device row counters are kept
+  bool prof_on = false;                 // the batch being issued is profiled (events + device row counters)
   int prof_level = 0;                   // 0 off, 1 every phase bracketed, 2 only the gather kernels
+  int prof_every = 1;                   // profile one batch in this many (tuning key "profile_every")
+  int64_t prof_seq = 0;                 // batches begun since profiling was switched on
   std::vector<EventPair> prof_events;   // recorded, not yet resolved
   std::vector<hipEvent_t> prof_used;    // every event recorded since the last read (pairs may share one)
   std::vector<hipEvent_t> prof_free;    // recycled events
@@ -191,6 +193,10 @@ int prof_end(Server *s, hipStream_t st, int handle);
 // One event closes the pair left open on the caller's stream and opens the next
 // phase (next_kind < 0: only close), so a batch costs one event per phase boundary.
 hipEvent_t prof_phase(Server *s, hipStream_t st, int *open, int next_kind);
+// A start / stop event pair for one kernel launch of kind `kind` (both null when profiling
+// is off): handed to hipExtLaunchKernelGGL, which stamps them with the kernel's own begin
+// and end, so nothing is queued between the kernel and its neighbours.
+void prof_kernel_events(Server *s, int kind, hipEvent_t *start, hipEvent_t *stop);
 
 // sampler.hip
 // stage_seeds: also run the seed-staging kernel now (otherwise hop 0 stages them itself)
