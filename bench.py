@@ -44,7 +44,8 @@ WORKLOADS = {
     "products": dict(nodes=2_449_029, mean_deg=25.27, alpha=2.1, d_max=17_000, dim=100, dtype="f32",
                      batch=800, fanout=[25, 10], train=196_615, cache=("static_frac", 0.30)),
     "paper100m-lru": dict(nodes=111_059_956, mean_deg=14.548, alpha=2.0, d_max=100_000, dim=128, dtype="f32",
-                          batch=4096, fanout=[15, 10, 5], train=1_200_000, cache=("lru", 20e9)),
+                          batch=4096, fanout=[15, 10, 5], train=1_200_000, cache=("lru", 20e9),
+                          locality=(0.8, 10)),   # 80 % of a batch's seeds come from the last 10 batches' frontiers
     "mag240m-int8": dict(nodes=244_160_499, mean_deg=7.08, alpha=2.0, d_max=100_000, dim=768, dtype="f16",
                          batch=1024, fanout=[25, 15], train=1_112_392, cache=("int8", 80e9)),
     "cora": dict(nodes=2_708, mean_deg=7.8, alpha=None, d_max=40, dim=1433, dtype="f32",
@@ -142,6 +143,29 @@ def build_workload(lmi, w, seed, pipes, host_budget_gb, table=2, policy="degree"
     return srv, info
 
 
+def record_seed_plan(lmi, srv, w, info, n_batches, seed):
+    """Seed batches with temporal locality: a fraction of every batch is drawn from the frontiers
+    (all node ids) of the previous batches, the rest uniformly from the train set.  The frontiers
+    depend on the sampled batches, so the sequence is recorded in one untimed pass; the caller
+    resets the cache afterwards and replays the recorded seeds (same RNG seeds, same batches)."""
+    frac, depth = w["locality"]
+    rng = np.random.default_rng(seed + 7)
+    B, train = w["batch"], info["train"]
+    recent, plan = [], []
+    for t in range(n_batches):
+        n_loc = int(frac * B) if recent else 0
+        parts = [train[rng.integers(0, len(train), B - n_loc)]]
+        if n_loc:
+            pool = np.concatenate(recent[-depth:])
+            parts.insert(0, pool[rng.integers(0, len(pool), n_loc)])
+        seeds = np.array(list(dict.fromkeys(np.concatenate(parts).tolist())), np.int32)   # distinct, order kept
+        srv.run_once(seeds, rng_seed=seed + t)
+        recent.append(srv.fetch_ids())
+        recent = recent[-depth:]
+        plan.append(seeds)
+    return plan
+
+
 def cpu_baseline(lmi, srv, w, info, seed, budget_s):
     """The CPU oracle on the same workload and host cores; also checks the GPU
     output of the same batches bit for bit."""
@@ -231,13 +255,20 @@ def main():
         srv.tune(k, int(v))
     steps_per_epoch = -(-info["n_train"] // w["batch"])
     streams = [lmi.stream_create() for _ in range(max(1, args.streams))]
+    plan = None
+    if w.get("locality"):
+        t0 = time.time()
+        plan = record_seed_plan(lmi, srv, w, info, args.warmup + args.steps + min(args.steps, 20), args.seed)
+        ci = srv.cache_info()
+        srv.build_lru_cache(int(ci.n_sets), int(ci.ways))   # start the replay from an empty cache again
+        log("recorded %d seed batches with temporal locality (%.1f s)" % (len(plan), time.time() - t0))
 
     def step(i):
         # consecutive batches alternate output buffer sets (pipes), so the host-link part of batch i
         # (on the server's side stream) overlaps the sampling of batch i+1; a pipe always uses the
         # same caller stream
         p = i % args.pipes
-        srv.run_once(None, batch_counter=i % steps_per_epoch, rng_seed=args.seed + i, pipe=p,
+        srv.run_once(plan[i] if plan else None, batch_counter=i % steps_per_epoch, rng_seed=args.seed + i, pipe=p,
                      stream=streams[p % len(streams)])
 
     for i in range(args.warmup):
@@ -299,6 +330,9 @@ def main():
                    "cache": "%s, %d rows, %s id->slot table" % (info["cache_kind"], info["cache_rows"], args.table),
                    "pipes": args.pipes, "streams": args.streams, "cache_policy": args.policy,
                    "graph": "Zipf-Mandelbrot degrees alpha=%s, degree-proportional neighbours" % w["alpha"],
+                   "seeds": ("%d %% of a batch from the frontiers of the previous %d batches, the rest uniform from the "
+                             "train set" % (w["locality"][0] * 100, w["locality"][1])) if w.get("locality")
+                   else "consecutive slices of the train set",
                    "note": info["note"]},
         "feature_gather_gbs": round(achieved, 1),
         "feature_gather_frac_hbm_peak": round(achieved / HBM_PEAK_GBS, 4),

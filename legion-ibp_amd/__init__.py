@@ -316,6 +316,11 @@ class Server:
             b.features = to_host(v.features, n * d, self.np_dtype).reshape(n, d)
         return b
 
+    def fetch_ids(self, pipe=0, stream=None):
+        """Synchronise and copy only the batch's node ids (its frontier) to the host."""
+        nc, _ = self.counters(pipe, stream)
+        return to_host(self.view(pipe).ids, int(nc[9 + int(nc[8])]), np.int32)
+
     # measurement -------------------------------------------------------------
     def profile_enable(self, level=1):
         """0 / False: off; 1 / True: events around every phase; 2: around the gather kernels only."""
