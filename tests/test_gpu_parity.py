@@ -58,6 +58,48 @@ def test_sample_batch_parity(lmi, oracle, fanout, n_nodes, mean_deg, batch):
         feats.free()
 
 
+@pytest.mark.parametrize("case", range(24))
+def test_random_shapes_sweep(lmi, oracle, case):
+    """Seeded sweep over shapes the fixed cases do not reach: one-node and two-node graphs,
+    edgeless graphs, batches of one seed, repeated seeds, fan-outs 1..64 in any order, hubs with
+    more than 2^16 neighbours, with and without a static cache, on a stream or not."""
+    rng = np.random.default_rng(1000 + case)
+    hops = int(rng.integers(1, 4))
+    fanout = [int(rng.choice([1, 2, 3, 5, 8, 16, 25, 33, 64])) for _ in range(hops)]
+    n_nodes = int(rng.choice([1, 2, 50, 1000, 20000]))
+    mean_deg = float(rng.choice([0, 1, 5, 40]))
+    batch = int(rng.choice([1, 7, 64, 500]))
+    hubs = int(rng.integers(0, 3)) if n_nodes >= 1000 else 0
+    indptr, indices = random_graph(rng, n_nodes, mean_deg, hubs=hubs, hub_deg=int(rng.choice([300, 70000])),
+                                   zero_frac=float(rng.choice([0.0, 0.3])))
+    dim = int(rng.choice([4, 20, 128]))
+    feats = make_features(lmi, rng, n_nodes, dim)
+    srv = lmi.Server(batch, fanout, dim, pipes=2, seed=5)
+    stream = lmi.stream_create() if case % 2 else None
+    slot_ref = None
+    try:
+        if case % 3 == 0:
+            srv.tune("use_graph", 1)
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        if case % 4 != 3:
+            cap = int(rng.integers(1, n_nodes + 1))
+            srv.build_static_cache(cap, int(rng.integers(0, 3)))
+            slot_ref = oracle.static_cache_build(indptr, cap)
+        for it in range(3):
+            seeds = rng.integers(0, n_nodes, int(rng.integers(1, batch + 1))).astype(np.int32)   # repeats allowed
+            srv.run_once(seeds, rng_seed=50 + it, pipe=it % 2, stream=stream)
+            g = srv.fetch(pipe=it % 2, stream=stream)
+            o = oracle.sample_batch(indptr, indices, seeds, fanout, 50 + it)
+            assert_batch_equal(g, o)
+            assert g.features.tobytes() == feats.array[o.ids].tobytes()
+            if slot_ref is not None:
+                np.testing.assert_array_equal(g.cache_index, slot_ref[o.ids])
+    finally:
+        srv.close()
+        feats.free()
+
+
 @pytest.mark.parametrize("fanout", [[25, 10], [64, 3], [5, 4, 3]])
 def test_lds_staged_dedup_gives_the_same_batches(lmi, oracle, fanout):
     rng = np.random.default_rng(sum(fanout))
