@@ -182,16 +182,10 @@ def cpu_baseline(lmi, srv, w, info, seed, budget_s):
     B = w["batch"]
     done, spent, parity_ok, rows = 0, 0.0, True, 0
     max_batches = min(256, len(info["train"]) // B)
-    while done < max_batches and spent < budget_s:
-        seeds = info["train"][done * B:(done + 1) * B]
-        rs = seed + done
-        t0 = time.time()
-        o = orc.sample_batch(indptr, indices, seeds, w["fanout"], rs, threads=threads)
-        out = orc.gather_rows(o.ids, np.full(len(o.ids), -1, np.int32), None, feats, threads=threads)
-        spent += time.time() - t0
-        rows += len(o.ids)
-        srv.run_once(None, batch_counter=done, rng_seed=rs)
-        g = srv.fetch()
+    pipes = max(1, int(srv.cfg.pipes))
+    stream = lmi.stream_create()
+
+    def same_as_oracle(g, o, out):
         same = (np.array_equal(g.ids, o.ids) and np.array_equal(g.agg_src_off, o.agg_src_off) and
                 np.array_equal(g.agg_dst_off, o.agg_dst_off) and np.array_equal(g.agg_src_ids, o.agg_src_ids) and
                 list(g.node_counter) == list(o.node_counter) and list(g.edge_counter) == list(o.edge_counter) and
@@ -207,8 +201,23 @@ def cpu_baseline(lmi, srv, w, info, seed, budget_s):
             hit = g.cache_index >= 0
             if hit.any() and (~hit).any():
                 same = same and deg[hit].min() >= deg[~hit].max()
-        parity_ok = parity_ok and same
-        done += 1
+        return same
+
+    while done < max_batches and spent < budget_s:
+        # the GPU issues `pipes` batches back to back, as in the timed region (the host-link gather of
+        # one overlaps the sampling of the next), before any of them is read back
+        group = list(range(done, min(done + pipes, max_batches)))
+        for k, b in enumerate(group):
+            srv.run_once(None, batch_counter=b, rng_seed=seed + b, pipe=k, stream=stream)
+        for k, b in enumerate(group):
+            seeds = info["train"][b * B:(b + 1) * B]
+            t0 = time.time()
+            o = orc.sample_batch(indptr, indices, seeds, w["fanout"], seed + b, threads=threads)
+            out = orc.gather_rows(o.ids, np.full(len(o.ids), -1, np.int32), None, feats, threads=threads)
+            spent += time.time() - t0
+            rows += len(o.ids)
+            parity_ok = same_as_oracle(srv.fetch(pipe=k, stream=stream), o, out) and parity_ok
+            done += 1
     return dict(value=done / spent, unit="batches/s", cores=threads, kind="port",
                 sample="%d batches of the same workload (oracle sample_batch + gather, OpenMP over %d threads); "
                        "GPU output of the same batches %s" % (done, threads,
