@@ -255,8 +255,6 @@ def main():
         w["train"] = max(w["batch"], int(w["train"] * args.scale))
         if w["cache"][0] in ("static", "lru", "int8"):
             w["cache"] = (w["cache"][0], w["cache"][1] * args.scale)
-    if w["cache"][0] == "lru":
-        args.pipes = 1   # the LRU state is batch-synchronous: batches may not overlap
     srv, info = build_workload(lmi, w, args.seed, args.pipes, args.host_gb,
                                {"hash": 0, "direct": 1, "rank": 2}[args.table], args.policy)
     for kv in args.tune:

@@ -237,6 +237,7 @@ int lmi_server_create(const lmi_config *cfg, lmi_server **out) {
     if ((rc = pipe_alloc(s, p)) != LMI_OK) break;
   if (rc == LMI_OK && hipMalloc(&s->d_scalar, 64) != hipSuccess) rc = LMI_ERR_HIP;
   if (rc == LMI_OK && hipStreamCreateWithFlags(&s->side, hipStreamNonBlocking) != hipSuccess) rc = LMI_ERR_HIP;
+  if (rc == LMI_OK && hipEventCreateWithFlags(&s->lru_ready, hipEventDisableTiming) != hipSuccess) rc = LMI_ERR_HIP;
   if (rc == LMI_OK && (hipMalloc(&s->d_prof_rows, 16) != hipSuccess || hipMemset(s->d_prof_rows, 0, 16) != hipSuccess))
     rc = LMI_ERR_HIP;
   if (rc != LMI_OK) {
@@ -268,6 +269,7 @@ int lmi_server_destroy(lmi_server *h) {
   if (s->d_scalar) (void)hipFree(s->d_scalar);
   if (s->hot) (void)hipFree(s->hot);
   if (s->side) (void)hipStreamDestroy(s->side);
+  if (s->lru_ready) (void)hipEventDestroy(s->lru_ready);
   delete s;
   return LMI_OK;
 }
@@ -538,9 +540,10 @@ int lmi_op_cache_lookup(lmi_server *h, int pipe, void *stream, int segment) {
   if (segment < 0 || segment > p.hops_done) LMI_FAIL(LMI_ERR_ARG, "segment %d not sampled yet", segment);
   hipStream_t st = (hipStream_t)stream;
   LMI_TRY(pipe_join(p, st));
+  LMI_TRY(lru_wait_ready(s, st));
   prof_phase(s, st, &s->prof_open, PROF_LOOKUP);
   LMI_TRY(launch_lookup(s, p, st, segment, segment));
-  LMI_TRY(launch_gather_seg(s, p, st, segment, segment));
+  LMI_TRY(launch_gather_seg(s, p, st, segment, segment, 0));
   prof_phase(s, st, &s->prof_open, -1);
   return LMI_OK;
 }
@@ -633,16 +636,17 @@ int lmi_run_once(lmi_server *h, int pipe, void *stream, const int32_t *seeds, in
   LMI_TRY(pipe_join(p, st));  // the previous batch of this pipe may still be gathering misses
   prof_phase(s, st, &s->prof_open, PROF_SAMPLE);
   if (s->use_graph && st != nullptr) {  // the legacy default stream cannot be captured
+    LMI_TRY(lru_wait_ready(s, st));       // the lookup sits inside the graph: the whole replay waits
     if (!p.graph_exec) LMI_TRY(capture_batch_graph(s, p, st, bp));
     LMI_TRY(graph_update_begin(s, p, bp));
     LMI_HIP(hipGraphLaunch(p.graph_exec, st));
   } else {
     LMI_TRY(launch_batch_generate(s, p, st, bp, false));
     for (int k = 0; k < s->cfg.hops; ++k) LMI_TRY(launch_hop(s, p, st, k, true, true));
+    LMI_TRY(lru_wait_ready(s, st));  // sampling may overlap the previous batch's insertion, the lookup may not
     LMI_TRY(launch_lookup(s, p, st, 0, s->cfg.hops));
   }
-  LMI_TRY(launch_gather_seg(s, p, st, 0, s->cfg.hops));
-  LMI_TRY(launch_lru_insert(s, p, st, 1));
+  LMI_TRY(launch_gather_seg(s, p, st, 0, s->cfg.hops, s->cache_kind == LMI_CACHE_LRU ? 1 : 0));
   prof_phase(s, st, &s->prof_open, -1);
   return LMI_OK;
 }

@@ -505,7 +505,7 @@ static int launch_misses(Server *s, Pipe &p, hipStream_t st, int seg, int seg_la
 //      is done.
 // With 1 and 2 the caller's stream does not wait here: the next call on this pipe,
 // or lmi_batch_wait, joins.  The LRU cache joins at once (its insert copies the rows).
-int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last) {
+int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last, int lru_lists) {
   const bool have_cache = s->cache_kind != LMI_CACHE_NONE;
   int mode = (s->feat_loc == LMI_LOC_HOST && have_cache) ? s->split_miss : 0;
   // The gather kernels carry their own profiling events (prof_kernel_events); a bracket
@@ -514,6 +514,7 @@ int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last)
   if (mode == 0) {
     if (have_cache) LMI_TRY(launch_hits(s, p, st, seg, seg_last));
     LMI_TRY(launch_misses(s, p, st, seg, seg_last));
+    if (lru_lists > 0) LMI_TRY(launch_lru_insert(s, p, st, lru_lists));
     return LMI_OK;
   }
   hipEvent_t fork = closing;  // when mode 2 forks right here, the closing event doubles as the fork
@@ -528,9 +529,11 @@ int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last)
   LMI_HIP(hipStreamWaitEvent(s->side, fork, 0));
   if (mode == 2) LMI_TRY(launch_hits(s, p, s->side, seg, seg_last));
   LMI_TRY(launch_misses(s, p, s->side, seg, seg_last));
+  if (lru_lists > 0) LMI_TRY(launch_lru_insert(s, p, s->side, lru_lists));  // reads the rows just gathered
   LMI_HIP(hipEventRecord(p.join, s->side));
   p.side_pending = true;
-  if (s->cache_kind == LMI_CACHE_LRU) LMI_TRY(pipe_join(p, st));
+  // an LRU insertion that comes later on the caller's stream copies the gathered rows: join now
+  if (s->cache_kind == LMI_CACHE_LRU && lru_lists == 0) LMI_TRY(pipe_join(p, st));
   return LMI_OK;
 }
 
@@ -629,6 +632,21 @@ int launch_lru_insert(Server *s, Pipe &p, hipStream_t st, int n_lists) {
     m.n_max = s->node_cap[s->cfg.hops];
     LMI_TRY(launch_move_rows(s, st, m, false));
   }
+  LMI_HIP(hipEventRecord(s->lru_ready, st));
+  s->lru_pending = true;
+  return LMI_OK;
+}
+
+// The LRU state is batch-synchronous: a lookup sees the cache after the previous batch's
+// insertion.  Sampling does not touch the cache, so only the lookup has to wait.
+int lru_wait_ready(Server *s, hipStream_t st) {
+  if (s->cache_kind != LMI_CACHE_LRU || !s->lru_pending) return LMI_OK;
+  if (hipEventQuery(s->lru_ready) == hipSuccess) {
+    s->lru_pending = false;
+    return LMI_OK;
+  }
+  (void)hipGetLastError();  // "not ready" is an answer, not a failure
+  LMI_HIP(hipStreamWaitEvent(st, s->lru_ready, 0));
   return LMI_OK;
 }
 
@@ -757,6 +775,8 @@ int launch_table_clear(Table &t, hipStream_t st) {
 }
 
 void cache_free(Server *s) {
+  (void)hipDeviceSynchronize();  // batches in flight (side stream included) still read the old cache
+  s->lru_pending = false;
   if (s->cache_data) (void)hipFree(s->cache_data);
   if (s->cache_scale) (void)hipFree(s->cache_scale);
   if (s->id_table.slots) (void)hipFree(s->id_table.slots);

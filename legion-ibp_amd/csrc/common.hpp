@@ -150,6 +150,8 @@ struct Server {
   int32_t lru_ways = 0;
   int32_t lru_tick = 0;
   int32_t *lru_keys = nullptr, *lru_use = nullptr, *lru_claim[2] = {nullptr, nullptr};
+  hipEvent_t lru_ready = nullptr;  // recorded behind every LRU insertion: the next lookup waits for it
+  bool lru_pending = false;        // an insertion may still be running
   // pipes
   std::vector<Pipe> pipes;
   hipStream_t side = nullptr;  // server-owned second stream for gathers that must not hold up the caller's stream
@@ -222,8 +224,11 @@ void cache_free(Server *s);
 // it on the side stream instead, ahead of the host-link gather, measured 2 % slower.)
 int launch_lookup(Server *s, Pipe &p, hipStream_t st, int seg_first, int seg_last);
 int launch_hotness(Server *s, Pipe &p, hipStream_t st);
-int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last);
+// lru_lists > 0: the LRU insertion of that many miss lists follows the gather on the stream the
+// misses were gathered on (the side stream when it is in use), and the caller's stream does not wait.
+int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last, int lru_lists);
 int launch_lru_insert(Server *s, Pipe &p, hipStream_t st, int n_lists);
+int lru_wait_ready(Server *s, hipStream_t st);  // orders `st` behind the last LRU insertion
 int pipe_join(Pipe &p, hipStream_t st);  // make `st` wait for the pipe's side-stream work
 int cache_dump(Server *s, int32_t *slot_of, int64_t n, int32_t *aux);
 

@@ -327,6 +327,51 @@ def test_lru_cache_parity(lmi, oracle, n_sets, ways):
         feats.free()
 
 
+@pytest.mark.parametrize("schedule", [0, 1, 2])
+def test_lru_batches_in_flight_on_two_pipes(lmi, oracle, schedule):
+    """Four batches are issued back to back on alternating pipes before any is read: the
+    sampling of a batch may overlap the host-link gather and the insertion of the one before
+    it, but every lookup sees the cache after the previous batch's insertion."""
+    rng = np.random.default_rng(77 + schedule)
+    n_nodes, batch, fanout, dim = 4000, 256, [6, 4], 64
+    indptr, indices = random_graph(rng, n_nodes, 8, hubs=4, hub_deg=300)
+    feats = make_features(lmi, rng, n_nodes, dim)
+    hot = rng.choice(n_nodes, 400, replace=False)
+    srv = lmi.Server(batch, fanout, dim, pipes=2)
+    lru = oracle.Lru(96, 4, dim * 4)
+    host_rows = feats.array.view(np.uint8).reshape(n_nodes, dim * 4)
+    stream = lmi.stream_create()
+    try:
+        srv.tune("split_miss", schedule)
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        srv.build_lru_cache(96, 4)
+        for rnd in range(5):
+            group = []
+            for k in range(4):
+                seeds = np.concatenate([rng.choice(hot, 200, replace=False), rng.choice(n_nodes, 56, replace=False)])
+                seeds = np.array(list(dict.fromkeys(seeds.tolist())), np.int32)
+                group.append(seeds)
+            # two in flight at a time (a pipe's buffers are reused by the batch after next)
+            for half in (0, 2):
+                for k in (half, half + 1):
+                    srv.run_once(group[k], rng_seed=100 + rnd * 4 + k, pipe=k % 2, stream=stream)
+                for k in (half, half + 1):
+                    g = srv.fetch(pipe=k % 2, stream=stream)
+                    o = oracle.sample_batch(indptr, indices, group[k], fanout, 100 + rnd * 4 + k)
+                    assert_batch_equal(g, o)
+                    hit, fill, out = lru.access(o.ids, host_rows)
+                    np.testing.assert_array_equal(g.cache_index, hit)
+                    assert g.features.tobytes() == out.tobytes()
+        keys, use = srv.cache_dump(96 * 4, with_aux=True)
+        okeys, ouse = lru.state()
+        np.testing.assert_array_equal(keys, okeys)
+        np.testing.assert_array_equal(use, ouse)
+    finally:
+        srv.close()
+        feats.free()
+
+
 def test_lru_operator_chain(lmi, oracle):
     rng = np.random.default_rng(3)
     n_nodes, batch, fanout, dim = 800, 40, [4, 3], 16
