@@ -106,7 +106,7 @@ typedef struct lmi_profile {
   double  gather_miss_ms;  int64_t gather_miss_launches; int64_t gather_miss_rows;
   double  sample_ms;       int64_t sample_launches;      /* all kernels of the sampling hops */
   double  lookup_ms;       int64_t lookup_launches;
-  double  batch_ms;        int64_t batches;              /* whole lmi_run_once */
+  double  batch_ms;        int64_t batches;              /* reserved (0) */
 } lmi_profile;
 
 /* ---- lifecycle ------------------------------------------------------- */

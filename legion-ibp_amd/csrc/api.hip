@@ -30,22 +30,6 @@ static hipEvent_t prof_event(Server *s) {
   return e;
 }
 
-int prof_begin(Server *s, hipStream_t st, int kind) {
-  if (!s->prof_on) return -1;
-  EventPair p{prof_event(s), prof_event(s), kind};
-  s->prof_used.push_back(p.a);
-  s->prof_used.push_back(p.b);
-  (void)hipEventRecord(p.a, st);
-  s->prof_events.push_back(p);
-  return (int)s->prof_events.size() - 1;
-}
-
-int prof_end(Server *s, hipStream_t st, int handle) {
-  if (handle < 0) return LMI_OK;
-  (void)hipEventRecord(s->prof_events[handle].b, st);
-  return LMI_OK;
-}
-
 // Ends the open bracket of a stream and starts one of kind `next_kind` (-1: none) with a
 // single event record; returns that event, or nullptr when nothing was recorded.  Level 2
 // brackets only the gather kernels, so the sampling kernels run back to back as they do
@@ -739,7 +723,7 @@ int lmi_profile_read(lmi_server *h, lmi_profile *out, int reset) {
   }
   for (auto &ev : s->prof_used) s->prof_free.push_back(ev);
   s->prof_used.clear();
-  s->prof_open = s->prof_open_side = -1;
+  s->prof_open = -1;
   s->prof_events.clear();
   unsigned long long rows[2] = {0, 0};
   LMI_HIP(hipMemcpy(rows, s->d_prof_rows, 16, hipMemcpyDeviceToHost));

@@ -180,18 +180,15 @@ struct Server {
   std::vector<hipEvent_t> prof_used;    // every event recorded since the last read (pairs may share one)
   std::vector<hipEvent_t> prof_free;    // recycled events
   int prof_open = -1;                   // pair still waiting for its end event on the caller's stream
-  int prof_open_side = -1;              // the same for the side stream
   unsigned long long *d_prof_rows = nullptr;  // device counters: [0] rows offered to hit gathers, [1] miss rows
   lmi_profile prof{};
   int32_t *d_scalar = nullptr;          // small device scratch (counts for build-time launches)
   int n_cu = 256;
 };
 
-enum { PROF_GATHER_HIT = 0, PROF_GATHER_MISS = 1, PROF_SAMPLE = 2, PROF_LOOKUP = 3, PROF_BATCH = 4 };
+enum { PROF_GATHER_HIT = 0, PROF_GATHER_MISS = 1, PROF_SAMPLE = 2, PROF_LOOKUP = 3 };
 
 // profiling helpers (api.hip)
-int prof_begin(Server *s, hipStream_t st, int kind);
-int prof_end(Server *s, hipStream_t st, int handle);
 // One event closes the pair left open on the caller's stream and opens the next
 // phase (next_kind < 0: only close), so a batch costs one event per phase boundary.
 hipEvent_t prof_phase(Server *s, hipStream_t st, int *open, int next_kind);
