@@ -285,6 +285,8 @@ struct LookupArgs {
   int2 *miss_list;
   DevState *st;
   int seg_first, seg_last, seg;
+  const HashSlot *dedup;  // the batch's dedup table: value of a seed id = its first row
+  int dedup_log2cap;
   int lookup_blocks;  // blocks [0, lookup_blocks) look rows up, the rest carry `fill`
   FillArgs fill;      // last step of the hop sampled just before (hop -1: none)
 };
@@ -338,7 +340,9 @@ static __global__ __launch_bounds__(kLookupBlock) void lookup_kernel(LookupArgs 
           for (int w = 0; w < a.lru_ways; ++w)
             if (a.lru_keys[base + w] == id) slot = (int)(base + w);
           if (slot >= 0) a.lru_use[slot] = a.st->lru_tick;
-          a.lru_fill[i] = -1;
+          // a repeated seed keeps both rows, but the id is offered for insertion once, by its first row
+          const bool repeat = i < a.st->n_seeds && table_find(a.dedup, a.dedup_log2cap, id) != i;
+          a.lru_fill[i] = repeat ? -2 : -1;
         } else if (a.kind != LMI_CACHE_NONE) {
           slot = static_find(a.table_kind, a.slots, a.log2cap, a.slot_of, a.rank_tab, id);
         }
@@ -385,6 +389,8 @@ int launch_lookup(Server *s, Pipe &p, hipStream_t st, int seg_first, int seg_las
   const int64_t base = seg_list_base(s, seg_first);
   a.miss_list = p.miss_list + base;
   a.lru_fill = p.lru_fill;
+  a.dedup = p.dedup.slots;
+  a.dedup_log2cap = p.dedup.log2cap;
   a.st = p.st;
   a.seg_first = seg_first;
   a.seg_last = seg_last;
@@ -558,6 +564,7 @@ static __global__ __launch_bounds__(256) void lru_bid_kernel(LruArgs a) {
     const int n = a.st->n_miss[l];
     for (int j = blockIdx.x * blockDim.x + threadIdx.x; j < n; j += gridDim.x * blockDim.x) {
       const int i = a.miss_list[l][j].x;
+      if (a.fill[i] != -1) continue;  // the later row of a repeated seed
       atomicMin(&a.claim_cur[(int64_t)a.ids[i] % a.sets], i);
     }
   }

@@ -319,6 +319,9 @@ void orc_lru_access(void *lru, const int32_t *ids, int64_t n, int32_t *hit_slot,
     fill_slot[i] = -1;
     if (hit_slot[i] >= 0) continue;
     const int64_t base = ((int64_t)ids[i] % c->sets) * c->ways;
+    bool placed = false;  // an id that appears twice in the batch (a repeated seed) is inserted once
+    for (int32_t w = 0; w < c->ways; ++w) placed = placed || c->keys[base + w] == ids[i];
+    if (placed) continue;
     int32_t best = -1;
     for (int32_t w = 0; w < c->ways; ++w)
       if (c->last_use[base + w] < t && (best < 0 || c->last_use[base + w] < c->last_use[base + best]))

@@ -77,7 +77,8 @@ void orc_static_cache_build_keys(const int64_t *keys, int64_t n_nodes, int64_t c
 void *orc_lru_create(int64_t n_sets, int32_t ways, int64_t row_bytes);
 void  orc_lru_destroy(void *lru);
 /* One batch.  hit_slot[i] = slot or -1 (state before the batch);
- * fill_slot[i] = slot a missing id was inserted into, or -1.
+ * fill_slot[i] = slot a missing id was inserted into, or -1.  An id that appears
+ * more than once in the batch is inserted once, by its first position.
  * If host_rows/out are non-null, also gathers: hits from the cache's own row
  * store, misses from host_rows, and copies inserted rows into the store. */
 void  orc_lru_access(void *lru, const int32_t *ids, int64_t n,

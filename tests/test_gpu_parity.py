@@ -372,6 +372,40 @@ def test_lru_batches_in_flight_on_two_pipes(lmi, oracle, schedule):
         feats.free()
 
 
+@pytest.mark.parametrize("n_sets,ways", [(1, 2), (3, 4), (40, 2)])
+def test_lru_with_repeated_seeds(lmi, oracle, n_sets, ways):
+    """A repeated seed keeps both of its rows, but its id is offered to the cache once."""
+    rng = np.random.default_rng(n_sets + ways)
+    n_nodes, batch, fanout, dim = 600, 64, [4, 2], 8
+    indptr, indices = random_graph(rng, n_nodes, 5)
+    feats = make_features(lmi, rng, n_nodes, dim)
+    srv = lmi.Server(batch, fanout, dim)
+    lru = oracle.Lru(n_sets, ways, dim * 4)
+    host_rows = feats.array.view(np.uint8).reshape(n_nodes, dim * 4)
+    try:
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        srv.build_lru_cache(n_sets, ways)
+        for it in range(8):
+            seeds = rng.integers(0, 60, batch).astype(np.int32)      # 64 draws from 60 ids: many repeats
+            srv.run_once(seeds, rng_seed=it + 1)
+            g = srv.fetch()
+            o = oracle.sample_batch(indptr, indices, seeds, fanout, it + 1)
+            assert_batch_equal(g, o)
+            hit, fill, out = lru.access(o.ids, host_rows)
+            np.testing.assert_array_equal(g.cache_index, hit)
+            assert g.features.tobytes() == out.tobytes()
+            keys, use = srv.cache_dump(n_sets * ways, with_aux=True)
+            okeys, ouse = lru.state()
+            np.testing.assert_array_equal(keys, okeys)
+            np.testing.assert_array_equal(use, ouse)
+            live = keys[keys >= 0]
+            assert len(set(live.tolist())) == len(live)              # no id cached twice
+    finally:
+        srv.close()
+        feats.free()
+
+
 def test_lru_operator_chain(lmi, oracle):
     rng = np.random.default_rng(3)
     n_nodes, batch, fanout, dim = 800, 40, [4, 3], 16

@@ -216,6 +216,9 @@ class PyLru:
                 fill.append(-1)
                 continue
             ways = self.tab[v % self.sets]
+            if any(ways[w][0] == v for w in range(self.ways)):   # an id repeated in the batch: placed by its first row
+                fill.append(-1)
+                continue
             cands = sorted((ways[w][1], w) for w in range(self.ways) if ways[w][1] < self.t)
             if not cands:
                 fill.append(-1)
@@ -234,9 +237,11 @@ def test_lru_trace_replay(oracle, sets, ways):
     hot = rng.choice(1000, 130, replace=False)
     lru, ref = oracle.Lru(sets, ways, 8), PyLru(sets, ways)
     rows = rng.integers(0, 255, (1000, 8)).astype(np.uint8)
-    for _ in range(40):
+    for it in range(40):
         ids = np.unique(np.concatenate([rng.choice(hot, 115), rng.choice(1000, 13)])).astype(np.int32)
         rng.shuffle(ids)
+        if it % 4 == 3:                                          # ids repeated within a batch (repeated seeds)
+            ids = np.concatenate([ids, ids[:9], ids[3:5]])
         hit, fill, out = lru.access(ids, rows)
         rhit, rfill = ref.access(ids.tolist())
         assert hit.tolist() == rhit and fill.tolist() == rfill
