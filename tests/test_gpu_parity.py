@@ -58,11 +58,11 @@ def test_sample_batch_parity(lmi, oracle, fanout, n_nodes, mean_deg, batch):
         feats.free()
 
 
-@pytest.mark.parametrize("case", range(24))
+@pytest.mark.parametrize("case", range(96))
 def test_random_shapes_sweep(lmi, oracle, case):
     """Seeded sweep over shapes the fixed cases do not reach: one-node and two-node graphs,
     edgeless graphs, batches of one seed, repeated seeds, fan-outs 1..64 in any order, hubs with
-    more than 2^16 neighbours, with and without a static cache, on a stream or not."""
+    more than 2^16 neighbours; static, LRU, int8 or no cache; on a stream or not, two pipes."""
     rng = np.random.default_rng(1000 + case)
     hops = int(rng.integers(1, 4))
     fanout = [int(rng.choice([1, 2, 3, 5, 8, 16, 25, 33, 64])) for _ in range(hops)]
@@ -74,27 +74,50 @@ def test_random_shapes_sweep(lmi, oracle, case):
                                    zero_frac=float(rng.choice([0.0, 0.3])))
     dim = int(rng.choice([4, 20, 128]))
     feats = make_features(lmi, rng, n_nodes, dim)
+    host_rows = feats.array.view(np.uint8).reshape(n_nodes, dim * 4)
     srv = lmi.Server(batch, fanout, dim, pipes=2, seed=5)
     stream = lmi.stream_create() if case % 2 else None
-    slot_ref = None
+    kind = ["static", "lru", "int8", "none"][case % 4]
+    slot_ref = lru = q = sc = None
     try:
         if case % 3 == 0:
             srv.tune("use_graph", 1)
         srv.load_graph(indptr, indices)
         srv.attach_features(feats)
-        if case % 4 != 3:
-            cap = int(rng.integers(1, n_nodes + 1))
+        cap = int(rng.integers(1, n_nodes + 1))
+        if kind == "static":
             srv.build_static_cache(cap, int(rng.integers(0, 3)))
             slot_ref = oracle.static_cache_build(indptr, cap)
+        elif kind == "int8":
+            srv.build_int8_cache(cap, int(rng.integers(0, 3)))
+            slot_ref = oracle.static_cache_build(indptr, cap)
+            q, sc = oracle.quantize_rows(feats.array[np.flatnonzero(slot_ref >= 0)])
+        elif kind == "lru":
+            n_sets, ways = int(rng.integers(1, 40)), int(rng.choice([1, 2, 8]))
+            srv.build_lru_cache(n_sets, ways)
+            lru = oracle.Lru(n_sets, ways, dim * 4)
         for it in range(3):
             seeds = rng.integers(0, n_nodes, int(rng.integers(1, batch + 1))).astype(np.int32)   # repeats allowed
             srv.run_once(seeds, rng_seed=50 + it, pipe=it % 2, stream=stream)
             g = srv.fetch(pipe=it % 2, stream=stream)
             o = oracle.sample_batch(indptr, indices, seeds, fanout, 50 + it)
             assert_batch_equal(g, o)
-            assert g.features.tobytes() == feats.array[o.ids].tobytes()
-            if slot_ref is not None:
+            if kind == "lru":
+                hit, fill, out = lru.access(o.ids, host_rows)
+                np.testing.assert_array_equal(g.cache_index, hit)
+                assert g.features.tobytes() == out.tobytes()
+            elif kind == "int8":
                 np.testing.assert_array_equal(g.cache_index, slot_ref[o.ids])
+                assert g.features.tobytes() == oracle.gather_rows_int8(o.ids, slot_ref[o.ids], q, sc, feats.array).tobytes()
+            else:
+                assert g.features.tobytes() == feats.array[o.ids].tobytes()
+                if slot_ref is not None:
+                    np.testing.assert_array_equal(g.cache_index, slot_ref[o.ids])
+        if kind == "lru":
+            keys, use = srv.cache_dump(lru.n_sets * lru.ways, with_aux=True)
+            okeys, ouse = lru.state()
+            np.testing.assert_array_equal(keys, okeys)
+            np.testing.assert_array_equal(use, ouse)
     finally:
         srv.close()
         feats.free()
