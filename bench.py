@@ -321,7 +321,10 @@ def main():
                     traffic=recorded_traffic(args.workload) if args.scale == 1.0 else None,
                     rows_per_launch=round(hit_rows, 1), bytes_per_row=hit_bytes, avg_launch_ms=round(hit_ms, 4),
                     measured_copy_gbs=round(copy_gbs, 1))
+    link_bytes = min(1 << 28, info["feats"].nbytes)
+    link_ms = lmi.bench_host_read(info["feats"], link_bytes)
     host_link = dict(bound="host-link", kernel="move_rows_kernel<u32x4,32,1,true,true> (host-link gather of misses)",
+                     measured_stream_read_gbs=round(link_bytes // 16 * 16 / (link_ms * 1e-3) / 1e9, 2),
                      achieved=round(miss_rows * rb / (miss_ms * 1e-3) / 1e9, 2) if miss_ms > 0 else 0.0,
                      peak=HOST_LINK_PEAK_GBS, unit="GB/s", rows_per_launch=round(miss_rows, 1),
                      avg_launch_ms=round(miss_ms, 4))

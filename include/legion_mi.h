@@ -230,6 +230,9 @@ int lmi_tune(lmi_server *s, const char *key, int64_t value);
 /* Plain device copy of `bytes` bytes, repeated; returns mean ms per copy
  * (the measured HBM ceiling quoted beside the nominal peak). */
 int lmi_bench_copy(size_t bytes, int repeats, double *ms_per_copy);
+/* Streaming zero-copy read of `bytes` bytes of pinned host memory (from lmi_host_alloc) into
+ * HBM, repeated; returns mean ms per pass (the measured host-link ceiling). */
+int lmi_bench_host_read(const void *host_ptr, size_t bytes, int repeats, double *ms_per_pass);
 
 /* ---- synthetic inputs (stand-in for the reference's dataset tooling) ---- */
 /* Power-law graph generated in HBM: degree(v) by inverse-CDF lookup of a Philox

@@ -756,6 +756,28 @@ int lmi_tune(lmi_server *h, const char *key, int64_t value) {
   return LMI_OK;
 }
 
+int lmi_bench_host_read(const void *host_ptr, size_t bytes, int repeats, double *ms_per_pass) {
+  if (!host_ptr || !ms_per_pass || repeats < 1 || bytes < 16) LMI_FAIL(LMI_ERR_ARG, "bad argument");
+  void *b = nullptr;
+  LMI_HIP(hipMalloc(&b, bytes));
+  hipEvent_t e0, e1;
+  LMI_HIP(hipEventCreate(&e0));
+  LMI_HIP(hipEventCreate(&e1));
+  const size_t n = bytes / 16;
+  hipLaunchKernelGGL(copy_kernel, dim3(1024), dim3(256), 0, 0, (const cp_u32x4 *)host_ptr, (cp_u32x4 *)b, n);
+  LMI_HIP(hipEventRecord(e0, 0));
+  for (int r = 0; r < repeats; ++r)
+    hipLaunchKernelGGL(copy_kernel, dim3(1024), dim3(256), 0, 0, (const cp_u32x4 *)host_ptr, (cp_u32x4 *)b, n);
+  LMI_HIP(hipEventRecord(e1, 0));
+  LMI_HIP(hipEventSynchronize(e1));
+  float ms = 0;
+  LMI_HIP(hipEventElapsedTime(&ms, e0, e1));
+  *ms_per_pass = ms / repeats;
+  (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
+  (void)hipFree(b);
+  return LMI_OK;
+}
+
 int lmi_bench_copy(size_t bytes, int repeats, double *ms_per_copy) {
   if (!ms_per_copy || repeats < 1 || bytes < 16) LMI_FAIL(LMI_ERR_ARG, "bad argument");
   void *a = nullptr, *b = nullptr;
