@@ -484,6 +484,22 @@ static int batch_params(Server *s, Pipe &p, hipStream_t st, const int32_t *seeds
     if (s->set_labels[mode]) bp->labels = s->set_labels[mode] + off;
   }
   bp->n_seeds = n;
+  // dedup-table epoch: keys carry it in the bits above the widest node id, so the table is
+  // wiped only when the epochs run out (or it is new, or the id width changed)
+  int id_bits = 1;
+  while (id_bits < 31 && (int64_t(1) << id_bits) < s->n_nodes) ++id_bits;
+  const int32_t max_epoch = (int32_t)std::min<int64_t>((int64_t(1) << (31 - id_bits)) - 1, s->table_epochs);  // 0: wipe every batch
+  if (p.table_dirty || p.epoch >= max_epoch || p.id_bits != id_bits) {
+    p.epoch = 0;
+    bp->clear_table = 1;
+  } else {
+    ++p.epoch;
+    bp->clear_table = 0;
+  }
+  p.table_dirty = false;
+  p.id_bits = id_bits;
+  bp->table_tag = max_epoch > 0 ? (int32_t)((uint32_t)p.epoch << id_bits) : 0;
+  bp->table_mask = max_epoch > 0 ? (int32_t)(0xFFFFFFFFu << id_bits) : kUntaggedMask;
   bp->rng_seed = rng_seed ? rng_seed : s->cfg.seed + (uint64_t)(uint32_t)batch_counter;
   if (s->cache_kind == LMI_CACHE_LRU) ++s->lru_tick;
   bp->lru_tick = s->lru_tick;
@@ -746,6 +762,10 @@ int lmi_tune(lmi_server *h, const char *key, int64_t value) {
   else if (!strcmp(key, "gather_nontemporal")) s->gather_nt = (int)value;
   else if (!strcmp(key, "lds_dedup")) s->lds_dedup = (int)value;
   else if (!strcmp(key, "fuse_count")) s->fuse_count = (int)value;
+  else if (!strcmp(key, "table_epochs")) {
+    s->table_epochs = std::max<int64_t>(0, value);
+    for (auto &p : s->pipes) p.table_dirty = true;
+  }
   else if (!strcmp(key, "profile_every")) s->prof_every = (int)std::max<int64_t>(1, value);
   else if (!strcmp(key, "fuse_small_max")) s->fuse_small_max = value;
   else if (!strcmp(key, "split_miss")) s->split_miss = (int)value;

@@ -341,7 +341,8 @@ static __global__ __launch_bounds__(kLookupBlock) void lookup_kernel(LookupArgs 
             if (a.lru_keys[base + w] == id) slot = (int)(base + w);
           if (slot >= 0) a.lru_use[slot] = a.st->lru_tick;
           // a repeated seed keeps both rows, but the id is offered for insertion once, by its first row
-          const bool repeat = i < a.st->n_seeds && table_find(a.dedup, a.dedup_log2cap, id) != i;
+          const bool repeat = i < a.st->n_seeds &&
+                              table_find(a.dedup, a.dedup_log2cap, id, a.st->table_tag, a.st->table_mask) != i;
           a.lru_fill[i] = repeat ? -2 : -1;
         } else if (a.kind != LMI_CACHE_NONE) {
           slot = static_find(a.table_kind, a.slots, a.log2cap, a.slot_of, a.rank_tab, id);

@@ -14,6 +14,7 @@ namespace lmi {
 
 constexpr int kWave = 64;
 constexpr int32_t kEmptyKey = -1;
+constexpr int32_t kUntaggedMask = (int32_t)0x80000000u;  // tag mask of an untagged table: only key -1 is free
 constexpr int32_t kIntMax = 0x7fffffff;
 
 // ---------------------------------------------------------------- errors
@@ -57,6 +58,7 @@ struct DevState {
   uint32_t rng_lo, rng_hi;   // 64-bit Philox key of this batch
   int32_t lru_tick;
   int32_t n_seeds;
+  int32_t table_tag, table_mask;  // epoch tag of this batch's dedup-table keys (table_insert_min)
   const int32_t *seeds;      // device address of this batch's seed ids
   const int32_t *labels_in;  // device address of their labels (or null)
 };
@@ -86,6 +88,9 @@ struct Pipe {
   Table dedup;                 // global id -> local id (per batch)
   int32_t *eslot[2] = {nullptr, nullptr};  // [max_edges_hop] table slot of each edge's source; hops alternate
                                            // so that a hop's slots survive into the next hop's first kernel
+  int32_t epoch = 0;           // dedup-table epoch of the last batch
+  int id_bits = 0;             // key bits below the epoch tag when that batch ran
+  bool table_dirty = true;     // the table must be wiped before its next use
   int fill_pending = -1;       // hop whose edge sources still wait for their local ids (launch_fill)
   unsigned long long *chain_status[2] = {nullptr, nullptr};  // look-back scan state: [0] node scans, [1] edge scans
   int32_t max_tiles = 0;
@@ -106,6 +111,9 @@ struct Pipe {
 struct BatchParams {
   int32_t n_seeds;
   int32_t lru_tick;
+  int32_t table_tag, table_mask;  // see table_insert_min
+  int32_t clear_table;            // 1: the epochs ran out (or the table is new): wipe it first
+  int32_t pad;
   uint64_t rng_seed;
   const int32_t *seeds;
   const int32_t *labels;
@@ -162,6 +170,8 @@ struct Server {
   int gather_blocks = 0;  // 0 = auto
   int gather_nt = 1;      // non-temporal output stores
   int64_t fuse_small_max = 32768;  // hops of at most this many nodes use the small tile of hop_tile_nodes
+  int64_t table_epochs = int64_t(1) << 30;  // batches a dedup table serves between wipes, less one (also
+                                            // bounded by the key bits the node ids leave free)
   int fuse_count = 1;     // 1: row counts, their scan and the sampling of a hop share one launch
   int lds_dedup = 0;      // 1: hop_sample stages its probes through an LDS hash table
   int split_miss = 1;     // gather schedule, see launch_gather_seg

@@ -39,25 +39,33 @@ __device__ __forceinline__ uint32_t hash_id(int32_t key, int log2cap) {
   return ((uint32_t)key * 0x9E3779B1u) >> (32 - log2cap);
 }
 
+// A stored key is `key | tag`: the tag (an epoch number in the bits above the widest id)
+// says which batch wrote the slot.  A slot whose tag bits differ from the current tag is
+// free -- never written (key -1: every tag bit set) or left by an earlier batch -- so the
+// table needs no clearing between batches until the epochs run out.  Untagged tables use
+// tag 0 with the sign bit as mask: only the empty key -1 is free.
 // Insert `key` (if absent) and lower its value to min(value, cand); returns the
-// slot index.  One 8-byte load reads key and value together.  Keys only ever go
-// EMPTY -> key, so a stale non-empty read is still correct and a stale EMPTY read
-// is resolved by the CAS.  Values only ever decrease, so a stale value is never
-// too low: when the value read is already <= cand the atomic can be skipped, which
-// removes almost all same-address atomics on frequently sampled hub nodes.
-__device__ __forceinline__ uint32_t table_insert_min(HashSlot *slots, int log2cap, int32_t key,
-                                                     int32_t cand) {
+// slot index.  One 8-byte load reads key and value together; a free slot is claimed
+// with one 8-byte compare-and-swap that writes key and value at once.  Within a batch
+// a slot only ever goes free -> key, so a stale non-free read is still correct and a
+// stale free read is resolved by the CAS.  Values only ever decrease, so a stale value
+// is never too low: when the value read is already <= cand the atomic can be skipped,
+// which removes almost all same-address atomics on frequently sampled hub nodes.
+__device__ __forceinline__ uint32_t table_insert_min(HashSlot *slots, int log2cap, int32_t key, int32_t cand,
+                                                     int32_t tag = 0, int32_t tag_mask = kUntaggedMask) {
   const uint32_t mask = (1u << log2cap) - 1u;
+  const int32_t stored = key | tag;
   uint32_t h = hash_id(key, log2cap);
   while (true) {
-    const int2 kv = *reinterpret_cast<const int2 *>(&slots[h]);
-    int32_t k = kv.x, v = kv.y;
-    if (k == kEmptyKey) {
-      k = atomicCAS(&slots[h].key, kEmptyKey, key);
-      if (k == kEmptyKey) k = key;
-      v = kIntMax;  // unknown: take the atomic path
+    unsigned long long *word = reinterpret_cast<unsigned long long *>(&slots[h]);
+    const unsigned long long raw = *reinterpret_cast<const volatile unsigned long long *>(word);
+    const int32_t k = (int32_t)(uint32_t)raw, v = (int32_t)(uint32_t)(raw >> 32);
+    if ((k & tag_mask) != tag) {  // free: claim it with key and value together
+      const unsigned long long mine = (unsigned long long)(uint32_t)stored | ((unsigned long long)(uint32_t)cand << 32);
+      if (atomicCAS(word, raw, mine) == raw) return h;
+      continue;  // somebody else took it: look at what it holds now
     }
-    if (k == key) {
+    if (k == stored) {
       if (v > cand) atomicMin(&slots[h].val, cand);
       return h;
     }
@@ -66,13 +74,15 @@ __device__ __forceinline__ uint32_t table_insert_min(HashSlot *slots, int log2ca
 }
 
 // Read-only probe: value or -1.
-__device__ __forceinline__ int32_t table_find(const HashSlot *slots, int log2cap, int32_t key) {
+__device__ __forceinline__ int32_t table_find(const HashSlot *slots, int log2cap, int32_t key, int32_t tag = 0,
+                                              int32_t tag_mask = kUntaggedMask) {
   const uint32_t mask = (1u << log2cap) - 1u;
+  const int32_t stored = key | tag;
   uint32_t h = hash_id(key, log2cap);
   while (true) {
     const int2 kv = *reinterpret_cast<const int2 *>(&slots[h]);
-    if (kv.x == key) return kv.y;
-    if (kv.x == kEmptyKey) return -1;
+    if (kv.x == stored) return kv.y;
+    if ((kv.x & tag_mask) != tag) return -1;
     h = (h + 1) & mask;
   }
 }

@@ -61,9 +61,11 @@ static __global__ __launch_bounds__(256) void batch_begin_kernel(HashSlot *slots
   const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   // two slots (16 bytes) per store
-  const int4 fill = make_int4(kEmptyKey, kIntMax, kEmptyKey, kIntMax);
-  int4 *p = reinterpret_cast<int4 *>(slots);
-  for (int64_t i = tid; i < n_slots / 2; i += stride) p[i] = fill;
+  if (bp.clear_table) {
+    const int4 fill = make_int4(kEmptyKey, kIntMax, kEmptyKey, kIntMax);
+    int4 *p = reinterpret_cast<int4 *>(slots);
+    for (int64_t i = tid; i < n_slots / 2; i += stride) p[i] = fill;
+  }
   scan_chain_reset(chain_nodes, max_tiles, tid, stride);
   scan_chain_reset(chain_edges, max_tiles, tid, stride);
   if (tid == 0) {
@@ -77,6 +79,8 @@ static __global__ __launch_bounds__(256) void batch_begin_kernel(HashSlot *slots
     st->rng_hi = (uint32_t)(bp.rng_seed >> 32);
     st->lru_tick = bp.lru_tick;
     st->n_seeds = bp.n_seeds;
+    st->table_tag = bp.table_tag;
+    st->table_mask = bp.table_mask;
     st->seeds = bp.seeds;
     st->labels_in = bp.labels;
   }
@@ -95,7 +99,7 @@ static __global__ __launch_bounds__(256) void batch_generate_kernel(int64_t n_no
     st->bad_id = 1;
     return;
   }
-  table_insert_min(slots, log2cap, id, i);
+  table_insert_min(slots, log2cap, id, i, st->table_tag, st->table_mask);
 }
 
 // ------------------------------------------------------------- hop, phase 1
@@ -154,7 +158,7 @@ static __global__ __launch_bounds__(kScanBlock) void hop_count_scan_kernel(HopAr
     if (a.stage_seeds) {
 #pragma unroll
       for (int j = 0; j < ITEMS; ++j)
-        if (id[j] >= 0) table_insert_min(a.slots, a.log2cap, id[j], base + j);
+        if (id[j] >= 0) table_insert_min(a.slots, a.log2cap, id[j], base + j, st->table_tag, st->table_mask);
     }
     int v[ITEMS], sum = 0;
 #pragma unroll
@@ -191,6 +195,7 @@ static __global__ __launch_bounds__(256) void hop_sample_kernel(HopArgs a) {
   const int64_t flat = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   scan_chain_reset(a.chain_edges, a.max_tiles, flat, (int64_t)gridDim.x * blockDim.x);
   const uint64_t seed = (uint64_t)st->rng_lo | ((uint64_t)st->rng_hi << 32);
+  const int32_t tag = st->table_tag, tag_mask = st->table_mask;
   const int n_prev = st->node_counter[9 + a.hop];
   const int eoff = st->edge_counter[12 + a.hop + 1];
   const int fanout = a.fanout;
@@ -225,7 +230,7 @@ static __global__ __launch_bounds__(256) void hop_sample_kernel(HopArgs a) {
       const int e = base + lane;
       a.agg_src_ids[eoff + e] = nbr;
       a.agg_dst_off[eoff + e] = i;
-      a.eslot[e] = (int)table_insert_min(a.slots, a.log2cap, nbr, n_prev + e);
+      a.eslot[e] = (int)table_insert_min(a.slots, a.log2cap, nbr, n_prev + e, tag, tag_mask);
     }
   }
 }
@@ -302,7 +307,8 @@ static __global__ __launch_bounds__(256) void hop_sample_lds_kernel(HopArgs a) {
       }
     }
     __syncthreads();
-    if (active && lds_min[h] == e) lds_slot[h] = (int)table_insert_min(a.slots, a.log2cap, nbr, n_prev + e);
+    if (active && lds_min[h] == e)
+      lds_slot[h] = (int)table_insert_min(a.slots, a.log2cap, nbr, n_prev + e, st->table_tag, st->table_mask);
     __syncthreads();
     if (active) a.eslot[e] = lds_slot[h];
     __syncthreads();
@@ -364,7 +370,7 @@ static __global__ __launch_bounds__(256) void hop_count_sample_kernel(HopArgs a)
     if (id >= 0) {
       lo = a.indptr[id];
       hi = a.indptr[id + 1];
-      if (a.stage_seeds) table_insert_min(a.slots, a.log2cap, id, my);
+      if (a.stage_seeds) table_insert_min(a.slots, a.log2cap, id, my, st->table_tag, st->table_mask);
     }
     const int64_t deg = hi - lo;
     cnt = (int)(deg < (int64_t)a.fanout ? deg : (int64_t)a.fanout);
@@ -387,6 +393,7 @@ static __global__ __launch_bounds__(256) void hop_count_sample_kernel(HopArgs a)
   __syncthreads();
   // ---- sampling: the edge offset of the hop is fixed by the hops before it
   const uint64_t seed = (uint64_t)st->rng_lo | ((uint64_t)st->rng_hi << 32);
+  const int32_t tag = st->table_tag, tag_mask = st->table_mask;
   const int eoff = (a.hop == 0) ? 0 : st->edge_counter[12 + a.hop] + st->edge_counter[9 + a.hop];
   const int fanout = a.fanout;
   const int lane = t & (G - 1);
@@ -419,7 +426,7 @@ static __global__ __launch_bounds__(256) void hop_count_sample_kernel(HopArgs a)
       const int e = base + lane;
       a.agg_src_ids[eoff + e] = nbr;
       a.agg_dst_off[eoff + e] = i;
-      a.eslot[e] = (int)table_insert_min(a.slots, a.log2cap, nbr, n_prev + e);
+      a.eslot[e] = (int)table_insert_min(a.slots, a.log2cap, nbr, n_prev + e, tag, tag_mask);
     }
   }
 }

@@ -174,6 +174,32 @@ def test_count_and_sample_in_one_launch_or_two(lmi, oracle, batch, fanout, fused
         feats.free()
 
 
+@pytest.mark.parametrize("epochs", [0, 1, 3])
+def test_dedup_table_epochs_wrap(lmi, oracle, epochs):
+    """The dedup table is wiped only when its epoch tags run out; with the number of epochs
+    capped at 0, 1 or 3 the wipe comes every batch, every 2nd or every 4th batch of a pipe, and
+    entries left by earlier batches sit in the table in between."""
+    rng = np.random.default_rng(90 + epochs)
+    n_nodes, batch, fanout = 3000, 200, [12, 6]
+    indptr, indices = random_graph(rng, n_nodes, 14, hubs=4, hub_deg=500)
+    feats = make_features(lmi, rng, n_nodes, 4)
+    srv = lmi.Server(batch, fanout, 4, pipes=2)
+    stream = lmi.stream_create()
+    try:
+        srv.tune("table_epochs", epochs)
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        for it in range(14):
+            # the same few seeds again and again: earlier batches leave exactly the keys the next one probes for
+            seeds = rng.choice(400, batch, replace=False).astype(np.int32)
+            srv.run_once(seeds, rng_seed=3 + it, pipe=it % 2, stream=stream if it % 3 else None)
+            g = srv.fetch(pipe=it % 2, stream=stream if it % 3 else None)
+            assert_batch_equal(g, oracle.sample_batch(indptr, indices, seeds, fanout, 3 + it))
+    finally:
+        srv.close()
+        feats.free()
+
+
 def test_duplicate_seeds_and_isolated_nodes(lmi, oracle):
     rng = np.random.default_rng(5)
     indptr, indices = random_graph(rng, 300, 6, zero_frac=0.4)
