@@ -102,7 +102,17 @@ __device__ __forceinline__ void fill_local_ids(const FillArgs &f, int64_t tid, i
   if (f.hop < 0) return;
   const int n = f.st->edge_counter[9 + f.hop + 1];
   const int eoff = f.st->edge_counter[12 + f.hop + 1];
-  for (int64_t e = tid; e < n; e += n_threads) f.agg_src_off[eoff + e] = f.slots[f.eslot[e]].val;
+  // four edges in flight per thread: the two dependent reads of each overlap those of the others
+  for (int64_t e = tid; e < n; e += 4 * n_threads) {
+    int32_t slot[4], val[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) slot[u] = (e + u * n_threads < n) ? f.eslot[e + u * n_threads] : 0;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) val[u] = (e + u * n_threads < n) ? f.slots[slot[u]].val : 0;
+#pragma unroll
+    for (int u = 0; u < 4; ++u)
+      if (e + u * n_threads < n) f.agg_src_off[eoff + e + u * n_threads] = val[u];
+  }
 }
 
 // ------------------------------------------------------------------- scans

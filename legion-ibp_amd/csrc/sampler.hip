@@ -642,8 +642,8 @@ FillArgs fill_args(const Pipe &p, int hop) {
   return f;
 }
 
-int fill_blocks(int64_t e_max, int block) {
-  return (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(e_max, block), 1024));
+int fill_blocks(int64_t e_max, int block) {  // four edges per thread
+  return (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(e_max, (int64_t)block * 4), 1024));
 }
 
 int launch_fill(Server *s, Pipe &p, hipStream_t st) {
