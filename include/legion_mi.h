@@ -32,7 +32,7 @@ extern "C" {
 #define LMI_ABI_VERSION 1
 #define LMI_MAX_HOPS    3   /* the 16-int headers hold 3 hops (INTRABATCH_CON, include/system_config.cuh:47-57) */
 #define LMI_MAX_FANOUT  64  /* one wavefront lane per slot; the reference asserts <= 32 (operator_impl.cu:504) */
-#define LMI_MAX_PIPES   4   /* output buffer sets; the reference uses INTERBATCH_CON = 2 */
+#define LMI_MAX_PIPES   8   /* output buffer sets; the reference uses INTERBATCH_CON = 2 */
 
 enum {
   LMI_OK = 0,
@@ -201,6 +201,16 @@ int lmi_op_io_complete(lmi_server *s, int pipe, void *stream);
  * possibly still running on the server's side stream: see lmi_batch_wait. */
 int lmi_run_once(lmi_server *s, int pipe, void *stream, const int32_t *seeds, int32_t n,
                  int seeds_location, int32_t batch_counter, int mode, uint64_t rng_seed);
+
+/* n_batches mini-batches at once, batch k into pipe pipes[k] (distinct pipes): the same as
+ * n_batches calls of lmi_run_once, but every launch of the sampling phase serves all of them
+ * (those kernels are latency-bound, so the batches after the first cost little).  seeds,
+ * n_seeds and rng_seeds may be NULL (slices batch_counters[k] of id set `mode`, default RNG
+ * seeds).  Not with the LRU cache, whose state advances batch by batch.  No counterpart in
+ * the reference, which runs one batch per RunOnce. */
+int lmi_run_group(lmi_server *s, int n_batches, const int32_t *pipes, void *stream,
+                  const int32_t *const *seeds, const int32_t *n_seeds, int seeds_location,
+                  const int32_t *batch_counters, int mode, const uint64_t *rng_seeds);
 
 /* ---- outputs ----------------------------------------------------------- */
 /* Makes `stream` wait until every output of the pipe's last batch is complete,

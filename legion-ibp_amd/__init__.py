@@ -31,7 +31,7 @@ ABI_SYMBOLS = [
     "lmi_cache_policy", "lmi_cache_build_static", "lmi_cache_build_lru", "lmi_cache_build_int8",
     "lmi_cache_info_get", "lmi_cache_dump", "lmi_op_batch_generate", "lmi_op_random_sample",
     "lmi_op_cache_lookup", "lmi_op_io_submit", "lmi_op_io_complete", "lmi_run_once",
-    "lmi_batch_wait", "lmi_batch_view_get", "lmi_batch_counters", "lmi_steps_per_epoch", "lmi_profile_enable",
+    "lmi_run_group", "lmi_batch_wait", "lmi_batch_view_get", "lmi_batch_counters", "lmi_steps_per_epoch", "lmi_profile_enable",
     "lmi_profile_read", "lmi_tune", "lmi_bench_copy", "lmi_bench_host_read", "lmi_synth_graph", "lmi_synth_trainset",
     "lmi_synth_features",
 ]
@@ -119,6 +119,8 @@ def lib():
         L.lmi_batch_wait.argtypes = [C.c_void_p, C.c_int, C.c_void_p]
         L.lmi_batch_view_get.argtypes = [C.c_void_p, C.c_int, C.POINTER(BatchView)]
         L.lmi_batch_counters.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
+        L.lmi_run_group.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
+                                    C.c_void_p, C.c_int, C.c_void_p]
         L.lmi_steps_per_epoch.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_int32)]
         L.lmi_profile_enable.argtypes = [C.c_void_p, C.c_int]
         L.lmi_profile_read.argtypes = [C.c_void_p, C.POINTER(Profile), C.c_int]
@@ -278,6 +280,19 @@ class Server:
     def run_once(self, seeds=None, batch_counter=0, mode=MODE_TRAIN, rng_seed=0, pipe=0, stream=None):
         p, n, keep = self._seed_args(seeds)
         check(lib().lmi_run_once(self.h, pipe, stream, p, n, LOC_HOST, batch_counter, mode, rng_seed))
+
+    def run_group(self, pipes, batch_counters, seeds=None, mode=MODE_TRAIN, rng_seeds=None, stream=None):
+        """One batch per listed pipe, all served by the same launches (lmi_run_group)."""
+        n = len(pipes)
+        pa = (C.c_int32 * n)(*pipes)
+        bc = (C.c_int32 * n)(*batch_counters)
+        rs = (C.c_uint64 * n)(*rng_seeds) if rng_seeds is not None else None
+        sp = ns = keep = None
+        if seeds is not None:
+            keep = [np.ascontiguousarray(x, dtype=np.int32) for x in seeds]
+            sp = (C.c_void_p * n)(*[x.ctypes.data for x in keep])
+            ns = (C.c_int32 * n)(*[len(x) for x in keep])
+        check(lib().lmi_run_group(self.h, n, pa, stream, sp, ns, LOC_HOST, bc, mode, rs))
 
     # outputs -----------------------------------------------------------------
     def batch_wait(self, pipe=0, stream=None):

@@ -516,7 +516,8 @@ int lmi_op_batch_generate(lmi_server *h, int pipe, void *stream, const int32_t *
   prof_batch(s);
   LMI_TRY(pipe_join(p, st));
   LMI_TRY(batch_params(s, p, st, seeds, n, seeds_location, batch_counter, mode, rng_seed, &bp));
-  return launch_batch_generate(s, p, st, bp, true);
+  Pipe *pp[1] = {&p};
+  return launch_batch_generate(s, pp, &bp, 1, st, true);
 }
 
 int lmi_op_random_sample(lmi_server *h, int pipe, void *stream, int hop) {
@@ -527,7 +528,8 @@ int lmi_op_random_sample(lmi_server *h, int pipe, void *stream, int hop) {
   if (hop != p.hops_done || hop >= s->cfg.hops) LMI_FAIL(LMI_ERR_ARG, "hop %d out of order (next is %d)", hop, p.hops_done);
   hipStream_t st = (hipStream_t)stream;
   prof_phase(s, st, &s->prof_open, PROF_SAMPLE);
-  LMI_TRY(launch_hop(s, p, st, hop, false, false));
+  Pipe *pp[1] = {&p};
+  LMI_TRY(launch_hop(s, pp, 1, st, hop, false, false));
   prof_phase(s, st, &s->prof_open, -1);
   return LMI_OK;
 }
@@ -542,7 +544,8 @@ int lmi_op_cache_lookup(lmi_server *h, int pipe, void *stream, int segment) {
   LMI_TRY(pipe_join(p, st));
   LMI_TRY(lru_wait_ready(s, st));
   prof_phase(s, st, &s->prof_open, PROF_LOOKUP);
-  LMI_TRY(launch_lookup(s, p, st, segment, segment));
+  Pipe *pp[1] = {&p};
+  LMI_TRY(launch_lookup(s, pp, 1, st, segment, segment));
   LMI_TRY(launch_gather_seg(s, p, st, segment, segment, 0));
   prof_phase(s, st, &s->prof_open, -1);
   return LMI_OK;
@@ -567,9 +570,10 @@ int lmi_presample(lmi_server *h, int pipe, void *stream, int mode, int32_t first
     const int tick = s->lru_tick;
     LMI_TRY(batch_params(s, p, st, nullptr, 0, LMI_LOC_DEVICE, b, mode, 0, &bp));
     s->lru_tick = tick;  // presampling does not age the LRU cache
-    LMI_TRY(launch_batch_generate(s, p, st, bp, false));
-    for (int k = 0; k < s->cfg.hops; ++k) LMI_TRY(launch_hop(s, p, st, k, true, true));
-    LMI_TRY(launch_fill(s, p, st));
+    Pipe *pp[1] = {&p};
+    LMI_TRY(launch_batch_generate(s, pp, &bp, 1, st, false));
+    for (int k = 0; k < s->cfg.hops; ++k) LMI_TRY(launch_hop(s, pp, 1, st, k, true, true));
+    LMI_TRY(launch_fill(s, pp, 1, st));
     LMI_TRY(launch_hotness(s, p, st));
   }
   return LMI_OK;
@@ -597,9 +601,10 @@ static int capture_batch_graph(Server *s, Pipe &p, hipStream_t st, const BatchPa
   const bool prof = s->prof_on;
   s->prof_on = false;  // no event records inside the capture
   LMI_HIP(hipStreamBeginCapture(st, hipStreamCaptureModeThreadLocal));
-  int rc = launch_batch_generate(s, p, st, bp, false);
-  for (int k = 0; rc == LMI_OK && k < s->cfg.hops; ++k) rc = launch_hop(s, p, st, k, true, true);
-  if (rc == LMI_OK) rc = launch_lookup(s, p, st, 0, s->cfg.hops);
+  Pipe *pp[1] = {&p};
+  int rc = launch_batch_generate(s, pp, &bp, 1, st, false);
+  for (int k = 0; rc == LMI_OK && k < s->cfg.hops; ++k) rc = launch_hop(s, pp, 1, st, k, true, true);
+  if (rc == LMI_OK) rc = launch_lookup(s, pp, 1, st, 0, s->cfg.hops);
   hipGraph_t g = nullptr;
   const hipError_t e = hipStreamEndCapture(st, &g);
   s->prof_on = prof;
@@ -623,32 +628,63 @@ static int capture_batch_graph(Server *s, Pipe &p, hipStream_t st, const BatchPa
   return LMI_OK;
 }
 
+// One batch on each of n pipes, served by the same launches.
+static int run_group(Server *s, Pipe *const *pp, const BatchParams *bps, int n, hipStream_t st) {
+  for (int k = 0; k < n; ++k) LMI_TRY(pipe_join(*pp[k], st));  // a pipe's previous batch may still be gathering misses
+  prof_phase(s, st, &s->prof_open, PROF_SAMPLE);
+  if (s->use_graph && st != nullptr && n == 1) {  // the legacy default stream cannot be captured
+    Pipe &p = *pp[0];
+    LMI_TRY(lru_wait_ready(s, st));  // the lookup sits inside the graph: the whole replay waits
+    if (!p.graph_exec) LMI_TRY(capture_batch_graph(s, p, st, bps[0]));
+    LMI_TRY(graph_update_begin(s, p, bps[0]));
+    LMI_HIP(hipGraphLaunch(p.graph_exec, st));
+  } else {
+    LMI_TRY(launch_batch_generate(s, pp, bps, n, st, false));
+    for (int k = 0; k < s->cfg.hops; ++k) LMI_TRY(launch_hop(s, pp, n, st, k, true, true));
+    LMI_TRY(lru_wait_ready(s, st));  // sampling may overlap the previous batch's insertion, the lookup may not
+    LMI_TRY(launch_lookup(s, pp, n, st, 0, s->cfg.hops));
+  }
+  LMI_TRY(launch_gather_group(s, pp, n, st, 0, s->cfg.hops, s->cache_kind == LMI_CACHE_LRU ? 1 : 0));
+  prof_phase(s, st, &s->prof_open, -1);
+  return LMI_OK;
+}
+
 int lmi_run_once(lmi_server *h, int pipe, void *stream, const int32_t *seeds, int32_t n, int seeds_location,
                  int32_t batch_counter, int mode, uint64_t rng_seed) {
   Server *s = reinterpret_cast<Server *>(h);
   LMI_TRY(check_pipe(s, pipe));
   if (!s->feat) LMI_FAIL(LMI_ERR_STATE, "no features attached");
-  Pipe &p = s->pipes[pipe];
+  Pipe *pp[1] = {&s->pipes[pipe]};
   hipStream_t st = (hipStream_t)stream;
   BatchParams bp{};
   prof_batch(s);
-  LMI_TRY(batch_params(s, p, st, seeds, n, seeds_location, batch_counter, mode, rng_seed, &bp));
-  LMI_TRY(pipe_join(p, st));  // the previous batch of this pipe may still be gathering misses
-  prof_phase(s, st, &s->prof_open, PROF_SAMPLE);
-  if (s->use_graph && st != nullptr) {  // the legacy default stream cannot be captured
-    LMI_TRY(lru_wait_ready(s, st));       // the lookup sits inside the graph: the whole replay waits
-    if (!p.graph_exec) LMI_TRY(capture_batch_graph(s, p, st, bp));
-    LMI_TRY(graph_update_begin(s, p, bp));
-    LMI_HIP(hipGraphLaunch(p.graph_exec, st));
-  } else {
-    LMI_TRY(launch_batch_generate(s, p, st, bp, false));
-    for (int k = 0; k < s->cfg.hops; ++k) LMI_TRY(launch_hop(s, p, st, k, true, true));
-    LMI_TRY(lru_wait_ready(s, st));  // sampling may overlap the previous batch's insertion, the lookup may not
-    LMI_TRY(launch_lookup(s, p, st, 0, s->cfg.hops));
+  LMI_TRY(batch_params(s, *pp[0], st, seeds, n, seeds_location, batch_counter, mode, rng_seed, &bp));
+  return run_group(s, pp, &bp, 1, st);
+}
+
+int lmi_run_group(lmi_server *h, int n_batches, const int32_t *pipes, void *stream, const int32_t *const *seeds,
+                  const int32_t *n_seeds, int seeds_location, const int32_t *batch_counters, int mode,
+                  const uint64_t *rng_seeds) {
+  Server *s = reinterpret_cast<Server *>(h);
+  if (!s || !pipes || !batch_counters) LMI_FAIL(LMI_ERR_ARG, "null argument");
+  if (n_batches < 1 || n_batches > LMI_MAX_PIPES) LMI_FAIL(LMI_ERR_ARG, "a group holds 1..%d batches", LMI_MAX_PIPES);
+  if (!s->feat) LMI_FAIL(LMI_ERR_STATE, "no features attached");
+  if (s->cache_kind == LMI_CACHE_LRU && n_batches > 1)
+    LMI_FAIL(LMI_ERR_STATE, "the LRU cache takes one batch at a time (its state is batch-synchronous)");
+  Pipe *pp[LMI_MAX_PIPES];
+  BatchParams bps[LMI_MAX_PIPES];
+  hipStream_t st = (hipStream_t)stream;
+  for (int k = 0; k < n_batches; ++k) {
+    LMI_TRY(check_pipe(s, pipes[k]));
+    for (int j = 0; j < k; ++j)
+      if (pipes[j] == pipes[k]) LMI_FAIL(LMI_ERR_ARG, "pipe %d named twice in one group", pipes[k]);
+    pp[k] = &s->pipes[pipes[k]];
   }
-  LMI_TRY(launch_gather_seg(s, p, st, 0, s->cfg.hops, s->cache_kind == LMI_CACHE_LRU ? 1 : 0));
-  prof_phase(s, st, &s->prof_open, -1);
-  return LMI_OK;
+  prof_batch(s);
+  for (int k = 0; k < n_batches; ++k)
+    LMI_TRY(batch_params(s, *pp[k], st, seeds ? seeds[k] : nullptr, (seeds && n_seeds) ? n_seeds[k] : 0, seeds_location,
+                         batch_counters[k], mode, rng_seeds ? rng_seeds[k] : 0, &bps[k]));
+  return run_group(s, pp, bps, n_batches, st);
 }
 
 int lmi_batch_wait(lmi_server *h, int pipe, void *stream) {

@@ -315,7 +315,12 @@ __device__ __forceinline__ int32_t static_find(int table_kind, const HashSlot *s
 // rows directly and skips the misses.  List order is arbitrary; it only
 // schedules the host-link gather.
 constexpr int kLookupBlock = 1024;
-static __global__ __launch_bounds__(kLookupBlock) void lookup_kernel(LookupArgs a) {
+struct LookupGroup {  // one pipe per grid row, as in the sampling kernels
+  LookupArgs p[LMI_MAX_PIPES];
+};
+
+static __global__ __launch_bounds__(kLookupBlock) void lookup_kernel(LookupGroup g) {
+  const LookupArgs &a = g.p[blockIdx.y];
   __shared__ int wave_cnt[kLookupBlock / kWave];
   __shared__ int block_base;
   if ((int)blockIdx.x >= a.lookup_blocks) {
@@ -372,40 +377,43 @@ static __global__ __launch_bounds__(kLookupBlock) void lookup_kernel(LookupArgs 
 
 static inline int64_t seg_list_base(const Server *s, int seg) { return seg == 0 ? 0 : s->node_cap[seg - 1]; }
 
-int launch_lookup(Server *s, Pipe &p, hipStream_t st, int seg_first, int seg_last) {
-  LookupArgs a{};
-  a.ids = p.ids;
-  a.n_nodes = s->n_nodes;
-  a.kind = s->cache_kind;
-  a.table_kind = s->table_kind;
-  a.slots = s->id_table.slots;
-  a.log2cap = s->id_table.log2cap;
-  a.slot_of = s->slot_of;
-  a.rank_tab = s->rank_tab;
-  a.lru_keys = s->lru_keys;
-  a.lru_use = s->lru_use;
-  a.lru_sets = s->lru_sets;
-  a.lru_ways = s->lru_ways;
-  a.cache_index = p.cache_index;
-  const int64_t base = seg_list_base(s, seg_first);
-  a.miss_list = p.miss_list + base;
-  a.lru_fill = p.lru_fill;
-  a.dedup = p.dedup.slots;
-  a.dedup_log2cap = p.dedup.log2cap;
-  a.st = p.st;
-  a.seg_first = seg_first;
-  a.seg_last = seg_last;
-  a.seg = seg_first;
+int launch_lookup(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg_first, int seg_last) {
+  LookupGroup g{};
   const int64_t n_max = s->node_cap[seg_last];
-  int grid = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(n_max, kLookupBlock), (int64_t)s->n_cu * 2));
-  a.lookup_blocks = grid;
-  a.fill.hop = -1;
-  if (p.fill_pending >= 0) {  // the hop sampled last left its local ids to this kernel
-    a.fill = fill_args(p, p.fill_pending);
-    grid += fill_blocks(s->edge_cap[p.fill_pending], kLookupBlock);
+  const int lookup_blocks = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(n_max, kLookupBlock), (int64_t)s->n_cu * 2));
+  int grid = lookup_blocks;
+  const int pending = pp[0]->fill_pending;  // the hop sampled last left its local ids to this kernel
+  if (pending >= 0) grid += fill_blocks(s->edge_cap[pending], kLookupBlock);
+  for (int k = 0; k < n; ++k) {
+    Pipe &p = *pp[k];
+    LookupArgs &a = g.p[k];
+    a.ids = p.ids;
+    a.n_nodes = s->n_nodes;
+    a.kind = s->cache_kind;
+    a.table_kind = s->table_kind;
+    a.slots = s->id_table.slots;
+    a.log2cap = s->id_table.log2cap;
+    a.slot_of = s->slot_of;
+    a.rank_tab = s->rank_tab;
+    a.lru_keys = s->lru_keys;
+    a.lru_use = s->lru_use;
+    a.lru_sets = s->lru_sets;
+    a.lru_ways = s->lru_ways;
+    a.cache_index = p.cache_index;
+    a.miss_list = p.miss_list + seg_list_base(s, seg_first);
+    a.lru_fill = p.lru_fill;
+    a.dedup = p.dedup.slots;
+    a.dedup_log2cap = p.dedup.log2cap;
+    a.st = p.st;
+    a.seg_first = seg_first;
+    a.seg_last = seg_last;
+    a.seg = seg_first;
+    a.lookup_blocks = lookup_blocks;
+    a.fill.hop = -1;
+    if (pending >= 0) a.fill = fill_args(p, pending);
     p.fill_pending = -1;
   }
-  hipLaunchKernelGGL(lookup_kernel, dim3(grid), dim3(kLookupBlock), 0, st, a);
+  hipLaunchKernelGGL(lookup_kernel, dim3(grid, n), dim3(kLookupBlock), 0, st, g);
   LMI_HIP(hipGetLastError());
   return LMI_OK;
 }
@@ -512,36 +520,46 @@ static int launch_misses(Server *s, Pipe &p, hipStream_t st, int seg, int seg_la
 //      is done.
 // With 1 and 2 the caller's stream does not wait here: the next call on this pipe,
 // or lmi_batch_wait, joins.  The LRU cache joins at once (its insert copies the rows).
-int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last, int lru_lists) {
+int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg, int seg_last, int lru_lists) {
   const bool have_cache = s->cache_kind != LMI_CACHE_NONE;
   int mode = (s->feat_loc == LMI_LOC_HOST && have_cache) ? s->split_miss : 0;
   // The gather kernels carry their own profiling events (prof_kernel_events); a bracket
   // left open by the sampling phase ends here.
   hipEvent_t closing = prof_phase(s, st, &s->prof_open, -1);
   if (mode == 0) {
-    if (have_cache) LMI_TRY(launch_hits(s, p, st, seg, seg_last));
-    LMI_TRY(launch_misses(s, p, st, seg, seg_last));
-    if (lru_lists > 0) LMI_TRY(launch_lru_insert(s, p, st, lru_lists));
+    for (int k = 0; k < n; ++k) {
+      if (have_cache) LMI_TRY(launch_hits(s, *pp[k], st, seg, seg_last));
+      LMI_TRY(launch_misses(s, *pp[k], st, seg, seg_last));
+      if (lru_lists > 0) LMI_TRY(launch_lru_insert(s, *pp[k], st, lru_lists));
+    }
     return LMI_OK;
   }
   hipEvent_t fork = closing;  // when mode 2 forks right here, the closing event doubles as the fork
   if (mode == 1) {
-    LMI_TRY(launch_hits(s, p, st, seg, seg_last));
+    for (int k = 0; k < n; ++k) LMI_TRY(launch_hits(s, *pp[k], st, seg, seg_last));
     fork = nullptr;
   }
-  if (!fork) {
-    fork = p.fork;
+  if (!fork) {  // one fork for the whole group
+    fork = pp[0]->fork;
     LMI_HIP(hipEventRecord(fork, st));
   }
   LMI_HIP(hipStreamWaitEvent(s->side, fork, 0));
-  if (mode == 2) LMI_TRY(launch_hits(s, p, s->side, seg, seg_last));
-  LMI_TRY(launch_misses(s, p, s->side, seg, seg_last));
-  if (lru_lists > 0) LMI_TRY(launch_lru_insert(s, p, s->side, lru_lists));  // reads the rows just gathered
-  LMI_HIP(hipEventRecord(p.join, s->side));
-  p.side_pending = true;
-  // an LRU insertion that comes later on the caller's stream copies the gathered rows: join now
-  if (s->cache_kind == LMI_CACHE_LRU && lru_lists == 0) LMI_TRY(pipe_join(p, st));
+  for (int k = 0; k < n; ++k) {
+    Pipe &p = *pp[k];
+    if (mode == 2) LMI_TRY(launch_hits(s, p, s->side, seg, seg_last));
+    LMI_TRY(launch_misses(s, p, s->side, seg, seg_last));
+    if (lru_lists > 0) LMI_TRY(launch_lru_insert(s, p, s->side, lru_lists));  // reads the rows just gathered
+    LMI_HIP(hipEventRecord(p.join, s->side));
+    p.side_pending = true;
+    // an LRU insertion that comes later on the caller's stream copies the gathered rows: join now
+    if (s->cache_kind == LMI_CACHE_LRU && lru_lists == 0) LMI_TRY(pipe_join(p, st));
+  }
   return LMI_OK;
+}
+
+int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last, int lru_lists) {
+  Pipe *pp[1] = {&p};
+  return launch_gather_group(s, pp, 1, st, seg, seg_last, lru_lists);
 }
 
 // --------------------------------------------------------------- LRU insert

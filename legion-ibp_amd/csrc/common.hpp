@@ -209,13 +209,15 @@ void prof_kernel_events(Server *s, int kind, hipEvent_t *start, hipEvent_t *stop
 
 // sampler.hip
 // stage_seeds: also run the seed-staging kernel now (otherwise hop 0 stages them itself)
-int launch_batch_generate(Server *s, Pipe &p, hipStream_t st, const BatchParams &bp, bool stage_seeds);
+int launch_batch_generate(Server *s, Pipe *const *pp, const BatchParams *bps, int n, hipStream_t st, bool stage_seeds);
 int graph_update_begin(Server *s, Pipe &p, const BatchParams &bp);
 // defer_fill: leave the last step of the hop (local ids of the edge sources) to the next
 // kernel of the batch -- the next hop's first kernel or the lookup -- which carries it in
 // extra blocks; otherwise a kernel of its own finishes the hop.
-int launch_hop(Server *s, Pipe &p, hipStream_t st, int hop, bool stage_seeds, bool defer_fill);
-int launch_fill(Server *s, Pipe &p, hipStream_t st);  // finishes a hop left pending, if any
+// The launchers below take n pipes that are in step (same stage of their batches) and serve
+// them with the same launches, one grid row per pipe.
+int launch_hop(Server *s, Pipe *const *pp, int n, hipStream_t st, int hop, bool stage_seeds, bool defer_fill);
+int launch_fill(Server *s, Pipe *const *pp, int n, hipStream_t st);  // finishes a hop left pending, if any
 struct FillArgs;
 FillArgs fill_args(const Pipe &p, int hop);
 int fill_blocks(int64_t e_max, int block);  // grid share of a fill over at most e_max edges
@@ -229,11 +231,14 @@ int cache_build_lru(Server *s, int64_t n_sets, int32_t ways);
 void cache_free(Server *s);
 // Extra blocks of the lookup finish a hop left pending (launch_hop, defer_fill).  (Finishing
 // it on the side stream instead, ahead of the host-link gather, measured 2 % slower.)
-int launch_lookup(Server *s, Pipe &p, hipStream_t st, int seg_first, int seg_last);
+int launch_lookup(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg_first, int seg_last);
 int launch_hotness(Server *s, Pipe &p, hipStream_t st);
 // lru_lists > 0: the LRU insertion of that many miss lists follows the gather on the stream the
 // misses were gathered on (the side stream when it is in use), and the caller's stream does not wait.
 int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last, int lru_lists);
+// The same for n pipes in step: the HBM gathers one after another, one fork, then the
+// host-link gathers one after another on the side stream.
+int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg, int seg_last, int lru_lists);
 int launch_lru_insert(Server *s, Pipe &p, hipStream_t st, int n_lists);
 int lru_wait_ready(Server *s, hipStream_t st);  // orders `st` behind the last LRU insertion
 int pipe_join(Pipe &p, hipStream_t st);  // make `st` wait for the pipe's side-stream work

@@ -51,13 +51,35 @@ struct HopArgs {
   FillArgs fill;    // the previous hop's last step, carried by hop_count_sample (hop -1: none)
 };
 
+// Several mini-batches (pipes) can share every launch of the sampling phase: grid row y
+// works on pipe y.  The kernels are latency-bound, so a second batch in the same launch
+// costs far less than a second launch.
+constexpr int kMaxGroup = LMI_MAX_PIPES;
+struct HopGroup {
+  HopArgs p[kMaxGroup];
+};
+struct FillGroup {
+  FillArgs p[kMaxGroup];
+};
+struct BeginPipe {
+  HashSlot *slots;
+  DevState *st;
+  ScanChain chain_nodes, chain_edges;
+  BatchParams bp;
+};
+struct BeginGroup {
+  BeginPipe p[kMaxGroup];
+};
+
 // ------------------------------------------------------------ batch start
 // Clears the dedup table (key = -1, value = INT_MAX), resets the pipe state and
 // the scan chains, and stores the per-batch parameters where later kernels read them.
-static __global__ __launch_bounds__(256) void batch_begin_kernel(HashSlot *slots, int64_t n_slots, DevState *st,
-                                                                 int hops, ScanChain chain_nodes,
-                                                                 ScanChain chain_edges, int max_tiles,
-                                                                 BatchParams bp) {
+static __global__ __launch_bounds__(256) void batch_begin_kernel(BeginGroup g, int64_t n_slots, int hops,
+                                                                 int max_tiles) {
+  HashSlot *slots = g.p[blockIdx.y].slots;
+  DevState *st = g.p[blockIdx.y].st;
+  const ScanChain chain_nodes = g.p[blockIdx.y].chain_nodes, chain_edges = g.p[blockIdx.y].chain_edges;
+  const BatchParams &bp = g.p[blockIdx.y].bp;
   const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   // two slots (16 bytes) per store
@@ -108,7 +130,8 @@ static __global__ __launch_bounds__(256) void batch_generate_kernel(int64_t n_no
 // ids[i] = seed, labels, and table[seed] = min(i) so that a repeated seed resolves
 // to its first row.
 template <int ITEMS>
-static __global__ __launch_bounds__(kScanBlock) void hop_count_scan_kernel(HopArgs a) {
+static __global__ __launch_bounds__(kScanBlock) void hop_count_scan_kernel(HopGroup g) {
+  const HopArgs &a = g.p[blockIdx.y];  // one pipe (mini-batch) per grid row
   constexpr int TILE = kScanBlock * ITEMS;
   __shared__ int lds[kScanBlock / kWave + 1];
   __shared__ int s_prefix;
@@ -190,7 +213,8 @@ static __global__ __launch_bounds__(kScanBlock) void hop_count_scan_kernel(HopAr
 // Every sampled edge is inserted into the dedup table with candidate value
 // n_prev + e (e = edge index inside the hop); atomicMin keeps the first edge.
 template <int G>
-static __global__ __launch_bounds__(256) void hop_sample_kernel(HopArgs a) {
+static __global__ __launch_bounds__(256) void hop_sample_kernel(HopGroup g) {
+  const HopArgs &a = g.p[blockIdx.y];  // one pipe (mini-batch) per grid row
   const DevState *st = a.st;
   const int64_t flat = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
   scan_chain_reset(a.chain_edges, a.max_tiles, flat, (int64_t)gridDim.x * blockDim.x);
@@ -240,7 +264,8 @@ static __global__ __launch_bounds__(256) void hop_sample_kernel(HopArgs a) {
 // distinct neighbour probes the HBM table, the other lanes copy its slot.  Same
 // results (the HBM table still sees the minimum edge index per key).
 template <int G>
-static __global__ __launch_bounds__(256) void hop_sample_lds_kernel(HopArgs a) {
+static __global__ __launch_bounds__(256) void hop_sample_lds_kernel(HopGroup g) {
+  const HopArgs &a = g.p[blockIdx.y];  // one pipe (mini-batch) per grid row
   constexpr int TAB = 512;
   __shared__ int32_t lds_key[TAB];
   __shared__ int32_t lds_min[TAB];
@@ -322,7 +347,8 @@ static __global__ __launch_bounds__(256) void hop_sample_lds_kernel(HopArgs a) {
 // node, from the row bounds kept in LDS.  Same outputs as hop_count_scan_kernel
 // followed by hop_sample_kernel, one launch and one row-pointer read less.
 template <int G, int NPB>
-static __global__ __launch_bounds__(256) void hop_count_sample_kernel(HopArgs a) {
+static __global__ __launch_bounds__(256) void hop_count_sample_kernel(HopGroup g) {
+  const HopArgs &a = g.p[blockIdx.y];  // one pipe (mini-batch) per grid row
   static_assert(NPB <= kWave && NPB >= 256 / G, "tile = one wavefront of nodes at most, one pass at least");
   __shared__ int32_t s_id[NPB];
   __shared__ int64_t s_beg[NPB], s_deg[NPB];
@@ -438,7 +464,8 @@ static __global__ __launch_bounds__(256) void hop_count_sample_kernel(HopArgs a)
 // publishes the local id in the table.  Publishing while other tiles still read is safe: a
 // later edge of the same node compares the value with its own, larger, index either way.
 template <int ITEMS>
-static __global__ __launch_bounds__(kScanBlock) void hop_flag_scan_kernel(HopArgs a) {
+static __global__ __launch_bounds__(kScanBlock) void hop_flag_scan_kernel(HopGroup g) {
+  const HopArgs &a = g.p[blockIdx.y];  // one pipe (mini-batch) per grid row
   constexpr int TILE = kScanBlock * ITEMS;
   __shared__ int lds[kScanBlock / kWave + 1];
   __shared__ int s_prefix;
@@ -487,7 +514,8 @@ static __global__ __launch_bounds__(kScanBlock) void hop_flag_scan_kernel(HopArg
 }
 
 // ------------------------------------------------------------- hop, step 3
-static __global__ __launch_bounds__(256) void hop_fill_kernel(FillArgs f) {
+static __global__ __launch_bounds__(256) void hop_fill_kernel(FillGroup g) {
+  const FillArgs &f = g.p[blockIdx.y];
   fill_local_ids(f, (int64_t)blockIdx.x * blockDim.x + threadIdx.x, (int64_t)gridDim.x * blockDim.x);
 }
 
@@ -499,29 +527,45 @@ static int begin_grid(const Pipe &p) {
   return (int)std::min<int64_t>(ceil_div(n_slots / 2, 256), 2048);
 }
 
-int launch_batch_generate(Server *s, Pipe &p, hipStream_t st, const BatchParams &bp, bool stage_seeds) {
-  const int64_t n_slots = int64_t(1) << p.dedup.log2cap;
-  hipLaunchKernelGGL(batch_begin_kernel, dim3(begin_grid(p)), dim3(256), 0, st, p.dedup.slots, n_slots, p.st,
-                     s->cfg.hops, chain_of(p, 0), chain_of(p, 1), p.max_tiles, bp);
+static BeginGroup begin_group(Pipe *const *pp, const BatchParams *bps, int n) {
+  BeginGroup g{};
+  for (int k = 0; k < n; ++k) {
+    g.p[k].slots = pp[k]->dedup.slots;
+    g.p[k].st = pp[k]->st;
+    g.p[k].chain_nodes = chain_of(*pp[k], 0);
+    g.p[k].chain_edges = chain_of(*pp[k], 1);
+    g.p[k].bp = bps[k];
+  }
+  return g;
+}
+
+// First kernel of a batch for each of the n pipes (one launch); stage_seeds also stages the
+// seeds in a kernel of their own (operator-by-operator use, one pipe).
+int launch_batch_generate(Server *s, Pipe *const *pp, const BatchParams *bps, int n, hipStream_t st, bool stage_seeds) {
+  Pipe &p0 = *pp[0];
+  const int64_t n_slots = int64_t(1) << p0.dedup.log2cap;
+  hipLaunchKernelGGL(batch_begin_kernel, dim3(begin_grid(p0), n), dim3(256), 0, st, begin_group(pp, bps, n), n_slots,
+                     s->cfg.hops, p0.max_tiles);
   if (stage_seeds)
-    hipLaunchKernelGGL(batch_generate_kernel, dim3((s->cfg.batch_size + 255) / 256), dim3(256), 0, st, s->n_nodes,
-                       p.ids, p.labels, p.dedup.slots, p.dedup.log2cap, p.st);
+    for (int k = 0; k < n; ++k)
+      hipLaunchKernelGGL(batch_generate_kernel, dim3((s->cfg.batch_size + 255) / 256), dim3(256), 0, st, s->n_nodes,
+                         pp[k]->ids, pp[k]->labels, pp[k]->dedup.slots, pp[k]->dedup.log2cap, pp[k]->st);
   LMI_HIP(hipGetLastError());
-  p.n_seeds = bp.n_seeds;
-  p.hops_done = 0;
+  for (int k = 0; k < n; ++k) {
+    pp[k]->n_seeds = bps[k].n_seeds;
+    pp[k]->hops_done = 0;
+  }
   return LMI_OK;
 }
 
 // Re-points the captured graph's first kernel at this batch's parameters.
 int graph_update_begin(Server *s, Pipe &p, const BatchParams &bp) {
-  HashSlot *slots = p.dedup.slots;
+  Pipe *pp[1] = {&p};
+  BeginGroup g = begin_group(pp, &bp, 1);
   int64_t n_slots = int64_t(1) << p.dedup.log2cap;
-  DevState *st = p.st;
   int hops = s->cfg.hops;
-  ScanChain c0 = chain_of(p, 0), c1 = chain_of(p, 1);
   int max_tiles = p.max_tiles;
-  BatchParams bpc = bp;
-  void *args[8] = {&slots, &n_slots, &st, &hops, &c0, &c1, &max_tiles, &bpc};
+  void *args[4] = {&g, &n_slots, &hops, &max_tiles};
   hipKernelNodeParams kp{};
   kp.func = reinterpret_cast<void *>(batch_begin_kernel);
   kp.gridDim = dim3(begin_grid(p));
@@ -535,50 +579,58 @@ int graph_update_begin(Server *s, Pipe &p, const BatchParams &bp) {
   return LMI_OK;
 }
 
-int launch_hop(Server *s, Pipe &p, hipStream_t st, int hop, bool stage_seeds, bool defer_fill) {
+// One hop for each of the n pipes, all in the same launches (the pipes are in step: same hop,
+// same pending fill).
+int launch_hop(Server *s, Pipe *const *pp, int n, hipStream_t st, int hop, bool stage_seeds, bool defer_fill) {
   const int f = s->cfg.fanout[hop];
   const int64_t n_max = s->node_cap[hop], e_max = s->edge_cap[hop];
-  HopArgs a{};
-  a.indptr = s->indptr;
-  a.indices = s->indices;
-  a.n_nodes = s->n_nodes;
-  a.fanout = f;
-  a.hop = hop;
-  a.st = p.st;
-  a.ids = p.ids;
-  a.labels = p.labels;
-  a.row_ptr = p.blk_indptr[hop];
-  a.agg_src_ids = p.agg_src_ids;
-  a.agg_src_off = p.agg_src_off;
-  a.agg_dst_off = p.agg_dst_off;
-  a.slots = p.dedup.slots;
-  a.log2cap = p.dedup.log2cap;
-  a.eslot = p.eslot[hop & 1];
-  a.chain_nodes = chain_of(p, 0);
-  a.chain_edges = chain_of(p, 1);
-  a.max_tiles = p.max_tiles;
-  a.stage_seeds = (hop == 0 && stage_seeds) ? 1 : 0;
+  Pipe &p0 = *pp[0];
+  HopGroup g{};
+  for (int k = 0; k < n; ++k) {
+    Pipe &p = *pp[k];
+    HopArgs &a = g.p[k];
+    a.indptr = s->indptr;
+    a.indices = s->indices;
+    a.n_nodes = s->n_nodes;
+    a.fanout = f;
+    a.hop = hop;
+    a.st = p.st;
+    a.ids = p.ids;
+    a.labels = p.labels;
+    a.row_ptr = p.blk_indptr[hop];
+    a.agg_src_ids = p.agg_src_ids;
+    a.agg_src_off = p.agg_src_off;
+    a.agg_dst_off = p.agg_dst_off;
+    a.slots = p.dedup.slots;
+    a.log2cap = p.dedup.log2cap;
+    a.eslot = p.eslot[hop & 1];
+    a.chain_nodes = chain_of(p, 0);
+    a.chain_edges = chain_of(p, 1);
+    a.max_tiles = p.max_tiles;
+    a.stage_seeds = (hop == 0 && stage_seeds) ? 1 : 0;
+    a.fill.hop = -1;
+  }
   int G = 4;
   while (G < f) G <<= 1;
   const bool fused = s->fuse_count && !s->lds_dedup;
-  a.fill.hop = -1;
-  if (!fused) LMI_TRY(launch_fill(s, p, st));
+  if (!fused) LMI_TRY(launch_fill(s, pp, n, st));
   if (fused) {
     // counts, scan and sampling in one launch, one tile of nodes per block; a hop left
     // pending gets its local ids filled in by extra blocks behind the tile blocks
     const int npb = hop_tile_nodes(n_max, G, s->fuse_small_max);
-    a.tile_blocks = (int)ceil_div(std::max<int64_t>(n_max, 1), npb);
-    int grid = a.tile_blocks;
-    if (p.fill_pending >= 0) {
-      a.fill = fill_args(p, p.fill_pending);
-      grid += fill_blocks(s->edge_cap[p.fill_pending], 256);
-      p.fill_pending = -1;
+    const int tile_blocks = (int)ceil_div(std::max<int64_t>(n_max, 1), npb);
+    int grid = tile_blocks;
+    if (p0.fill_pending >= 0) grid += fill_blocks(s->edge_cap[p0.fill_pending], 256);
+    for (int k = 0; k < n; ++k) {
+      g.p[k].tile_blocks = tile_blocks;
+      if (pp[k]->fill_pending >= 0) g.p[k].fill = fill_args(*pp[k], pp[k]->fill_pending);
+      pp[k]->fill_pending = -1;
     }
 #define LMI_FUSED(GG)                                                                                   \
   if (npb == 64)                                                                                        \
-    hipLaunchKernelGGL((hop_count_sample_kernel<GG, 64>), dim3(grid), dim3(256), 0, st, a);             \
+    hipLaunchKernelGGL((hop_count_sample_kernel<GG, 64>), dim3(grid, n), dim3(256), 0, st, g);          \
   else                                                                                                  \
-    hipLaunchKernelGGL((hop_count_sample_kernel<GG, (256 / GG)>), dim3(grid), dim3(256), 0, st, a);
+    hipLaunchKernelGGL((hop_count_sample_kernel<GG, (256 / GG)>), dim3(grid, n), dim3(256), 0, st, g);
     switch (G) {
       case 4: LMI_FUSED(4) break;
       case 8: LMI_FUSED(8) break;
@@ -588,47 +640,50 @@ int launch_hop(Server *s, Pipe &p, hipStream_t st, int hop, bool stage_seeds, bo
     }
 #undef LMI_FUSED
   } else {
-  // one tile per block (blocks past the real item count leave at once); few items per
-  // thread while that keeps the tile count near a thousand: the row-pointer reads are
-  // dependent random accesses, so parallelism matters more than per-thread work
-  const int64_t nm = std::max<int64_t>(n_max, 1);
-  if (nm <= 256 * 1024)
-    hipLaunchKernelGGL(hop_count_scan_kernel<1>, dim3((int)ceil_div(nm, kScanBlock)), dim3(kScanBlock), 0, st, a);
-  else if (nm <= 512 * 1024)
-    hipLaunchKernelGGL(hop_count_scan_kernel<2>, dim3((int)ceil_div(nm, kScanBlock * 2)), dim3(kScanBlock), 0, st, a);
-  else if (nm <= 1024 * 1024)
-    hipLaunchKernelGGL(hop_count_scan_kernel<4>, dim3((int)ceil_div(nm, kScanBlock * 4)), dim3(kScanBlock), 0, st, a);
-  else
-    hipLaunchKernelGGL(hop_count_scan_kernel<8>, dim3((int)ceil_div(nm, kScanBlock * 8)), dim3(kScanBlock), 0, st, a);
-  const int grid = (int)std::min<int64_t>(ceil_div(n_max * G, 256), 8192);
-  if (s->lds_dedup) {
-    switch (G) {
-      case 4: hipLaunchKernelGGL(hop_sample_lds_kernel<4>, dim3(grid), dim3(256), 0, st, a); break;
-      case 8: hipLaunchKernelGGL(hop_sample_lds_kernel<8>, dim3(grid), dim3(256), 0, st, a); break;
-      case 16: hipLaunchKernelGGL(hop_sample_lds_kernel<16>, dim3(grid), dim3(256), 0, st, a); break;
-      case 32: hipLaunchKernelGGL(hop_sample_lds_kernel<32>, dim3(grid), dim3(256), 0, st, a); break;
-      default: hipLaunchKernelGGL(hop_sample_lds_kernel<64>, dim3(grid), dim3(256), 0, st, a); break;
+    // one tile per block (blocks past the real item count leave at once); few items per
+    // thread while that keeps the tile count near a thousand: the row-pointer reads are
+    // dependent random accesses, so parallelism matters more than per-thread work
+    const int64_t nm = std::max<int64_t>(n_max, 1);
+    if (nm <= 256 * 1024)
+      hipLaunchKernelGGL(hop_count_scan_kernel<1>, dim3((int)ceil_div(nm, kScanBlock), n), dim3(kScanBlock), 0, st, g);
+    else if (nm <= 512 * 1024)
+      hipLaunchKernelGGL(hop_count_scan_kernel<2>, dim3((int)ceil_div(nm, kScanBlock * 2), n), dim3(kScanBlock), 0, st, g);
+    else if (nm <= 1024 * 1024)
+      hipLaunchKernelGGL(hop_count_scan_kernel<4>, dim3((int)ceil_div(nm, kScanBlock * 4), n), dim3(kScanBlock), 0, st, g);
+    else
+      hipLaunchKernelGGL(hop_count_scan_kernel<8>, dim3((int)ceil_div(nm, kScanBlock * 8), n), dim3(kScanBlock), 0, st, g);
+    const int grid = (int)std::min<int64_t>(ceil_div(n_max * G, 256), 8192);
+    if (s->lds_dedup) {
+      switch (G) {
+        case 4: hipLaunchKernelGGL(hop_sample_lds_kernel<4>, dim3(grid, n), dim3(256), 0, st, g); break;
+        case 8: hipLaunchKernelGGL(hop_sample_lds_kernel<8>, dim3(grid, n), dim3(256), 0, st, g); break;
+        case 16: hipLaunchKernelGGL(hop_sample_lds_kernel<16>, dim3(grid, n), dim3(256), 0, st, g); break;
+        case 32: hipLaunchKernelGGL(hop_sample_lds_kernel<32>, dim3(grid, n), dim3(256), 0, st, g); break;
+        default: hipLaunchKernelGGL(hop_sample_lds_kernel<64>, dim3(grid, n), dim3(256), 0, st, g); break;
+      }
+    } else {
+      switch (G) {
+        case 4: hipLaunchKernelGGL(hop_sample_kernel<4>, dim3(grid, n), dim3(256), 0, st, g); break;
+        case 8: hipLaunchKernelGGL(hop_sample_kernel<8>, dim3(grid, n), dim3(256), 0, st, g); break;
+        case 16: hipLaunchKernelGGL(hop_sample_kernel<16>, dim3(grid, n), dim3(256), 0, st, g); break;
+        case 32: hipLaunchKernelGGL(hop_sample_kernel<32>, dim3(grid, n), dim3(256), 0, st, g); break;
+        default: hipLaunchKernelGGL(hop_sample_kernel<64>, dim3(grid, n), dim3(256), 0, st, g); break;
+      }
     }
-  } else
-  switch (G) {
-    case 4: hipLaunchKernelGGL(hop_sample_kernel<4>, dim3(grid), dim3(256), 0, st, a); break;
-    case 8: hipLaunchKernelGGL(hop_sample_kernel<8>, dim3(grid), dim3(256), 0, st, a); break;
-    case 16: hipLaunchKernelGGL(hop_sample_kernel<16>, dim3(grid), dim3(256), 0, st, a); break;
-    case 32: hipLaunchKernelGGL(hop_sample_kernel<32>, dim3(grid), dim3(256), 0, st, a); break;
-    default: hipLaunchKernelGGL(hop_sample_kernel<64>, dim3(grid), dim3(256), 0, st, a); break;
-  }
   }
   const int64_t em = std::max<int64_t>(e_max, 1);
   if (em <= 1024 * 1024)
-    hipLaunchKernelGGL(hop_flag_scan_kernel<2>, dim3((int)ceil_div(em, kScanBlock * 2)), dim3(kScanBlock), 0, st, a);
+    hipLaunchKernelGGL(hop_flag_scan_kernel<2>, dim3((int)ceil_div(em, kScanBlock * 2), n), dim3(kScanBlock), 0, st, g);
   else if (em <= 2560 * 1024)
-    hipLaunchKernelGGL(hop_flag_scan_kernel<4>, dim3((int)ceil_div(em, kScanBlock * 4)), dim3(kScanBlock), 0, st, a);
+    hipLaunchKernelGGL(hop_flag_scan_kernel<4>, dim3((int)ceil_div(em, kScanBlock * 4), n), dim3(kScanBlock), 0, st, g);
   else
-    hipLaunchKernelGGL(hop_flag_scan_kernel<8>, dim3((int)ceil_div(em, kScanBlock * 8)), dim3(kScanBlock), 0, st, a);
+    hipLaunchKernelGGL(hop_flag_scan_kernel<8>, dim3((int)ceil_div(em, kScanBlock * 8), n), dim3(kScanBlock), 0, st, g);
   LMI_HIP(hipGetLastError());
-  p.fill_pending = hop;
-  if (!defer_fill) LMI_TRY(launch_fill(s, p, st));
-  p.hops_done = hop + 1;
+  for (int k = 0; k < n; ++k) {
+    pp[k]->fill_pending = hop;
+    pp[k]->hops_done = hop + 1;
+  }
+  if (!defer_fill) LMI_TRY(launch_fill(s, pp, n, st));
   return LMI_OK;
 }
 
@@ -646,12 +701,16 @@ int fill_blocks(int64_t e_max, int block) {  // four edges per thread
   return (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(e_max, (int64_t)block * 4), 1024));
 }
 
-int launch_fill(Server *s, Pipe &p, hipStream_t st) {
-  if (p.fill_pending < 0) return LMI_OK;
-  hipLaunchKernelGGL(hop_fill_kernel, dim3(fill_blocks(s->edge_cap[p.fill_pending], 256)), dim3(256), 0, st,
-                     fill_args(p, p.fill_pending));
+int launch_fill(Server *s, Pipe *const *pp, int n, hipStream_t st) {
+  const int hop = pp[0]->fill_pending;
+  if (hop < 0) return LMI_OK;
+  FillGroup g{};
+  for (int k = 0; k < n; ++k) {
+    g.p[k] = fill_args(*pp[k], hop);
+    pp[k]->fill_pending = -1;
+  }
+  hipLaunchKernelGGL(hop_fill_kernel, dim3(fill_blocks(s->edge_cap[hop], 256), n), dim3(256), 0, st, g);
   LMI_HIP(hipGetLastError());
-  p.fill_pending = -1;
   return LMI_OK;
 }
 

@@ -200,6 +200,68 @@ def test_dedup_table_epochs_wrap(lmi, oracle, epochs):
         feats.free()
 
 
+@pytest.mark.parametrize("cache", ["static", "int8", "none"])
+@pytest.mark.parametrize("group,fanout", [(2, [25, 10]), (3, [6, 4, 3]), (4, [64, 2]), (8, [5])])
+def test_groups_of_batches_share_their_launches(lmi, oracle, group, fanout, cache):
+    """lmi_run_group: several mini-batches, each in its own pipe, go through the same kernel
+    launches; every one of them must come out as if it had been run alone."""
+    rng = np.random.default_rng(group * 10 + len(fanout))
+    n_nodes, batch, dim = 5000, 150, 16
+    indptr, indices = random_graph(rng, n_nodes, 15, hubs=5, hub_deg=600)
+    feats = make_features(lmi, rng, n_nodes, dim)
+    train = rng.permutation(n_nodes)[:4000].astype(np.int32)
+    srv = lmi.Server(batch, fanout, dim, pipes=group, seed=9)
+    stream = lmi.stream_create()
+    slot_ref = q = sc = None
+    try:
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        srv.load_idset(lmi.MODE_TRAIN, train)
+        if cache == "static":
+            srv.build_static_cache(1800, lmi.TABLE_RANK)
+            slot_ref = oracle.static_cache_build(indptr, 1800)
+        elif cache == "int8":
+            srv.build_int8_cache(1800, lmi.TABLE_HASH)
+            slot_ref = oracle.static_cache_build(indptr, 1800)
+            q, sc = oracle.quantize_rows(feats.array[np.flatnonzero(slot_ref >= 0)])
+        for rnd in range(3):
+            pipes = list(range(group))
+            if rnd == 1:   # caller seeds of different lengths, one batch short, one with a repeat
+                seeds = [rng.choice(n_nodes, int(rng.integers(1, batch + 1)), replace=False).astype(np.int32)
+                         for _ in pipes]
+                seeds[0][-1] = seeds[0][0]
+                srv.run_group(pipes, [0] * group, seeds=seeds, rng_seeds=[200 + k for k in pipes], stream=stream)
+                want = [(seeds[k], 200 + k) for k in pipes]
+            else:          # slices of the id set, default RNG seeds (server seed + batch counter)
+                counters = [rnd * group + k for k in pipes]
+                srv.run_group(pipes, counters, stream=stream if rnd else None)
+                want = [(train[c * batch:(c + 1) * batch], 9 + c) for c in counters]
+            for k in pipes:
+                g = srv.fetch(pipe=k, stream=stream if rnd else None)
+                o = oracle.sample_batch(indptr, indices, want[k][0], fanout, want[k][1])
+                assert_batch_equal(g, o)
+                if cache == "int8":
+                    ref = oracle.gather_rows_int8(o.ids, slot_ref[o.ids], q, sc, feats.array)
+                    assert g.features.tobytes() == ref.tobytes()
+                else:
+                    assert g.features.tobytes() == feats.array[o.ids].tobytes()
+                if slot_ref is not None:
+                    np.testing.assert_array_equal(g.cache_index, slot_ref[o.ids])
+        # a group may not name a pipe twice, and the LRU cache takes one batch at a time
+        with pytest.raises(lmi.LegionError):
+            srv.run_group([0, 0], [0, 1])
+        if group > 1:
+            srv.build_lru_cache(32, 4)
+            with pytest.raises(lmi.LegionError):
+                srv.run_group([0, 1], [0, 1])
+            srv.run_group([0], [0])
+            g = srv.fetch(pipe=0)
+            assert_batch_equal(g, oracle.sample_batch(indptr, indices, train[:batch], fanout, 9))
+    finally:
+        srv.close()
+        feats.free()
+
+
 def test_duplicate_seeds_and_isolated_nodes(lmi, oracle):
     rng = np.random.default_rng(5)
     indptr, indices = random_graph(rng, 300, 6, zero_frac=0.4)
