@@ -232,8 +232,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="paper100m", choices=sorted(WORKLOADS))
     ap.add_argument("--scale", type=float, default=1.0, help="shrink node/train counts (testing only)")
-    ap.add_argument("--pipes", type=int, default=2, help="output buffer sets in flight")
+    ap.add_argument("--pipes", type=int, default=4, help="output buffer sets in flight")
     ap.add_argument("--streams", type=int, default=1, help="caller streams the pipes are spread over")
+    ap.add_argument("--group", type=int, default=2,
+                    help="mini-batches issued together with lmi_run_group (their sampling kernels share launches)")
     ap.add_argument("--seed", type=int, default=20260101)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget (0 = skip)")
     ap.add_argument("--host-gb", type=float, default=64.0, help="pinned host memory budget for the feature table")
@@ -255,10 +257,18 @@ def main():
         w["train"] = max(w["batch"], int(w["train"] * args.scale))
         if w["cache"][0] in ("static", "lru", "int8"):
             w["cache"] = (w["cache"][0], w["cache"][1] * args.scale)
+    if w["cache"][0] == "lru":
+        args.group = 1                      # the LRU cache takes one batch at a time
+        args.pipes = min(args.pipes, 2)
     srv, info = build_workload(lmi, w, args.seed, args.pipes, args.host_gb,
                                {"hash": 0, "direct": 1, "rank": 2}[args.table], args.policy)
-    for kv in args.tune:
-        k, v = kv.split("=")
+    tunes = dict(kv.split("=") for kv in args.tune)
+    if args.group > 1:
+        # with two batches per launch the sampling phase is short enough that the host link sets the
+        # pace: a few more host-link blocks than the library's default of 32 (measured: 36 -> 6.0 k
+        # batches/s with the HBM gather at 62 % of peak, 40 -> 5.8 k at 65 %, 44 -> 5.65 k at 66 %)
+        tunes.setdefault("miss_blocks", "40")
+    for k, v in tunes.items():
         srv.tune(k, int(v))
     steps_per_epoch = -(-info["n_train"] // w["batch"])
     streams = [lmi.stream_create() for _ in range(max(1, args.streams))]
@@ -270,15 +280,29 @@ def main():
         srv.build_lru_cache(int(ci.n_sets), int(ci.ways))   # start the replay from an empty cache again
         log("recorded %d seed batches with temporal locality (%.1f s)" % (len(plan), time.time() - t0))
 
+    group = max(1, args.group)
+    if group > 1 and (args.pipes % group or info["cache_kind"] == "lru"):
+        print("bench.py: --group needs a pipe count that is a multiple of it, and no LRU cache", file=sys.stderr)
+        sys.exit(2)
+
     def step(i):
         # consecutive batches alternate output buffer sets (pipes), so the host-link part of batch i
         # (on the server's side stream) overlaps the sampling of batch i+1; a pipe always uses the
-        # same caller stream
+        # same caller stream.  With --group g, batches i .. i+g-1 are issued together (step is then
+        # called with i a multiple of g) and consecutive groups alternate sets of g pipes.
         p = i % args.pipes
-        srv.run_once(plan[i] if plan else None, batch_counter=i % steps_per_epoch, rng_seed=args.seed + i, pipe=p,
-                     stream=streams[p % len(streams)])
+        if group == 1:
+            srv.run_once(plan[i] if plan else None, batch_counter=i % steps_per_epoch, rng_seed=args.seed + i, pipe=p,
+                         stream=streams[p % len(streams)])
+        else:
+            ks = range(i, i + group)
+            srv.run_group([k % args.pipes for k in ks], [k % steps_per_epoch for k in ks],
+                          seeds=[plan[k] for k in ks] if plan else None, rng_seeds=[args.seed + k for k in ks],
+                          stream=streams[(p // group) % len(streams)])
 
-    for i in range(args.warmup):
+    args.warmup = -(-args.warmup // group) * group   # whole groups
+    args.steps = -(-args.steps // group) * group
+    for i in range(0, args.warmup, group):
         step(i)
     lmi.check(lmi.lib().lmi_device_sync())
     srv.profile_read(reset=True)
@@ -288,7 +312,7 @@ def main():
     srv.tune("profile_every", args.profile_every)
     srv.profile_enable(2)
     t0 = time.perf_counter()
-    for i in range(args.warmup, args.warmup + args.steps):
+    for i in range(args.warmup, args.warmup + args.steps, group):
         step(i)
     lmi.check(lmi.lib().lmi_device_sync())
     t1 = time.perf_counter()
@@ -298,7 +322,7 @@ def main():
     # untimed extra leg with every phase of every batch bracketed (level 1), for the per-phase breakdown only
     srv.tune("profile_every", 1)
     srv.profile_enable(1)
-    for i in range(args.warmup + args.steps, args.warmup + args.steps + min(args.steps, 20)):
+    for i in range(args.warmup + args.steps, args.warmup + args.steps + -(-min(args.steps, 20) // group) * group, group):
         step(i)
     srv.profile_enable(0)
     phases = srv.profile_read(reset=True)
@@ -338,7 +362,8 @@ def main():
         "config": {"workload": args.workload, "nodes": info["n_nodes"], "edges": info["n_edges"],
                    "feat_dim": w["dim"], "batch": w["batch"], "fanout": w["fanout"],
                    "cache": "%s, %d rows, %s id->slot table" % (info["cache_kind"], info["cache_rows"], args.table),
-                   "pipes": args.pipes, "streams": args.streams, "cache_policy": args.policy,
+                   "pipes": args.pipes, "streams": args.streams, "group": group, "tune": tunes,
+                   "cache_policy": args.policy,
                    "graph": "Zipf-Mandelbrot degrees alpha=%s, degree-proportional neighbours" % w["alpha"],
                    "seeds": ("%d %% of a batch from the frontiers of the previous %d batches, the rest uniform from the "
                              "train set" % (w["locality"][0] * 100, w["locality"][1])) if w.get("locality")

@@ -154,6 +154,7 @@ static int pipe_alloc(Server *s, Pipe &p) {
 // 16 KB chunk at a time, non-temporal both ways: the measured HBM copy ceiling (the best of
 // the layouts tried: grid-wide strides between a lane's four vectors lose a quarter).
 typedef uint32_t cp_u32x4 __attribute__((ext_vector_type(4)));
+template <bool HOSTLINK>  // only names the instantiation that reads pinned host memory, so that profiles tell the two apart
 static __global__ __launch_bounds__(256) void copy_kernel(const cp_u32x4 *__restrict__ src, cp_u32x4 *__restrict__ dst,
                                                           size_t n) {
   const size_t stride = (size_t)gridDim.x * blockDim.x * 4;
@@ -222,6 +223,7 @@ int lmi_server_create(const lmi_config *cfg, lmi_server **out) {
   if (rc == LMI_OK && hipMalloc(&s->d_scalar, 64) != hipSuccess) rc = LMI_ERR_HIP;
   if (rc == LMI_OK && hipStreamCreateWithFlags(&s->side, hipStreamNonBlocking) != hipSuccess) rc = LMI_ERR_HIP;
   if (rc == LMI_OK && hipEventCreateWithFlags(&s->lru_ready, hipEventDisableTiming) != hipSuccess) rc = LMI_ERR_HIP;
+  if (rc == LMI_OK && hipEventCreateWithFlags(&s->side_idle, hipEventDisableTiming) != hipSuccess) rc = LMI_ERR_HIP;
   if (rc == LMI_OK && (hipMalloc(&s->d_prof_rows, 16) != hipSuccess || hipMemset(s->d_prof_rows, 0, 16) != hipSuccess))
     rc = LMI_ERR_HIP;
   if (rc != LMI_OK) {
@@ -254,6 +256,7 @@ int lmi_server_destroy(lmi_server *h) {
   if (s->hot) (void)hipFree(s->hot);
   if (s->side) (void)hipStreamDestroy(s->side);
   if (s->lru_ready) (void)hipEventDestroy(s->lru_ready);
+  if (s->side_idle) (void)hipEventDestroy(s->side_idle);
   delete s;
   return LMI_OK;
 }
@@ -798,6 +801,7 @@ int lmi_tune(lmi_server *h, const char *key, int64_t value) {
   else if (!strcmp(key, "gather_nontemporal")) s->gather_nt = (int)value;
   else if (!strcmp(key, "lds_dedup")) s->lds_dedup = (int)value;
   else if (!strcmp(key, "fuse_count")) s->fuse_count = (int)value;
+  else if (!strcmp(key, "protect_hits")) s->protect_hits = (int)value;
   else if (!strcmp(key, "table_epochs")) {
     s->table_epochs = std::max<int64_t>(0, value);
     for (auto &p : s->pipes) p.table_dirty = true;
@@ -820,10 +824,10 @@ int lmi_bench_host_read(const void *host_ptr, size_t bytes, int repeats, double 
   LMI_HIP(hipEventCreate(&e0));
   LMI_HIP(hipEventCreate(&e1));
   const size_t n = bytes / 16;
-  hipLaunchKernelGGL(copy_kernel, dim3(1024), dim3(256), 0, 0, (const cp_u32x4 *)host_ptr, (cp_u32x4 *)b, n);
+  hipLaunchKernelGGL(copy_kernel<true>, dim3(1024), dim3(256), 0, 0, (const cp_u32x4 *)host_ptr, (cp_u32x4 *)b, n);
   LMI_HIP(hipEventRecord(e0, 0));
   for (int r = 0; r < repeats; ++r)
-    hipLaunchKernelGGL(copy_kernel, dim3(1024), dim3(256), 0, 0, (const cp_u32x4 *)host_ptr, (cp_u32x4 *)b, n);
+    hipLaunchKernelGGL(copy_kernel<true>, dim3(1024), dim3(256), 0, 0, (const cp_u32x4 *)host_ptr, (cp_u32x4 *)b, n);
   LMI_HIP(hipEventRecord(e1, 0));
   LMI_HIP(hipEventSynchronize(e1));
   float ms = 0;
@@ -844,10 +848,10 @@ int lmi_bench_copy(size_t bytes, int repeats, double *ms_per_copy) {
   LMI_HIP(hipEventCreate(&e0));
   LMI_HIP(hipEventCreate(&e1));
   const size_t n = bytes / 16;
-  hipLaunchKernelGGL(copy_kernel, dim3(16384), dim3(256), 0, 0, (const cp_u32x4 *)a, (cp_u32x4 *)b, n);
+  hipLaunchKernelGGL(copy_kernel<false>, dim3(16384), dim3(256), 0, 0, (const cp_u32x4 *)a, (cp_u32x4 *)b, n);
   LMI_HIP(hipEventRecord(e0, 0));
   for (int r = 0; r < repeats; ++r)
-    hipLaunchKernelGGL(copy_kernel, dim3(16384), dim3(256), 0, 0, (const cp_u32x4 *)a, (cp_u32x4 *)b, n);
+    hipLaunchKernelGGL(copy_kernel<false>, dim3(16384), dim3(256), 0, 0, (const cp_u32x4 *)a, (cp_u32x4 *)b, n);
   LMI_HIP(hipEventRecord(e1, 0));
   LMI_HIP(hipEventSynchronize(e1));
   float ms = 0;

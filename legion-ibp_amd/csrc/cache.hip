@@ -317,22 +317,24 @@ __device__ __forceinline__ int32_t static_find(int table_kind, const HashSlot *s
 constexpr int kLookupBlock = 1024;
 struct LookupGroup {  // one pipe per grid row, as in the sampling kernels
   LookupArgs p[LMI_MAX_PIPES];
+  int n;
 };
 
 static __global__ __launch_bounds__(kLookupBlock) void lookup_kernel(LookupGroup g) {
-  const LookupArgs &a = g.p[blockIdx.y];
+  LMI_GRID_ROW(g.n);
+  const LookupArgs &a = g.p[row];
   __shared__ int wave_cnt[kLookupBlock / kWave];
   __shared__ int block_base;
-  if ((int)blockIdx.x >= a.lookup_blocks) {
-    fill_local_ids(a.fill, (int64_t)(blockIdx.x - a.lookup_blocks) * blockDim.x + threadIdx.x,
-                   (int64_t)(gridDim.x - a.lookup_blocks) * blockDim.x);
+  if (bx >= a.lookup_blocks) {
+    fill_local_ids(a.fill, (int64_t)(bx - a.lookup_blocks) * blockDim.x + threadIdx.x,
+                   (int64_t)(gx - a.lookup_blocks) * blockDim.x);
     return;
   }
   const int first = (a.seg_first == 0) ? 0 : a.st->node_counter[9 + a.seg_first - 1];
   const int last = a.st->node_counter[9 + a.seg_last];
   const int lane = threadIdx.x & (kWave - 1), wid = threadIdx.x / kWave;
   const int stride = a.lookup_blocks * blockDim.x;
-  for (int b = first + blockIdx.x * blockDim.x; b < last; b += stride) {
+  for (int b = first + bx * blockDim.x; b < last; b += stride) {
     const int i = b + threadIdx.x;
     bool miss = false;
     int32_t id = -1;
@@ -379,6 +381,7 @@ static inline int64_t seg_list_base(const Server *s, int seg) { return seg == 0 
 
 int launch_lookup(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg_first, int seg_last) {
   LookupGroup g{};
+  g.n = n;
   const int64_t n_max = s->node_cap[seg_last];
   const int lookup_blocks = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(n_max, kLookupBlock), (int64_t)s->n_cu * 2));
   int grid = lookup_blocks;
@@ -413,7 +416,7 @@ int launch_lookup(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg_fir
     if (pending >= 0) a.fill = fill_args(p, pending);
     p.fill_pending = -1;
   }
-  hipLaunchKernelGGL(lookup_kernel, dim3(grid, n), dim3(kLookupBlock), 0, st, g);
+  hipLaunchKernelGGL(lookup_kernel, dim3(grid * n), dim3(kLookupBlock), 0, st, g);
   LMI_HIP(hipGetLastError());
   return LMI_OK;
 }
@@ -536,6 +539,16 @@ int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int s
   }
   hipEvent_t fork = closing;  // when mode 2 forks right here, the closing event doubles as the fork
   if (mode == 1) {
+    // Host-link reads in flight halve the HBM gather's bandwidth: optionally hold the hits back
+    // until the side stream has drained the host-link gathers issued before (other pipes').
+    if (s->protect_hits && s->side_busy) {
+      if (hipEventQuery(s->side_idle) != hipSuccess) {
+        (void)hipGetLastError();
+        LMI_HIP(hipStreamWaitEvent(st, s->side_idle, 0));
+      } else {
+        s->side_busy = false;
+      }
+    }
     for (int k = 0; k < n; ++k) LMI_TRY(launch_hits(s, *pp[k], st, seg, seg_last));
     fork = nullptr;
   }
@@ -553,6 +566,10 @@ int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int s
     p.side_pending = true;
     // an LRU insertion that comes later on the caller's stream copies the gathered rows: join now
     if (s->cache_kind == LMI_CACHE_LRU && lru_lists == 0) LMI_TRY(pipe_join(p, st));
+  }
+  if (s->protect_hits) {
+    LMI_HIP(hipEventRecord(s->side_idle, s->side));
+    s->side_busy = true;
   }
   return LMI_OK;
 }

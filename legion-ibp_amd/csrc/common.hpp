@@ -158,6 +158,9 @@ struct Server {
   int32_t lru_ways = 0;
   int32_t lru_tick = 0;
   int32_t *lru_keys = nullptr, *lru_use = nullptr, *lru_claim[2] = {nullptr, nullptr};
+  hipEvent_t side_idle = nullptr;  // recorded behind the last host-link gather issued on the side stream
+  bool side_busy = false;
+  int protect_hits = 0;            // 1: HBM gathers wait until earlier host-link gathers have drained
   hipEvent_t lru_ready = nullptr;  // recorded behind every LRU insertion: the next lookup waits for it
   bool lru_pending = false;        // an insertion may still be running
   // pipes

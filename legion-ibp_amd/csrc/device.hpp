@@ -51,6 +51,10 @@ __device__ __forceinline__ uint32_t hash_id(int32_t key, int log2cap) {
 // stale free read is resolved by the CAS.  Values only ever decrease, so a stale value
 // is never too low: when the value read is already <= cand the atomic can be skipped,
 // which removes almost all same-address atomics on frequently sampled hub nodes.
+// The slot index comes back with kKnownRepeat set when the insert already saw a lower
+// value: such a candidate is certainly not the key's first occurrence, and whoever asks
+// later need not read the slot to learn that.  (Without the bit it may or may not be.)
+constexpr uint32_t kKnownRepeat = 0x80000000u;
 __device__ __forceinline__ uint32_t table_insert_min(HashSlot *slots, int log2cap, int32_t key, int32_t cand,
                                                      int32_t tag = 0, int32_t tag_mask = kUntaggedMask) {
   const uint32_t mask = (1u << log2cap) - 1u;
@@ -66,8 +70,11 @@ __device__ __forceinline__ uint32_t table_insert_min(HashSlot *slots, int log2ca
       continue;  // somebody else took it: look at what it holds now
     }
     if (k == stored) {
-      if (v > cand) atomicMin(&slots[h].val, cand);
-      return h;
+      if (v > cand) {
+        atomicMin(&slots[h].val, cand);
+        return h;
+      }
+      return h | kKnownRepeat;  // a lower candidate is already there: this one cannot be the minimum
     }
     h = (h + 1) & mask;
   }
@@ -93,7 +100,7 @@ __device__ __forceinline__ int32_t table_find(const HashSlot *slots, int log2cap
 struct FillArgs {
   const DevState *st;
   const HashSlot *slots;
-  const int32_t *eslot;  // table slot per edge of hop `hop`
+  const int32_t *eslot;  // table slot per edge of hop `hop` (| kKnownRepeat)
   int32_t *agg_src_off;
   int hop;               // -1: nothing to fill
 };
@@ -106,7 +113,7 @@ __device__ __forceinline__ void fill_local_ids(const FillArgs &f, int64_t tid, i
   for (int64_t e = tid; e < n; e += 4 * n_threads) {
     int32_t slot[4], val[4];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) slot[u] = (e + u * n_threads < n) ? f.eslot[e + u * n_threads] : 0;
+    for (int u = 0; u < 4; ++u) slot[u] = (e + u * n_threads < n) ? (f.eslot[e + u * n_threads] & (int32_t)~kKnownRepeat) : 0;
 #pragma unroll
     for (int u = 0; u < 4; ++u) val[u] = (e + u * n_threads < n) ? f.slots[slot[u]].val : 0;
 #pragma unroll
@@ -114,6 +121,15 @@ __device__ __forceinline__ void fill_local_ids(const FillArgs &f, int64_t tid, i
       if (e + u * n_threads < n) f.agg_src_off[eoff + e + u * n_threads] = val[u];
   }
 }
+
+// A launch that serves n pipes interleaves them over blockIdx.x: block b works on pipe b % n
+// as that pipe's block b / n of gridDim.x / n.  Every pipe's blocks are then dispatched in
+// step and in ascending order, which the look-back scans rely on.
+#define LMI_GRID_ROW(n_rows)                                     \
+  const int row = (int)(blockIdx.x % (unsigned)(n_rows));        \
+  const int bx = (int)(blockIdx.x / (unsigned)(n_rows));         \
+  const int gx = (int)(gridDim.x / (unsigned)(n_rows));          \
+  (void)gx
 
 // ------------------------------------------------------------------- scans
 __device__ __forceinline__ int wave_inclusive_scan(int v) {

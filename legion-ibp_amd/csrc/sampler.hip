@@ -43,7 +43,7 @@ struct HopArgs {
   int32_t *agg_src_ids, *agg_src_off, *agg_dst_off;
   HashSlot *slots;
   int log2cap;
-  int32_t *eslot;   // table slot per edge of this hop
+  int32_t *eslot;   // table slot per edge of this hop (| kKnownRepeat)
   ScanChain chain_nodes, chain_edges;
   int max_tiles;
   int stage_seeds;  // hop 0 only: the seeds have not been staged by batch_generate_kernel yet
@@ -57,9 +57,11 @@ struct HopArgs {
 constexpr int kMaxGroup = LMI_MAX_PIPES;
 struct HopGroup {
   HopArgs p[kMaxGroup];
+  int n;
 };
 struct FillGroup {
   FillArgs p[kMaxGroup];
+  int n;
 };
 struct BeginPipe {
   HashSlot *slots;
@@ -69,6 +71,7 @@ struct BeginPipe {
 };
 struct BeginGroup {
   BeginPipe p[kMaxGroup];
+  int n;
 };
 
 // ------------------------------------------------------------ batch start
@@ -76,12 +79,13 @@ struct BeginGroup {
 // the scan chains, and stores the per-batch parameters where later kernels read them.
 static __global__ __launch_bounds__(256) void batch_begin_kernel(BeginGroup g, int64_t n_slots, int hops,
                                                                  int max_tiles) {
-  HashSlot *slots = g.p[blockIdx.y].slots;
-  DevState *st = g.p[blockIdx.y].st;
-  const ScanChain chain_nodes = g.p[blockIdx.y].chain_nodes, chain_edges = g.p[blockIdx.y].chain_edges;
-  const BatchParams &bp = g.p[blockIdx.y].bp;
-  const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  LMI_GRID_ROW(g.n);
+  HashSlot *slots = g.p[row].slots;
+  DevState *st = g.p[row].st;
+  const ScanChain chain_nodes = g.p[row].chain_nodes, chain_edges = g.p[row].chain_edges;
+  const BatchParams &bp = g.p[row].bp;
+  const int64_t tid = (int64_t)bx * blockDim.x + threadIdx.x;
+  const int64_t stride = (int64_t)gx * blockDim.x;
   // two slots (16 bytes) per store
   if (bp.clear_table) {
     const int4 fill = make_int4(kEmptyKey, kIntMax, kEmptyKey, kIntMax);
@@ -131,7 +135,8 @@ static __global__ __launch_bounds__(256) void batch_generate_kernel(int64_t n_no
 // to its first row.
 template <int ITEMS>
 static __global__ __launch_bounds__(kScanBlock) void hop_count_scan_kernel(HopGroup g) {
-  const HopArgs &a = g.p[blockIdx.y];  // one pipe (mini-batch) per grid row
+  LMI_GRID_ROW(g.n);
+  const HopArgs &a = g.p[row];  // one pipe (mini-batch) per grid row
   constexpr int TILE = kScanBlock * ITEMS;
   __shared__ int lds[kScanBlock / kWave + 1];
   __shared__ int s_prefix;
@@ -139,13 +144,13 @@ static __global__ __launch_bounds__(kScanBlock) void hop_count_scan_kernel(HopGr
   const int n = st->node_counter[9 + a.hop];
   const int n_tiles = (n + TILE - 1) / TILE;
   if (n_tiles == 0) {
-    if (blockIdx.x == 0 && threadIdx.x == 0) {
+    if (bx == 0 && threadIdx.x == 0) {
       a.row_ptr[0] = 0;
       scan_epilogue(SCAN_EPI_HOP_EDGES, st, a.hop, 0);
     }
     return;
   }
-  const int tile = blockIdx.x;
+  const int tile = bx;
   if (tile < n_tiles) {
     const int base = tile * TILE + threadIdx.x * ITEMS;
     int32_t id[ITEMS];
@@ -214,10 +219,11 @@ static __global__ __launch_bounds__(kScanBlock) void hop_count_scan_kernel(HopGr
 // n_prev + e (e = edge index inside the hop); atomicMin keeps the first edge.
 template <int G>
 static __global__ __launch_bounds__(256) void hop_sample_kernel(HopGroup g) {
-  const HopArgs &a = g.p[blockIdx.y];  // one pipe (mini-batch) per grid row
+  LMI_GRID_ROW(g.n);
+  const HopArgs &a = g.p[row];  // one pipe (mini-batch) per grid row
   const DevState *st = a.st;
-  const int64_t flat = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  scan_chain_reset(a.chain_edges, a.max_tiles, flat, (int64_t)gridDim.x * blockDim.x);
+  const int64_t flat = (int64_t)bx * blockDim.x + threadIdx.x;
+  scan_chain_reset(a.chain_edges, a.max_tiles, flat, (int64_t)gx * blockDim.x);
   const uint64_t seed = (uint64_t)st->rng_lo | ((uint64_t)st->rng_hi << 32);
   const int32_t tag = st->table_tag, tag_mask = st->table_mask;
   const int n_prev = st->node_counter[9 + a.hop];
@@ -225,7 +231,7 @@ static __global__ __launch_bounds__(256) void hop_sample_kernel(HopGroup g) {
   const int fanout = a.fanout;
   const int lane = threadIdx.x & (G - 1);
   const int group = (int)(flat / G);
-  const int n_groups = gridDim.x * blockDim.x / G;
+  const int n_groups = gx * blockDim.x / G;
   for (int i = group; i < n_prev; i += n_groups) {
     const int32_t v = a.ids[i];
     if (v < 0 || v >= a.n_nodes) continue;
@@ -265,25 +271,26 @@ static __global__ __launch_bounds__(256) void hop_sample_kernel(HopGroup g) {
 // results (the HBM table still sees the minimum edge index per key).
 template <int G>
 static __global__ __launch_bounds__(256) void hop_sample_lds_kernel(HopGroup g) {
-  const HopArgs &a = g.p[blockIdx.y];  // one pipe (mini-batch) per grid row
+  LMI_GRID_ROW(g.n);
+  const HopArgs &a = g.p[row];  // one pipe (mini-batch) per grid row
   constexpr int TAB = 512;
   __shared__ int32_t lds_key[TAB];
   __shared__ int32_t lds_min[TAB];
   __shared__ int32_t lds_slot[TAB];
   const DevState *st = a.st;
-  const int64_t flat = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  scan_chain_reset(a.chain_edges, a.max_tiles, flat, (int64_t)gridDim.x * blockDim.x);
+  const int64_t flat = (int64_t)bx * blockDim.x + threadIdx.x;
+  scan_chain_reset(a.chain_edges, a.max_tiles, flat, (int64_t)gx * blockDim.x);
   const uint64_t seed = (uint64_t)st->rng_lo | ((uint64_t)st->rng_hi << 32);
   const int n_prev = st->node_counter[9 + a.hop];
   const int eoff = st->edge_counter[12 + a.hop + 1];
   const int fanout = a.fanout;
   const int lane = threadIdx.x & (G - 1);
   const int group = (int)(flat / G);
-  const int n_groups = gridDim.x * blockDim.x / G;
+  const int n_groups = gx * blockDim.x / G;
   const int groups_per_block = 256 / G;
   // uniform trip count per block: the block's first group decides
-  for (int i0 = blockIdx.x * groups_per_block; i0 < n_prev; i0 += n_groups) {
-    const int i = i0 + (group - blockIdx.x * groups_per_block);
+  for (int i0 = bx * groups_per_block; i0 < n_prev; i0 += n_groups) {
+    const int i = i0 + (group - bx * groups_per_block);
     for (int t = threadIdx.x; t < TAB; t += 256) {
       lds_key[t] = kEmptyKey;
       lds_min[t] = kIntMax;
@@ -335,7 +342,8 @@ static __global__ __launch_bounds__(256) void hop_sample_lds_kernel(HopGroup g) 
     if (active && lds_min[h] == e)
       lds_slot[h] = (int)table_insert_min(a.slots, a.log2cap, nbr, n_prev + e, st->table_tag, st->table_mask);
     __syncthreads();
-    if (active) a.eslot[e] = lds_slot[h];
+    // an edge that lost inside the block is a repeat whatever the table said to the winner
+    if (active) a.eslot[e] = (lds_min[h] == e) ? lds_slot[h] : (lds_slot[h] | (int32_t)kKnownRepeat);
     __syncthreads();
   }
 }
@@ -348,30 +356,31 @@ static __global__ __launch_bounds__(256) void hop_sample_lds_kernel(HopGroup g) 
 // followed by hop_sample_kernel, one launch and one row-pointer read less.
 template <int G, int NPB>
 static __global__ __launch_bounds__(256) void hop_count_sample_kernel(HopGroup g) {
-  const HopArgs &a = g.p[blockIdx.y];  // one pipe (mini-batch) per grid row
+  LMI_GRID_ROW(g.n);
+  const HopArgs &a = g.p[row];  // one pipe (mini-batch) per grid row
   static_assert(NPB <= kWave && NPB >= 256 / G, "tile = one wavefront of nodes at most, one pass at least");
   __shared__ int32_t s_id[NPB];
   __shared__ int64_t s_beg[NPB], s_deg[NPB];
   __shared__ int s_row[NPB];
   __shared__ int s_prefix;
   DevState *st = a.st;
-  const int64_t flat = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  scan_chain_reset(a.chain_edges, a.max_tiles, flat, (int64_t)gridDim.x * blockDim.x);
-  if ((int)blockIdx.x >= a.tile_blocks) {  // extra blocks: the previous hop's local ids
-    fill_local_ids(a.fill, (int64_t)(blockIdx.x - a.tile_blocks) * blockDim.x + threadIdx.x,
-                   (int64_t)(gridDim.x - a.tile_blocks) * blockDim.x);
+  const int64_t flat = (int64_t)bx * blockDim.x + threadIdx.x;
+  scan_chain_reset(a.chain_edges, a.max_tiles, flat, (int64_t)gx * blockDim.x);
+  if (bx >= a.tile_blocks) {  // extra blocks: the previous hop's local ids
+    fill_local_ids(a.fill, (int64_t)(bx - a.tile_blocks) * blockDim.x + threadIdx.x,
+                   (int64_t)(gx - a.tile_blocks) * blockDim.x);
     return;
   }
   const int n_prev = st->node_counter[9 + a.hop];
   const int n_tiles = (n_prev + NPB - 1) / NPB;
   if (n_tiles == 0) {
-    if (blockIdx.x == 0 && threadIdx.x == 0) {
+    if (bx == 0 && threadIdx.x == 0) {
       a.row_ptr[0] = 0;
       scan_epilogue(SCAN_EPI_HOP_EDGES, st, a.hop, 0);
     }
     return;
   }
-  const int tile = blockIdx.x;
+  const int tile = bx;
   if (tile >= n_tiles) return;
   // ---- counts, tile scan (wavefront 0)
   const int t = threadIdx.x;
@@ -465,22 +474,23 @@ static __global__ __launch_bounds__(256) void hop_count_sample_kernel(HopGroup g
 // later edge of the same node compares the value with its own, larger, index either way.
 template <int ITEMS>
 static __global__ __launch_bounds__(kScanBlock) void hop_flag_scan_kernel(HopGroup g) {
-  const HopArgs &a = g.p[blockIdx.y];  // one pipe (mini-batch) per grid row
+  LMI_GRID_ROW(g.n);
+  const HopArgs &a = g.p[row];  // one pipe (mini-batch) per grid row
   constexpr int TILE = kScanBlock * ITEMS;
   __shared__ int lds[kScanBlock / kWave + 1];
   __shared__ int s_prefix;
   DevState *st = a.st;
-  const int64_t flat = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  scan_chain_reset(a.chain_nodes, a.max_tiles, flat, (int64_t)gridDim.x * blockDim.x);  // for the next hop
+  const int64_t flat = (int64_t)bx * blockDim.x + threadIdx.x;
+  scan_chain_reset(a.chain_nodes, a.max_tiles, flat, (int64_t)gx * blockDim.x);  // for the next hop
   const int n_prev = st->node_counter[9 + a.hop];
   const int n = st->edge_counter[9 + a.hop + 1];
   const int eoff = st->edge_counter[12 + a.hop + 1];
   const int n_tiles = (n + TILE - 1) / TILE;
   if (n_tiles == 0) {
-    if (blockIdx.x == 0 && threadIdx.x == 0) scan_epilogue(SCAN_EPI_HOP_NODES, st, a.hop, 0);
+    if (bx == 0 && threadIdx.x == 0) scan_epilogue(SCAN_EPI_HOP_NODES, st, a.hop, 0);
     return;
   }
-  const int tile = blockIdx.x;
+  const int tile = bx;
   if (tile < n_tiles) {
     const int base = tile * TILE + threadIdx.x * ITEMS;
     int v[ITEMS], slot[ITEMS], sum = 0;
@@ -490,8 +500,9 @@ static __global__ __launch_bounds__(kScanBlock) void hop_flag_scan_kernel(HopGro
       int flag = 0;
       slot[j] = 0;
       if (e < n) {
-        slot[j] = a.eslot[e];
-        flag = (a.slots[slot[j]].val == n_prev + e) ? 1 : 0;
+        const int32_t es = a.eslot[e];  // sign bit = kKnownRepeat: no need to look
+        slot[j] = es & (int32_t)~kKnownRepeat;
+        if (es >= 0) flag = (a.slots[slot[j]].val == n_prev + e) ? 1 : 0;
       }
       v[j] = flag;
       sum += flag;
@@ -515,8 +526,9 @@ static __global__ __launch_bounds__(kScanBlock) void hop_flag_scan_kernel(HopGro
 
 // ------------------------------------------------------------- hop, step 3
 static __global__ __launch_bounds__(256) void hop_fill_kernel(FillGroup g) {
-  const FillArgs &f = g.p[blockIdx.y];
-  fill_local_ids(f, (int64_t)blockIdx.x * blockDim.x + threadIdx.x, (int64_t)gridDim.x * blockDim.x);
+  LMI_GRID_ROW(g.n);
+  const FillArgs &f = g.p[row];
+  fill_local_ids(f, (int64_t)bx * blockDim.x + threadIdx.x, (int64_t)gx * blockDim.x);
 }
 
 // ---------------------------------------------------------------- launchers
@@ -529,6 +541,7 @@ static int begin_grid(const Pipe &p) {
 
 static BeginGroup begin_group(Pipe *const *pp, const BatchParams *bps, int n) {
   BeginGroup g{};
+  g.n = n;
   for (int k = 0; k < n; ++k) {
     g.p[k].slots = pp[k]->dedup.slots;
     g.p[k].st = pp[k]->st;
@@ -544,7 +557,7 @@ static BeginGroup begin_group(Pipe *const *pp, const BatchParams *bps, int n) {
 int launch_batch_generate(Server *s, Pipe *const *pp, const BatchParams *bps, int n, hipStream_t st, bool stage_seeds) {
   Pipe &p0 = *pp[0];
   const int64_t n_slots = int64_t(1) << p0.dedup.log2cap;
-  hipLaunchKernelGGL(batch_begin_kernel, dim3(begin_grid(p0), n), dim3(256), 0, st, begin_group(pp, bps, n), n_slots,
+  hipLaunchKernelGGL(batch_begin_kernel, dim3((begin_grid(p0)) * n), dim3(256), 0, st, begin_group(pp, bps, n), n_slots,
                      s->cfg.hops, p0.max_tiles);
   if (stage_seeds)
     for (int k = 0; k < n; ++k)
@@ -586,6 +599,7 @@ int launch_hop(Server *s, Pipe *const *pp, int n, hipStream_t st, int hop, bool 
   const int64_t n_max = s->node_cap[hop], e_max = s->edge_cap[hop];
   Pipe &p0 = *pp[0];
   HopGroup g{};
+  g.n = n;
   for (int k = 0; k < n; ++k) {
     Pipe &p = *pp[k];
     HopArgs &a = g.p[k];
@@ -628,9 +642,9 @@ int launch_hop(Server *s, Pipe *const *pp, int n, hipStream_t st, int hop, bool 
     }
 #define LMI_FUSED(GG)                                                                                   \
   if (npb == 64)                                                                                        \
-    hipLaunchKernelGGL((hop_count_sample_kernel<GG, 64>), dim3(grid, n), dim3(256), 0, st, g);          \
+    hipLaunchKernelGGL((hop_count_sample_kernel<GG, 64>), dim3((grid) * n), dim3(256), 0, st, g);          \
   else                                                                                                  \
-    hipLaunchKernelGGL((hop_count_sample_kernel<GG, (256 / GG)>), dim3(grid, n), dim3(256), 0, st, g);
+    hipLaunchKernelGGL((hop_count_sample_kernel<GG, (256 / GG)>), dim3((grid) * n), dim3(256), 0, st, g);
     switch (G) {
       case 4: LMI_FUSED(4) break;
       case 8: LMI_FUSED(8) break;
@@ -645,39 +659,39 @@ int launch_hop(Server *s, Pipe *const *pp, int n, hipStream_t st, int hop, bool 
     // dependent random accesses, so parallelism matters more than per-thread work
     const int64_t nm = std::max<int64_t>(n_max, 1);
     if (nm <= 256 * 1024)
-      hipLaunchKernelGGL(hop_count_scan_kernel<1>, dim3((int)ceil_div(nm, kScanBlock), n), dim3(kScanBlock), 0, st, g);
+      hipLaunchKernelGGL(hop_count_scan_kernel<1>, dim3(((int)ceil_div(nm, kScanBlock)) * n), dim3(kScanBlock), 0, st, g);
     else if (nm <= 512 * 1024)
-      hipLaunchKernelGGL(hop_count_scan_kernel<2>, dim3((int)ceil_div(nm, kScanBlock * 2), n), dim3(kScanBlock), 0, st, g);
+      hipLaunchKernelGGL(hop_count_scan_kernel<2>, dim3(((int)ceil_div(nm, kScanBlock * 2)) * n), dim3(kScanBlock), 0, st, g);
     else if (nm <= 1024 * 1024)
-      hipLaunchKernelGGL(hop_count_scan_kernel<4>, dim3((int)ceil_div(nm, kScanBlock * 4), n), dim3(kScanBlock), 0, st, g);
+      hipLaunchKernelGGL(hop_count_scan_kernel<4>, dim3(((int)ceil_div(nm, kScanBlock * 4)) * n), dim3(kScanBlock), 0, st, g);
     else
-      hipLaunchKernelGGL(hop_count_scan_kernel<8>, dim3((int)ceil_div(nm, kScanBlock * 8), n), dim3(kScanBlock), 0, st, g);
+      hipLaunchKernelGGL(hop_count_scan_kernel<8>, dim3(((int)ceil_div(nm, kScanBlock * 8)) * n), dim3(kScanBlock), 0, st, g);
     const int grid = (int)std::min<int64_t>(ceil_div(n_max * G, 256), 8192);
     if (s->lds_dedup) {
       switch (G) {
-        case 4: hipLaunchKernelGGL(hop_sample_lds_kernel<4>, dim3(grid, n), dim3(256), 0, st, g); break;
-        case 8: hipLaunchKernelGGL(hop_sample_lds_kernel<8>, dim3(grid, n), dim3(256), 0, st, g); break;
-        case 16: hipLaunchKernelGGL(hop_sample_lds_kernel<16>, dim3(grid, n), dim3(256), 0, st, g); break;
-        case 32: hipLaunchKernelGGL(hop_sample_lds_kernel<32>, dim3(grid, n), dim3(256), 0, st, g); break;
-        default: hipLaunchKernelGGL(hop_sample_lds_kernel<64>, dim3(grid, n), dim3(256), 0, st, g); break;
+        case 4: hipLaunchKernelGGL(hop_sample_lds_kernel<4>, dim3((grid) * n), dim3(256), 0, st, g); break;
+        case 8: hipLaunchKernelGGL(hop_sample_lds_kernel<8>, dim3((grid) * n), dim3(256), 0, st, g); break;
+        case 16: hipLaunchKernelGGL(hop_sample_lds_kernel<16>, dim3((grid) * n), dim3(256), 0, st, g); break;
+        case 32: hipLaunchKernelGGL(hop_sample_lds_kernel<32>, dim3((grid) * n), dim3(256), 0, st, g); break;
+        default: hipLaunchKernelGGL(hop_sample_lds_kernel<64>, dim3((grid) * n), dim3(256), 0, st, g); break;
       }
     } else {
       switch (G) {
-        case 4: hipLaunchKernelGGL(hop_sample_kernel<4>, dim3(grid, n), dim3(256), 0, st, g); break;
-        case 8: hipLaunchKernelGGL(hop_sample_kernel<8>, dim3(grid, n), dim3(256), 0, st, g); break;
-        case 16: hipLaunchKernelGGL(hop_sample_kernel<16>, dim3(grid, n), dim3(256), 0, st, g); break;
-        case 32: hipLaunchKernelGGL(hop_sample_kernel<32>, dim3(grid, n), dim3(256), 0, st, g); break;
-        default: hipLaunchKernelGGL(hop_sample_kernel<64>, dim3(grid, n), dim3(256), 0, st, g); break;
+        case 4: hipLaunchKernelGGL(hop_sample_kernel<4>, dim3((grid) * n), dim3(256), 0, st, g); break;
+        case 8: hipLaunchKernelGGL(hop_sample_kernel<8>, dim3((grid) * n), dim3(256), 0, st, g); break;
+        case 16: hipLaunchKernelGGL(hop_sample_kernel<16>, dim3((grid) * n), dim3(256), 0, st, g); break;
+        case 32: hipLaunchKernelGGL(hop_sample_kernel<32>, dim3((grid) * n), dim3(256), 0, st, g); break;
+        default: hipLaunchKernelGGL(hop_sample_kernel<64>, dim3((grid) * n), dim3(256), 0, st, g); break;
       }
     }
   }
   const int64_t em = std::max<int64_t>(e_max, 1);
   if (em <= 1024 * 1024)
-    hipLaunchKernelGGL(hop_flag_scan_kernel<2>, dim3((int)ceil_div(em, kScanBlock * 2), n), dim3(kScanBlock), 0, st, g);
+    hipLaunchKernelGGL(hop_flag_scan_kernel<2>, dim3(((int)ceil_div(em, kScanBlock * 2)) * n), dim3(kScanBlock), 0, st, g);
   else if (em <= 2560 * 1024)
-    hipLaunchKernelGGL(hop_flag_scan_kernel<4>, dim3((int)ceil_div(em, kScanBlock * 4), n), dim3(kScanBlock), 0, st, g);
+    hipLaunchKernelGGL(hop_flag_scan_kernel<4>, dim3(((int)ceil_div(em, kScanBlock * 4)) * n), dim3(kScanBlock), 0, st, g);
   else
-    hipLaunchKernelGGL(hop_flag_scan_kernel<8>, dim3((int)ceil_div(em, kScanBlock * 8), n), dim3(kScanBlock), 0, st, g);
+    hipLaunchKernelGGL(hop_flag_scan_kernel<8>, dim3(((int)ceil_div(em, kScanBlock * 8)) * n), dim3(kScanBlock), 0, st, g);
   LMI_HIP(hipGetLastError());
   for (int k = 0; k < n; ++k) {
     pp[k]->fill_pending = hop;
@@ -705,11 +719,12 @@ int launch_fill(Server *s, Pipe *const *pp, int n, hipStream_t st) {
   const int hop = pp[0]->fill_pending;
   if (hop < 0) return LMI_OK;
   FillGroup g{};
+  g.n = n;
   for (int k = 0; k < n; ++k) {
     g.p[k] = fill_args(*pp[k], hop);
     pp[k]->fill_pending = -1;
   }
-  hipLaunchKernelGGL(hop_fill_kernel, dim3(fill_blocks(s->edge_cap[hop], 256), n), dim3(256), 0, st, g);
+  hipLaunchKernelGGL(hop_fill_kernel, dim3((fill_blocks(s->edge_cap[hop], 256)) * n), dim3(256), 0, st, g);
   LMI_HIP(hipGetLastError());
   return LMI_OK;
 }

@@ -214,6 +214,8 @@ def test_groups_of_batches_share_their_launches(lmi, oracle, group, fanout, cach
     stream = lmi.stream_create()
     slot_ref = q = sc = None
     try:
+        if group == 3:
+            srv.tune("protect_hits", 1)   # HBM gathers held back until earlier host-link gathers have drained
         srv.load_graph(indptr, indices)
         srv.attach_features(feats)
         srv.load_idset(lmi.MODE_TRAIN, train)
