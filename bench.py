@@ -232,9 +232,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="paper100m", choices=sorted(WORKLOADS))
     ap.add_argument("--scale", type=float, default=1.0, help="shrink node/train counts (testing only)")
-    ap.add_argument("--pipes", type=int, default=4, help="output buffer sets in flight")
+    ap.add_argument("--pipes", type=int, default=8, help="output buffer sets in flight")
     ap.add_argument("--streams", type=int, default=1, help="caller streams the pipes are spread over")
-    ap.add_argument("--group", type=int, default=2,
+    ap.add_argument("--group", type=int, default=4,
                     help="mini-batches issued together with lmi_run_group (their sampling kernels share launches)")
     ap.add_argument("--seed", type=int, default=20260101)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget (0 = skip)")
@@ -264,9 +264,10 @@ def main():
                                {"hash": 0, "direct": 1, "rank": 2}[args.table], args.policy)
     tunes = dict(kv.split("=") for kv in args.tune)
     if args.group > 1:
-        # with two batches per launch the sampling phase is short enough that the host link sets the
-        # pace: a few more host-link blocks than the library's default of 32 (measured: 36 -> 6.0 k
-        # batches/s with the HBM gather at 62 % of peak, 40 -> 5.8 k at 65 %, 44 -> 5.65 k at 66 %)
+        # with several batches per launch the sampling phase is short enough that the host link sets
+        # the pace: a few more host-link blocks than the library's default of 32 (measured on
+        # paper100m-shaped, groups of 4 on 8 pipes: 32 -> 6.7 k batches/s with the HBM gather at 59 %
+        # of peak, 36 -> 7.1 k at 62 %, 40 -> 7.0 k at 62 %, 48 -> 6.8 k at 62 %, 64 -> 6.0 k at 65 %)
         tunes.setdefault("miss_blocks", "40")
     for k, v in tunes.items():
         srv.tune(k, int(v))
@@ -285,7 +286,7 @@ def main():
         print("bench.py: --group needs a pipe count that is a multiple of it, and no LRU cache", file=sys.stderr)
         sys.exit(2)
 
-    def step(i):
+    def step(i, n=None):
         # consecutive batches alternate output buffer sets (pipes), so the host-link part of batch i
         # (on the server's side stream) overlaps the sampling of batch i+1; a pipe always uses the
         # same caller stream.  With --group g, batches i .. i+g-1 are issued together (step is then
@@ -295,13 +296,12 @@ def main():
             srv.run_once(plan[i] if plan else None, batch_counter=i % steps_per_epoch, rng_seed=args.seed + i, pipe=p,
                          stream=streams[p % len(streams)])
         else:
-            ks = range(i, i + group)
+            ks = range(i, i + (n or group))   # the timed region's last group may be a partial one
             srv.run_group([k % args.pipes for k in ks], [k % steps_per_epoch for k in ks],
                           seeds=[plan[k] for k in ks] if plan else None, rng_seeds=[args.seed + k for k in ks],
                           stream=streams[(p // group) % len(streams)])
 
-    args.warmup = -(-args.warmup // group) * group   # whole groups
-    args.steps = -(-args.steps // group) * group
+    args.warmup = -(-args.warmup // group) * group   # whole groups, so that the timed region starts on pipe 0
     for i in range(0, args.warmup, group):
         step(i)
     lmi.check(lmi.lib().lmi_device_sync())
@@ -313,7 +313,7 @@ def main():
     srv.profile_enable(2)
     t0 = time.perf_counter()
     for i in range(args.warmup, args.warmup + args.steps, group):
-        step(i)
+        step(i, min(group, args.warmup + args.steps - i))   # exactly --steps batches
     lmi.check(lmi.lib().lmi_device_sync())
     t1 = time.perf_counter()
     srv.profile_enable(0)
@@ -322,7 +322,8 @@ def main():
     # untimed extra leg with every phase of every batch bracketed (level 1), for the per-phase breakdown only
     srv.tune("profile_every", 1)
     srv.profile_enable(1)
-    for i in range(args.warmup + args.steps, args.warmup + args.steps + -(-min(args.steps, 20) // group) * group, group):
+    leg = -(-(args.warmup + args.steps) // group) * group
+    for i in range(leg, leg + -(-min(args.steps, 20) // group) * group, group):
         step(i)
     srv.profile_enable(0)
     phases = srv.profile_read(reset=True)
@@ -333,6 +334,9 @@ def main():
         hit_bytes = w["dim"] + 4 + rb + 8
     else:
         hit_bytes = 2 * rb + 8
+    # a group's hit gathers are one launch (fp32 rows, hits on the caller's stream); the host-link
+    # gathers and the int8 gathers stay one launch per batch
+    hit_batches = group if (info["cache_kind"] != "int8" and int(tunes.get("split_miss", 1)) == 1) else 1
     hit_ms = prof.gather_hit_ms / max(prof.gather_hit_launches, 1)
     hit_rows = prof.gather_hit_rows / max(prof.gather_hit_launches, 1)
     miss_ms = prof.gather_miss_ms / max(prof.gather_miss_launches, 1)
@@ -343,7 +347,8 @@ def main():
     roofline = dict(bound="hbm", kernel="move_rows_kernel<u32x4,32,1,true,false> (HBM gather of cache hits)", achieved=round(achieved, 1),
                     peak=HBM_PEAK_GBS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBS, 4),
                     traffic=recorded_traffic(args.workload) if args.scale == 1.0 else None,
-                    rows_per_launch=round(hit_rows, 1), bytes_per_row=hit_bytes, avg_launch_ms=round(hit_ms, 4),
+                    rows_per_launch=round(hit_rows, 1), batches_per_launch=hit_batches, bytes_per_row=hit_bytes,
+                    avg_launch_ms=round(hit_ms, 4),
                     measured_copy_gbs=round(copy_gbs, 1))
     link_bytes = min(1 << 28, info["feats"].nbytes)
     link_ms = lmi.bench_host_read(info["feats"], link_bytes)
@@ -374,8 +379,8 @@ def main():
         "cache_hit_rate": round(prof.gather_hit_rows / total_rows, 4) if total_rows else None,
         "rows_per_batch": round(total_rows / max(prof.gather_hit_launches, prof.gather_miss_launches, 1), 1),
         "profiled_batches": int(max(prof.gather_hit_launches, prof.gather_miss_launches)),
-        "phase_ms_per_batch": {"sample_dedup_lookup": round(phases.sample_ms / max(phases.sample_launches, 1), 4),
-                               "gather_hit": round(hit_ms, 4), "gather_miss_side_stream": round(miss_ms, 4)},
+        "phase_ms_per_batch": {"sample_dedup_lookup": round(phases.sample_ms / max(phases.sample_launches, 1) / group, 4),
+                               "gather_hit": round(hit_ms / hit_batches, 4), "gather_miss_side_stream": round(miss_ms, 4)},
         "roofline": roofline, "host_link": host_link,
     }
     if args.cpu_seconds > 0:

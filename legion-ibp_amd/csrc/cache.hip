@@ -32,18 +32,34 @@ namespace lmi {
 // row, each moving sizeof(V) bytes per step, with U rows in flight per lane.
 // HOSTLINK only names the instantiation that reads over the host link, so that
 // profiles list the HBM gather and the host-link gather as two kernels.
+// One launch can serve several pipes (output buffers): their blocks interleave over
+// blockIdx.x like those of the sampling kernels, and the source table is shared.
+struct MoveRow {
+  const int2 *list;
+  const int32_t *first_ptr, *n_ptr, *src_index, *dst_index;
+  uint8_t *dst;
+};
+struct MoveGroup {
+  MoveRow p[LMI_MAX_PIPES];
+  int n;
+};
+
 template <typename V, int LPR, int U, bool NT, bool HOSTLINK>
 static __global__ __launch_bounds__(256) void move_rows_kernel(
-    const int2 *list, const int32_t *first_ptr, const int32_t *n_ptr, const int32_t *src_index,
-    const int32_t *dst_index, int src_from_list, const uint8_t *src, uint8_t *dst, int chunks,
-    int64_t src_row_bytes, int64_t dst_row_bytes, unsigned long long *row_counter) {
-  const int n = *n_ptr;
-  const int first = first_ptr ? *first_ptr : 0;
-  if (row_counter && blockIdx.x == 0 && threadIdx.x == 0 && n > first)
+    MoveGroup g, int src_from_list, const uint8_t *src, int chunks, int64_t src_row_bytes, int64_t dst_row_bytes,
+    unsigned long long *row_counter) {
+  LMI_GRID_ROW(g.n);
+  const MoveRow &r = g.p[row];
+  const int2 *list = r.list;
+  const int32_t *src_index = r.src_index, *dst_index = r.dst_index;
+  uint8_t *dst = r.dst;
+  const int n = *r.n_ptr;
+  const int first = r.first_ptr ? *r.first_ptr : 0;
+  if (row_counter && bx == 0 && threadIdx.x == 0 && n > first)
     atomicAdd(row_counter, (unsigned long long)(n - first));  // work items offered to this launch (profiling)
   const int lane = threadIdx.x & (LPR - 1);
-  const int group = (blockIdx.x * blockDim.x + threadIdx.x) / LPR;
-  const int n_groups = gridDim.x * blockDim.x / LPR;
+  const int group = (bx * blockDim.x + threadIdx.x) / LPR;
+  const int n_groups = gx * blockDim.x / LPR;
   for (int j0 = first + group; j0 < n; j0 += n_groups * U) {
     int64_t so[U], dofs[U];
 #pragma unroll
@@ -86,18 +102,16 @@ typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
 
 struct MoveArgs {
-  const int2 *list;
-  const int32_t *first_ptr, *n_ptr, *src_index, *dst_index;
+  MoveGroup g;     // per pipe: work list, bounds, index arrays, destination
   int src_from_list;
-  int max_blocks;  // 0 = fill the device
+  int max_blocks;  // per pipe; 0 = fill the device
   int unroll;      // 0 = the server's gather_unroll
   int host_link;   // the source is pinned host memory read over the host link
   unsigned long long *row_counter;  // device counter that receives the number of work items, or null
   hipEvent_t ev_start, ev_stop;     // stamped with the kernel's begin and end when not null (profiling)
   const uint8_t *src;
-  uint8_t *dst;
   int64_t src_row_bytes, dst_row_bytes, row_bytes;  // row_bytes = bytes moved per row
-  int64_t n_max;
+  int64_t n_max;   // per pipe
 };
 
 template <typename V, int LPR, int U>
@@ -106,14 +120,12 @@ static void launch_move_vlu(hipStream_t st, const MoveArgs &a, int grid, bool nt
   // with profiling on, the launch carries its own start / stop events
 #define LMI_MOVE(NT_, HL_)                                                                                      \
   if (a.ev_start)                                                                                               \
-    hipExtLaunchKernelGGL((move_rows_kernel<V, LPR, U, NT_, HL_>), dim3(grid), dim3(256), 0, st, a.ev_start,     \
-                          a.ev_stop, 0, a.list, a.first_ptr, a.n_ptr, a.src_index, a.dst_index,                  \
-                          a.src_from_list, a.src, a.dst, chunks, a.src_row_bytes, a.dst_row_bytes,               \
-                          a.row_counter);                                                                        \
+    hipExtLaunchKernelGGL((move_rows_kernel<V, LPR, U, NT_, HL_>), dim3(grid * a.g.n), dim3(256), 0, st,         \
+                          a.ev_start, a.ev_stop, 0, a.g, a.src_from_list, a.src, chunks, a.src_row_bytes,        \
+                          a.dst_row_bytes, a.row_counter);                                                       \
   else                                                                                                          \
-    hipLaunchKernelGGL((move_rows_kernel<V, LPR, U, NT_, HL_>), dim3(grid), dim3(256), 0, st, a.list,            \
-                       a.first_ptr, a.n_ptr, a.src_index, a.dst_index, a.src_from_list, a.src, a.dst, chunks,    \
-                       a.src_row_bytes, a.dst_row_bytes, a.row_counter)
+    hipLaunchKernelGGL((move_rows_kernel<V, LPR, U, NT_, HL_>), dim3(grid * a.g.n), dim3(256), 0, st, a.g,       \
+                       a.src_from_list, a.src, chunks, a.src_row_bytes, a.dst_row_bytes, a.row_counter)
   if (a.host_link) {
     LMI_MOVE(true, true);
   } else if (nt) {
@@ -150,8 +162,9 @@ static void launch_move_v(hipStream_t st, const MoveArgs &a, int grid, bool nt, 
 // power-of-two lane group that covers one row when possible.
 static int launch_move_rows(Server *s, hipStream_t st, const MoveArgs &a, bool nt) {
   if (a.n_max <= 0 || a.row_bytes <= 0) return LMI_OK;
-  const uintptr_t align = (uintptr_t)a.src | (uintptr_t)a.dst | (uintptr_t)a.src_row_bytes |
-                          (uintptr_t)a.dst_row_bytes | (uintptr_t)a.row_bytes;
+  if (a.g.n < 1 || a.g.n > LMI_MAX_PIPES) LMI_FAIL(LMI_ERR_ARG, "a row move serves 1..LMI_MAX_PIPES pipes");
+  uintptr_t align = (uintptr_t)a.src | (uintptr_t)a.src_row_bytes | (uintptr_t)a.dst_row_bytes | (uintptr_t)a.row_bytes;
+  for (int k = 0; k < a.g.n; ++k) align |= (uintptr_t)a.g.p[k].dst;
   int vec = (align % 16 == 0) ? 16 : (align % 8 == 0) ? 8 : 4;
   if (align % 4 != 0) LMI_FAIL(LMI_ERR_ARG, "feature rows must be 4-byte aligned");
   if (s->gather_vec == 4 || (s->gather_vec == 8 && vec == 16)) vec = s->gather_vec;  // narrower on request
@@ -436,18 +449,17 @@ int pipe_join(Pipe &p, hipStream_t st) {
   return LMI_OK;
 }
 
-// HBM gather of the cache hits of rows [first, last) on stream `st`.
-static int launch_hits(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last) {
+// int8 rows: dequantised inside the gather, one launch per pipe.
+static int launch_hits_int8(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last) {
   const int64_t n_max = s->node_cap[seg_last];
-  if (s->cache_kind == LMI_CACHE_INT8) {
-    const int dim = s->cfg.feat_dim;
-    const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(n_max, 4), (int64_t)s->n_cu * 8));
-    const int32_t *first_ptr = seg == 0 ? nullptr : &p.st->node_counter[9 + seg - 1];
-    const int32_t *n_ptr = &p.st->node_counter[9 + seg_last];
-    const int8_t *q = (const int8_t *)s->cache_data;
-    unsigned long long *rc = s->prof_on ? s->d_prof_rows : nullptr;
-    hipEvent_t e0, e1;
-    prof_kernel_events(s, PROF_GATHER_HIT, &e0, &e1);
+  const int dim = s->cfg.feat_dim;
+  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(n_max, 4), (int64_t)s->n_cu * 8));
+  const int32_t *first_ptr = seg == 0 ? nullptr : &p.st->node_counter[9 + seg - 1];
+  const int32_t *n_ptr = &p.st->node_counter[9 + seg_last];
+  const int8_t *q = (const int8_t *)s->cache_data;
+  unsigned long long *rc = s->prof_on ? s->d_prof_rows : nullptr;
+  hipEvent_t e0, e1;
+  prof_kernel_events(s, PROF_GATHER_HIT, &e0, &e1);
 #define LMI_INT8(KERN, OUT_T)                                                                                   \
   if (e0)                                                                                                       \
     hipExtLaunchKernelGGL((KERN), dim3(grid), dim3(256), 0, st, e0, e1, 0, first_ptr, n_ptr, p.cache_index, q,   \
@@ -455,34 +467,47 @@ static int launch_hits(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last
   else                                                                                                          \
     hipLaunchKernelGGL((KERN), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr, p.cache_index, q, s->cache_scale, \
                        (OUT_T *)p.features, dim, rc)
-    const bool half = s->cfg.feat_dtype == LMI_F16;
-    if (dim % 16 == 0) {
-      const bool narrow = dim / 16 <= 32;
-      if (half && narrow) {
-        LMI_INT8((gather_int8_kernel<__half, 32>), __half);
-      } else if (half) {
-        LMI_INT8((gather_int8_kernel<__half, 64>), __half);
-      } else if (narrow) {
-        LMI_INT8((gather_int8_kernel<float, 32>), float);
-      } else {
-        LMI_INT8((gather_int8_kernel<float, 64>), float);
-      }
+  const bool half = s->cfg.feat_dtype == LMI_F16;
+  if (dim % 16 == 0) {
+    const bool narrow = dim / 16 <= 32;
+    if (half && narrow) {
+      LMI_INT8((gather_int8_kernel<__half, 32>), __half);
     } else if (half) {
-      LMI_INT8((gather_int8_generic_kernel<__half>), __half);
+      LMI_INT8((gather_int8_kernel<__half, 64>), __half);
+    } else if (narrow) {
+      LMI_INT8((gather_int8_kernel<float, 32>), float);
     } else {
-      LMI_INT8((gather_int8_generic_kernel<float>), float);
+      LMI_INT8((gather_int8_kernel<float, 64>), float);
     }
+  } else if (half) {
+    LMI_INT8((gather_int8_generic_kernel<__half>), __half);
+  } else {
+    LMI_INT8((gather_int8_generic_kernel<float>), float);
+  }
 #undef LMI_INT8
-    LMI_HIP(hipGetLastError());
+  LMI_HIP(hipGetLastError());
+  return LMI_OK;
+}
+
+// HBM gather of the cache hits of rows [first, last) on stream `st`, for all n pipes in one launch.
+static int launch_hits(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg, int seg_last) {
+  const int64_t n_max = s->node_cap[seg_last];
+  if (s->cache_kind == LMI_CACHE_INT8) {
+    for (int k = 0; k < n; ++k) LMI_TRY(launch_hits_int8(s, *pp[k], st, seg, seg_last));
     return LMI_OK;
   }
   MoveArgs m{};
-  m.list = nullptr;  // rows [first, n) directly; cache_index < 0 (a miss) skips the row
-  m.first_ptr = seg == 0 ? nullptr : &p.st->node_counter[9 + seg - 1];
-  m.n_ptr = &p.st->node_counter[9 + seg_last];
-  m.src_index = p.cache_index;
+  m.g.n = n;
+  for (int k = 0; k < n; ++k) {
+    const Pipe &p = *pp[k];
+    MoveRow &r = m.g.p[k];
+    r.list = nullptr;  // rows [first, n) directly; cache_index < 0 (a miss) skips the row
+    r.first_ptr = seg == 0 ? nullptr : &p.st->node_counter[9 + seg - 1];
+    r.n_ptr = &p.st->node_counter[9 + seg_last];
+    r.src_index = p.cache_index;
+    r.dst = (uint8_t *)p.features;
+  }
   m.src = s->cache_data;
-  m.dst = (uint8_t *)p.features;
   m.src_row_bytes = m.dst_row_bytes = m.row_bytes = s->row_bytes;
   m.n_max = n_max;
   m.row_counter = s->prof_on ? s->d_prof_rows : nullptr;  // all rows of the segment: hits + misses
@@ -494,11 +519,13 @@ static int launch_hits(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last
 // small grid when the table sits behind the host link (few bytes in flight fill it).
 static int launch_misses(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last) {
   MoveArgs m{};
-  m.list = p.miss_list + seg_list_base(s, seg);
-  m.n_ptr = &p.st->n_miss[seg];
+  m.g.n = 1;
+  MoveRow &r = m.g.p[0];
+  r.list = p.miss_list + seg_list_base(s, seg);
+  r.n_ptr = &p.st->n_miss[seg];
   m.src_from_list = 1;
   m.src = s->feat;
-  m.dst = (uint8_t *)p.features;
+  r.dst = (uint8_t *)p.features;
   m.src_row_bytes = m.dst_row_bytes = m.row_bytes = s->row_bytes;
   m.n_max = s->node_cap[seg_last];
   if (s->feat_loc == LMI_LOC_HOST) {
@@ -531,7 +558,7 @@ int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int s
   hipEvent_t closing = prof_phase(s, st, &s->prof_open, -1);
   if (mode == 0) {
     for (int k = 0; k < n; ++k) {
-      if (have_cache) LMI_TRY(launch_hits(s, *pp[k], st, seg, seg_last));
+      if (have_cache) LMI_TRY(launch_hits(s, pp + k, 1, st, seg, seg_last));
       LMI_TRY(launch_misses(s, *pp[k], st, seg, seg_last));
       if (lru_lists > 0) LMI_TRY(launch_lru_insert(s, *pp[k], st, lru_lists));
     }
@@ -549,7 +576,7 @@ int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int s
         s->side_busy = false;
       }
     }
-    for (int k = 0; k < n; ++k) LMI_TRY(launch_hits(s, *pp[k], st, seg, seg_last));
+    LMI_TRY(launch_hits(s, pp, n, st, seg, seg_last));  // one launch for the group
     fork = nullptr;
   }
   if (!fork) {  // one fork for the whole group
@@ -559,7 +586,7 @@ int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int s
   LMI_HIP(hipStreamWaitEvent(s->side, fork, 0));
   for (int k = 0; k < n; ++k) {
     Pipe &p = *pp[k];
-    if (mode == 2) LMI_TRY(launch_hits(s, p, s->side, seg, seg_last));
+    if (mode == 2) LMI_TRY(launch_hits(s, pp + k, 1, s->side, seg, seg_last));
     LMI_TRY(launch_misses(s, p, s->side, seg, seg_last));
     if (lru_lists > 0) LMI_TRY(launch_lru_insert(s, p, s->side, lru_lists));  // reads the rows just gathered
     LMI_HIP(hipEventRecord(p.join, s->side));
@@ -664,13 +691,15 @@ int launch_lru_insert(Server *s, Pipe &p, hipStream_t st, int n_lists) {
   // copy the granted rows from the output buffer (already gathered) into the cache
   for (int l = 0; l < n_lists; ++l) {
     MoveArgs m{};
-    m.list = p.miss_list + seg_list_base(s, l);
-    m.n_ptr = &p.st->n_miss[l];
-    m.src_index = nullptr;
+    m.g.n = 1;
+    MoveRow &r = m.g.p[0];
+    r.list = p.miss_list + seg_list_base(s, l);
+    r.n_ptr = &p.st->n_miss[l];
+    r.src_index = nullptr;
     m.src_from_list = 0;
-    m.dst_index = p.lru_fill;
+    r.dst_index = p.lru_fill;
     m.src = (const uint8_t *)p.features;
-    m.dst = s->cache_data;
+    r.dst = s->cache_data;
     m.src_row_bytes = m.dst_row_bytes = m.row_bytes = s->row_bytes;
     m.n_max = s->node_cap[s->cfg.hops];
     LMI_TRY(launch_move_rows(s, st, m, false));
@@ -945,12 +974,11 @@ int cache_build_static(Server *s, int64_t capacity_rows, int table_kind, bool in
     LMI_HIP(hipGetLastError());
   } else {
     MoveArgs m{};
-    m.list = nullptr;
-    m.n_ptr = d_n;
-    m.src_index = d_cached;
-    m.dst_index = nullptr;
+    m.g.n = 1;
+    m.g.p[0].n_ptr = d_n;
+    m.g.p[0].src_index = d_cached;
+    m.g.p[0].dst = s->cache_data;
     m.src = s->feat;
-    m.dst = s->cache_data;
     m.src_row_bytes = m.dst_row_bytes = m.row_bytes = s->row_bytes;
     m.n_max = cap;
     LMI_TRY(launch_move_rows(s, 0, m, false));
