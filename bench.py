@@ -265,10 +265,11 @@ def main():
     tunes = dict(kv.split("=") for kv in args.tune)
     if args.group > 1:
         # with several batches per launch the sampling phase is short enough that the host link sets
-        # the pace: a few more host-link blocks than the library's default of 32 (measured on
-        # paper100m-shaped, groups of 4 on 8 pipes: 32 -> 6.7 k batches/s with the HBM gather at 59 %
-        # of peak, 36 -> 7.1 k at 62 %, 40 -> 7.0 k at 62 %, 48 -> 6.8 k at 62 %, 64 -> 6.0 k at 65 %)
-        tunes.setdefault("miss_blocks", "40")
+        # the pace: a few more host-link blocks than the library's default of 32, shared by the group's
+        # batches (measured on paper100m-shaped, groups of 4 on 8 pipes: 28 -> 7.0 k batches/s with the
+        # HBM gather at 59 % of peak, the side stream never idle; 32 -> 7.3 k at 62 %; 36 -> 7.1 k at
+        # 62 %; 40 -> 6.8 k at 62 %; 48 -> 6.4 k at 64 %)
+        tunes.setdefault("miss_blocks", "36")
     for k, v in tunes.items():
         srv.tune(k, int(v))
     steps_per_epoch = -(-info["n_train"] // w["batch"])
@@ -334,9 +335,11 @@ def main():
         hit_bytes = w["dim"] + 4 + rb + 8
     else:
         hit_bytes = 2 * rb + 8
-    # a group's hit gathers are one launch (fp32 rows, hits on the caller's stream); the host-link
-    # gathers and the int8 gathers stay one launch per batch
-    hit_batches = group if (info["cache_kind"] != "int8" and int(tunes.get("split_miss", 1)) == 1) else 1
+    # a group's hit gathers are one launch (fp32 rows, hits on the caller's stream) and so are its
+    # host-link gathers (on the side stream); the int8 gathers stay one launch per batch
+    split = int(tunes.get("split_miss", 1)) == 1
+    hit_batches = group if (info["cache_kind"] != "int8" and split) else 1
+    miss_batches = group if (split and int(tunes.get("group_miss", 1))) else 1
     hit_ms = prof.gather_hit_ms / max(prof.gather_hit_launches, 1)
     hit_rows = prof.gather_hit_rows / max(prof.gather_hit_launches, 1)
     miss_ms = prof.gather_miss_ms / max(prof.gather_miss_launches, 1)
@@ -356,8 +359,10 @@ def main():
                      measured_stream_read_gbs=round(link_bytes // 16 * 16 / (link_ms * 1e-3) / 1e9, 2),
                      achieved=round(miss_rows * rb / (miss_ms * 1e-3) / 1e9, 2) if miss_ms > 0 else 0.0,
                      peak=HOST_LINK_PEAK_GBS, unit="GB/s", rows_per_launch=round(miss_rows, 1),
+                     batches_per_launch=miss_batches,
                      avg_launch_ms=round(miss_ms, 4))
     total_rows = prof.gather_hit_rows + prof.gather_miss_rows
+    profiled_batches = int(max(prof.gather_hit_launches * hit_batches, prof.gather_miss_launches * miss_batches))
     out = {
         "metric": "sampled mini-batches/sec", "value": round(args.steps / (t1 - t0), 2), "unit": "batches/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
@@ -377,10 +382,11 @@ def main():
         "feature_gather_gbs": round(achieved, 1),
         "feature_gather_frac_hbm_peak": round(achieved / HBM_PEAK_GBS, 4),
         "cache_hit_rate": round(prof.gather_hit_rows / total_rows, 4) if total_rows else None,
-        "rows_per_batch": round(total_rows / max(prof.gather_hit_launches, prof.gather_miss_launches, 1), 1),
-        "profiled_batches": int(max(prof.gather_hit_launches, prof.gather_miss_launches)),
+        "rows_per_batch": round(total_rows / max(profiled_batches, 1), 1),
+        "profiled_batches": profiled_batches,
         "phase_ms_per_batch": {"sample_dedup_lookup": round(phases.sample_ms / max(phases.sample_launches, 1) / group, 4),
-                               "gather_hit": round(hit_ms / hit_batches, 4), "gather_miss_side_stream": round(miss_ms, 4)},
+                               "gather_hit": round(hit_ms / hit_batches, 4),
+                               "gather_miss_side_stream": round(miss_ms / miss_batches, 4)},
         "roofline": roofline, "host_link": host_link,
     }
     if args.cpu_seconds > 0:

@@ -517,19 +517,23 @@ static int launch_hits(Server *s, Pipe *const *pp, int n, hipStream_t st, int se
 
 // Gather of the rows on the segment's miss list from the feature table, on a
 // small grid when the table sits behind the host link (few bytes in flight fill it).
-static int launch_misses(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last) {
+// One launch for all n pipes; the small grid is then shared between them.
+static int launch_misses(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg, int seg_last) {
   MoveArgs m{};
-  m.g.n = 1;
-  MoveRow &r = m.g.p[0];
-  r.list = p.miss_list + seg_list_base(s, seg);
-  r.n_ptr = &p.st->n_miss[seg];
+  m.g.n = n;
+  for (int k = 0; k < n; ++k) {
+    MoveRow &r = m.g.p[k];
+    r.list = pp[k]->miss_list + seg_list_base(s, seg);
+    r.n_ptr = &pp[k]->st->n_miss[seg];
+    r.dst = (uint8_t *)pp[k]->features;
+  }
   m.src_from_list = 1;
   m.src = s->feat;
-  r.dst = (uint8_t *)p.features;
   m.src_row_bytes = m.dst_row_bytes = m.row_bytes = s->row_bytes;
   m.n_max = s->node_cap[seg_last];
   if (s->feat_loc == LMI_LOC_HOST) {
-    m.max_blocks = s->miss_blocks > 0 ? s->miss_blocks : s->n_cu;
+    const int blocks = s->miss_blocks > 0 ? s->miss_blocks : s->n_cu;
+    m.max_blocks = std::max(1, (blocks + n - 1) / n);  // per pipe
     m.unroll = s->miss_unroll;
     m.host_link = 1;
   }
@@ -559,7 +563,7 @@ int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int s
   if (mode == 0) {
     for (int k = 0; k < n; ++k) {
       if (have_cache) LMI_TRY(launch_hits(s, pp + k, 1, st, seg, seg_last));
-      LMI_TRY(launch_misses(s, *pp[k], st, seg, seg_last));
+      LMI_TRY(launch_misses(s, pp + k, 1, st, seg, seg_last));
       if (lru_lists > 0) LMI_TRY(launch_lru_insert(s, *pp[k], st, lru_lists));
     }
     return LMI_OK;
@@ -584,10 +588,13 @@ int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int s
     LMI_HIP(hipEventRecord(fork, st));
   }
   LMI_HIP(hipStreamWaitEvent(s->side, fork, 0));
+  // the group's host-link gathers as one launch when nothing has to come between them
+  const bool misses_together = n > 1 && mode == 1 && lru_lists == 0 && s->group_miss;
+  if (misses_together) LMI_TRY(launch_misses(s, pp, n, s->side, seg, seg_last));
   for (int k = 0; k < n; ++k) {
     Pipe &p = *pp[k];
     if (mode == 2) LMI_TRY(launch_hits(s, pp + k, 1, s->side, seg, seg_last));
-    LMI_TRY(launch_misses(s, p, s->side, seg, seg_last));
+    if (!misses_together) LMI_TRY(launch_misses(s, pp + k, 1, s->side, seg, seg_last));
     if (lru_lists > 0) LMI_TRY(launch_lru_insert(s, p, s->side, lru_lists));  // reads the rows just gathered
     LMI_HIP(hipEventRecord(p.join, s->side));
     p.side_pending = true;
