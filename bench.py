@@ -335,10 +335,10 @@ def main():
         hit_bytes = w["dim"] + 4 + rb + 8
     else:
         hit_bytes = 2 * rb + 8
-    # a group's hit gathers are one launch (fp32 rows, hits on the caller's stream) and so are its
-    # host-link gathers (on the side stream); the int8 gathers stay one launch per batch
+    # a group's hit gathers are one launch (on the caller's stream) and so are its host-link
+    # gathers (on the side stream)
     split = int(tunes.get("split_miss", 1)) == 1
-    hit_batches = group if (info["cache_kind"] != "int8" and split) else 1
+    hit_batches = group if split else 1
     miss_batches = group if (split and int(tunes.get("group_miss", 1))) else 1
     hit_ms = prof.gather_hit_ms / max(prof.gather_hit_launches, 1)
     hit_rows = prof.gather_hit_rows / max(prof.gather_hit_launches, 1)
@@ -347,7 +347,12 @@ def main():
     achieved = hit_rows * hit_bytes / (hit_ms * 1e-3) / 1e9 if hit_ms > 0 else 0.0
     copy_ms = lmi.bench_copy(1 << 30, 10)
     copy_gbs = 2 * (1 << 30) / (copy_ms * 1e-3) / 1e9
-    roofline = dict(bound="hbm", kernel="move_rows_kernel<u32x4,32,1,true,false> (HBM gather of cache hits)", achieved=round(achieved, 1),
+    if info["cache_kind"] == "int8":
+        hit_kernel = "gather_int8_kernel<%s,%d> (HBM gather of cache hits, dequantisation fused)" % (
+            "__half" if w["dtype"] == "f16" else "float", 32 if w["dim"] // 16 <= 32 else 64)
+    else:
+        hit_kernel = "move_rows_kernel<u32x4,32,1,true,false> (HBM gather of cache hits)"
+    roofline = dict(bound="hbm", kernel=hit_kernel, achieved=round(achieved, 1),
                     peak=HBM_PEAK_GBS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBS, 4),
                     traffic=recorded_traffic(args.workload) if args.scale == 1.0 else None,
                     rows_per_launch=round(hit_rows, 1), batches_per_launch=hit_batches, bytes_per_row=hit_bytes,

@@ -219,17 +219,21 @@ static __global__ __launch_bounds__(256) void quantize_rows_kernel(
 
 // Dequantising gather for hits of the int8 cache, 16 elements per lane:
 // y = float(q) * scale, rounded to the output type (RNE for fp16).
+// Like the row mover, one launch serves several pipes (MoveGroup: src_index = slot per row,
+// dst = the pipe's output rows).
 template <typename OUT, int LPR>
-static __global__ __launch_bounds__(256) void gather_int8_kernel(
-    const int32_t *first_ptr, const int32_t *n_ptr, const int32_t *cache_index, const int8_t *q,
-    const float *scale, OUT *out, int dim, unsigned long long *row_counter) {
-  const int n = *n_ptr;
-  const int first = first_ptr ? *first_ptr : 0;
-  if (row_counter && blockIdx.x == 0 && threadIdx.x == 0 && n > first)
+static __global__ __launch_bounds__(256) void gather_int8_kernel(MoveGroup g, const int8_t *q, const float *scale,
+                                                                 int dim, unsigned long long *row_counter) {
+  LMI_GRID_ROW(g.n);
+  const int32_t *cache_index = g.p[row].src_index;
+  OUT *out = reinterpret_cast<OUT *>(g.p[row].dst);
+  const int n = *g.p[row].n_ptr;
+  const int first = g.p[row].first_ptr ? *g.p[row].first_ptr : 0;
+  if (row_counter && bx == 0 && threadIdx.x == 0 && n > first)
     atomicAdd(row_counter, (unsigned long long)(n - first));
   const int lane = threadIdx.x & (LPR - 1);
-  const int group = (blockIdx.x * blockDim.x + threadIdx.x) / LPR;
-  const int n_groups = gridDim.x * blockDim.x / LPR;
+  const int group = (bx * blockDim.x + threadIdx.x) / LPR;
+  const int n_groups = gx * blockDim.x / LPR;
   const int chunks = dim / 16;
   for (int i = first + group; i < n; i += n_groups) {
     const int slot = cache_index[i];
@@ -259,16 +263,19 @@ static __global__ __launch_bounds__(256) void gather_int8_kernel(
 
 // Element-wise fallback for row lengths that are not a multiple of 16.
 template <typename OUT>
-static __global__ __launch_bounds__(256) void gather_int8_generic_kernel(
-    const int32_t *first_ptr, const int32_t *n_ptr, const int32_t *cache_index, const int8_t *q,
-    const float *scale, OUT *out, int dim, unsigned long long *row_counter) {
-  const int n = *n_ptr;
-  const int first = first_ptr ? *first_ptr : 0;
-  if (row_counter && blockIdx.x == 0 && threadIdx.x == 0 && n > first)
+static __global__ __launch_bounds__(256) void gather_int8_generic_kernel(MoveGroup g, const int8_t *q,
+                                                                         const float *scale, int dim,
+                                                                         unsigned long long *row_counter) {
+  LMI_GRID_ROW(g.n);
+  const int32_t *cache_index = g.p[row].src_index;
+  OUT *out = reinterpret_cast<OUT *>(g.p[row].dst);
+  const int n = *g.p[row].n_ptr;
+  const int first = g.p[row].first_ptr ? *g.p[row].first_ptr : 0;
+  if (row_counter && bx == 0 && threadIdx.x == 0 && n > first)
     atomicAdd(row_counter, (unsigned long long)(n - first));
   const int lane = threadIdx.x & (kWave - 1);
-  const int wave = (blockIdx.x * blockDim.x + threadIdx.x) / kWave;
-  const int n_waves = gridDim.x * blockDim.x / kWave;
+  const int wave = (bx * blockDim.x + threadIdx.x) / kWave;
+  const int n_waves = gx * blockDim.x / kWave;
   for (int i = first + wave; i < n; i += n_waves) {
     const int slot = cache_index[i];
     if (slot < 0) continue;
@@ -449,40 +456,36 @@ int pipe_join(Pipe &p, hipStream_t st) {
   return LMI_OK;
 }
 
-// int8 rows: dequantised inside the gather, one launch per pipe.
-static int launch_hits_int8(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last) {
+// int8 rows: dequantised inside the gather.
+static int launch_hits_int8(Server *s, const MoveGroup &g, hipStream_t st, int seg_last) {
   const int64_t n_max = s->node_cap[seg_last];
   const int dim = s->cfg.feat_dim;
-  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(n_max, 4), (int64_t)s->n_cu * 8));
-  const int32_t *first_ptr = seg == 0 ? nullptr : &p.st->node_counter[9 + seg - 1];
-  const int32_t *n_ptr = &p.st->node_counter[9 + seg_last];
+  const int grid = g.n * (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(n_max, 4), (int64_t)s->n_cu * 8));
   const int8_t *q = (const int8_t *)s->cache_data;
   unsigned long long *rc = s->prof_on ? s->d_prof_rows : nullptr;
   hipEvent_t e0, e1;
   prof_kernel_events(s, PROF_GATHER_HIT, &e0, &e1);
-#define LMI_INT8(KERN, OUT_T)                                                                                   \
-  if (e0)                                                                                                       \
-    hipExtLaunchKernelGGL((KERN), dim3(grid), dim3(256), 0, st, e0, e1, 0, first_ptr, n_ptr, p.cache_index, q,   \
-                          s->cache_scale, (OUT_T *)p.features, dim, rc);                                         \
-  else                                                                                                          \
-    hipLaunchKernelGGL((KERN), dim3(grid), dim3(256), 0, st, first_ptr, n_ptr, p.cache_index, q, s->cache_scale, \
-                       (OUT_T *)p.features, dim, rc)
+#define LMI_INT8(KERN)                                                                                   \
+  if (e0)                                                                                                \
+    hipExtLaunchKernelGGL((KERN), dim3(grid), dim3(256), 0, st, e0, e1, 0, g, q, s->cache_scale, dim, rc); \
+  else                                                                                                   \
+    hipLaunchKernelGGL((KERN), dim3(grid), dim3(256), 0, st, g, q, s->cache_scale, dim, rc)
   const bool half = s->cfg.feat_dtype == LMI_F16;
   if (dim % 16 == 0) {
     const bool narrow = dim / 16 <= 32;
     if (half && narrow) {
-      LMI_INT8((gather_int8_kernel<__half, 32>), __half);
+      LMI_INT8((gather_int8_kernel<__half, 32>));
     } else if (half) {
-      LMI_INT8((gather_int8_kernel<__half, 64>), __half);
+      LMI_INT8((gather_int8_kernel<__half, 64>));
     } else if (narrow) {
-      LMI_INT8((gather_int8_kernel<float, 32>), float);
+      LMI_INT8((gather_int8_kernel<float, 32>));
     } else {
-      LMI_INT8((gather_int8_kernel<float, 64>), float);
+      LMI_INT8((gather_int8_kernel<float, 64>));
     }
   } else if (half) {
-    LMI_INT8((gather_int8_generic_kernel<__half>), __half);
+    LMI_INT8((gather_int8_generic_kernel<__half>));
   } else {
-    LMI_INT8((gather_int8_generic_kernel<float>), float);
+    LMI_INT8((gather_int8_generic_kernel<float>));
   }
 #undef LMI_INT8
   LMI_HIP(hipGetLastError());
@@ -492,10 +495,6 @@ static int launch_hits_int8(Server *s, Pipe &p, hipStream_t st, int seg, int seg
 // HBM gather of the cache hits of rows [first, last) on stream `st`, for all n pipes in one launch.
 static int launch_hits(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg, int seg_last) {
   const int64_t n_max = s->node_cap[seg_last];
-  if (s->cache_kind == LMI_CACHE_INT8) {
-    for (int k = 0; k < n; ++k) LMI_TRY(launch_hits_int8(s, *pp[k], st, seg, seg_last));
-    return LMI_OK;
-  }
   MoveArgs m{};
   m.g.n = n;
   for (int k = 0; k < n; ++k) {
@@ -507,6 +506,7 @@ static int launch_hits(Server *s, Pipe *const *pp, int n, hipStream_t st, int se
     r.src_index = p.cache_index;
     r.dst = (uint8_t *)p.features;
   }
+  if (s->cache_kind == LMI_CACHE_INT8) return launch_hits_int8(s, m.g, st, seg_last);
   m.src = s->cache_data;
   m.src_row_bytes = m.dst_row_bytes = m.row_bytes = s->row_bytes;
   m.n_max = n_max;
