@@ -158,6 +158,12 @@ static void launch_move_v(hipStream_t st, const MoveArgs &a, int grid, bool nt, 
   }
 }
 
+// Grid of an HBM gather whose worst case needs `want` blocks: a sixteenth of that, between 8
+// and 64 blocks per CU.
+static int64_t auto_gather_blocks(const Server *s, int64_t want) {
+  return std::min<int64_t>(std::max<int64_t>(want / 16, (int64_t)s->n_cu * 8), (int64_t)s->n_cu * 64);
+}
+
 // Picks the widest vector that divides the row and all base addresses, and a
 // power-of-two lane group that covers one row when possible.
 static int launch_move_rows(Server *s, hipStream_t st, const MoveArgs &a, bool nt) {
@@ -177,7 +183,12 @@ static int launch_move_rows(Server *s, hipStream_t st, const MoveArgs &a, bool n
   const int unroll = a.unroll > 0 ? a.unroll : s->gather_unroll;
   const int64_t groups_per_block = 256 / lpr;
   int64_t want = ceil_div(a.n_max, groups_per_block * (unroll > 0 ? unroll : 1));
-  int64_t cap = a.max_blocks > 0 ? a.max_blocks : s->gather_blocks > 0 ? s->gather_blocks : (int64_t)s->n_cu * 8;
+  // Many small blocks rather than one resident wave of them: blocks that run beside host-link reads
+  // are slowed unevenly, and the dispatcher evens that out (paper100m-shaped, 4 batches per launch:
+  // 8 blocks per CU and pipe 62 % of HBM peak, 32 66 %, 64 67 %, 128 66 %, 256 57 %).  A batch holds
+  // about a tenth of its worst-case rows, and blocks without rows are not free (products-shaped:
+  // 40 % of peak on 2048 blocks per pipe, 36 % on 16384), hence the sixteenth.
+  int64_t cap = a.max_blocks > 0 ? a.max_blocks : s->gather_blocks > 0 ? s->gather_blocks : auto_gather_blocks(s, want);
   const int grid = (int)std::max<int64_t>(1, std::min(want, cap));
   if (vec == 16) launch_move_v<u32x4>(st, a, grid, nt, unroll, lpr);
   else if (vec == 8) launch_move_v<u32x2>(st, a, grid, nt, unroll, lpr);
@@ -460,7 +471,9 @@ int pipe_join(Pipe &p, hipStream_t st) {
 static int launch_hits_int8(Server *s, const MoveGroup &g, hipStream_t st, int seg_last) {
   const int64_t n_max = s->node_cap[seg_last];
   const int dim = s->cfg.feat_dim;
-  const int grid = g.n * (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(n_max, 4), (int64_t)s->n_cu * 8));
+  const int64_t want = ceil_div(n_max, 4);
+  const int64_t cap = s->gather_blocks > 0 ? s->gather_blocks : auto_gather_blocks(s, want);
+  const int grid = g.n * (int)std::max<int64_t>(1, std::min<int64_t>(want, cap));
   const int8_t *q = (const int8_t *)s->cache_data;
   unsigned long long *rc = s->prof_on ? s->d_prof_rows : nullptr;
   hipEvent_t e0, e1;

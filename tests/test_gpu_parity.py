@@ -216,6 +216,8 @@ def test_groups_of_batches_share_their_launches(lmi, oracle, group, fanout, cach
     try:
         if group == 3:
             srv.tune("protect_hits", 1)   # HBM gathers held back until earlier host-link gathers have drained
+        if group == 4:
+            srv.tune("group_miss", 0)     # one host-link gather launch per batch instead of one per group
         srv.load_graph(indptr, indices)
         srv.attach_features(feats)
         srv.load_idset(lmi.MODE_TRAIN, train)
