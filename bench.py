@@ -263,13 +263,9 @@ def main():
     srv, info = build_workload(lmi, w, args.seed, args.pipes, args.host_gb,
                                {"hash": 0, "direct": 1, "rank": 2}[args.table], args.policy)
     tunes = dict(kv.split("=") for kv in args.tune)
-    if args.group > 1:
-        # with several batches per launch the sampling phase is short enough that the host link sets
-        # the pace: a few more host-link blocks than the library's default of 32, shared by the group's
-        # batches (measured on paper100m-shaped, groups of 4 on 8 pipes: 28 -> 7.0 k batches/s with the
-        # HBM gather at 59 % of peak, the side stream never idle; 32 -> 7.3 k at 62 %; 36 -> 7.1 k at
-        # 62 %; 40 -> 6.8 k at 62 %; 48 -> 6.4 k at 64 %)
-        tunes.setdefault("miss_blocks", "36")
+    # host-link gather grid (miss_blocks, library default 32), measured on paper100m-shaped in groups
+    # of 4 on 8 pipes: 24 -> 6.6 k batches/s, 28 -> 7.2 k, 32 -> 7.5 k, 36 -> 7.3 k, 40 -> 7.0 k,
+    # 48 -> 6.5 k; the HBM gather stays at 66-68 % of peak throughout
     for k, v in tunes.items():
         srv.tune(k, int(v))
     steps_per_epoch = -(-info["n_train"] // w["batch"])
