@@ -346,7 +346,7 @@ __device__ __forceinline__ int32_t static_find(int table_kind, const HashSlot *s
 // rows directly and skips the misses.  List order is arbitrary; it only
 // schedules the host-link gather.
 constexpr int kLookupBlock = 1024;
-struct LookupGroup {  // one pipe per grid row, as in the sampling kernels
+struct LookupGroup {  // blocks interleave over the pipes, as in the sampling kernels
   LookupArgs p[LMI_MAX_PIPES];
   int n;
 };
@@ -555,10 +555,12 @@ static int launch_misses(Server *s, Pipe *const *pp, int n, hipStream_t st, int 
   return launch_move_rows(s, st, m, s->gather_nt != 0);
 }
 
-// Gathers the rows [first, last) of a segment into the pipe's feature buffer:
-// cache hits from HBM, misses over the host link.  Host-link reads in flight beside
-// the HBM gather cut its bandwidth by more than half, so the two never run
-// concurrently.  Schedules (tuning key "split_miss"):
+// Gathers the rows [first, last) of a segment into each pipe's feature buffer:
+// cache hits from HBM, misses over the host link.  A wide host-link gather beside
+// the HBM gather cuts its bandwidth by more than half, so the misses of one batch
+// never share a stream with its hits, and run on a small grid (miss_blocks).  With
+// several pipes, the hits of all are one launch and so are the misses (group_miss).
+// Schedules (tuning key "split_miss"):
 //   0  both on the caller's stream, one after the other;
 //   1  hits on the caller's stream, misses after them on the server's side stream,
 //      where they overlap the next batch's sampling;

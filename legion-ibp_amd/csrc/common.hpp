@@ -170,15 +170,15 @@ struct Server {
   // tuning
   int gather_lpr = 0;     // lanes per row (0 = auto)
   int gather_vec = 0;     // bytes per lane access (0 = widest that fits: 16)
-  int gather_unroll = 1;  // rows in flight per lane (1 measured best: 62.5 % of HBM peak vs 60 % at 4)
-  int gather_blocks = 0;  // 0 = auto
+  int gather_unroll = 1;  // rows in flight per lane (1 measured best, a few percent ahead of 4)
+  int gather_blocks = 0;  // blocks per pipe; 0 = auto (auto_gather_blocks)
   int gather_nt = 1;      // non-temporal output stores
   int64_t fuse_small_max = 32768;  // hops of at most this many nodes use the small tile of hop_tile_nodes
   int64_t table_epochs = int64_t(1) << 30;  // batches a dedup table serves between wipes, less one (also
                                             // bounded by the key bits the node ids leave free)
   int fuse_count = 1;     // 1: row counts, their scan and the sampling of a hop share one launch
   int lds_dedup = 0;      // 1: hop_sample stages its probes through an LDS hash table
-  int split_miss = 1;     // gather schedule, see launch_gather_seg
+  int split_miss = 1;     // gather schedule, see launch_gather_group
   int use_graph = 0;      // 1: lmi_run_once replays a captured HIP graph of the sampling kernels (measured
                           // 2-3 % slower than plain launches here: the host enqueues a batch in 85 us,
                           // well inside its 205 us of device time, and a graph's end costs 9 us)
@@ -219,7 +219,7 @@ int graph_update_begin(Server *s, Pipe &p, const BatchParams &bp);
 // kernel of the batch -- the next hop's first kernel or the lookup -- which carries it in
 // extra blocks; otherwise a kernel of its own finishes the hop.
 // The launchers below take n pipes that are in step (same stage of their batches) and serve
-// them with the same launches, one grid row per pipe.
+// them with the same launches, their blocks interleaved over blockIdx.x (LMI_GRID_ROW).
 int launch_hop(Server *s, Pipe *const *pp, int n, hipStream_t st, int hop, bool stage_seeds, bool defer_fill);
 int launch_fill(Server *s, Pipe *const *pp, int n, hipStream_t st);  // finishes a hop left pending, if any
 struct FillArgs;

@@ -51,9 +51,9 @@ struct HopArgs {
   FillArgs fill;    // the previous hop's last step, carried by hop_count_sample (hop -1: none)
 };
 
-// Several mini-batches (pipes) can share every launch of the sampling phase: grid row y
-// works on pipe y.  The kernels are latency-bound, so a second batch in the same launch
-// costs far less than a second launch.
+// Several mini-batches (pipes) can share every launch of the sampling phase: block b
+// works on pipe b mod n (LMI_GRID_ROW).  The kernels are latency-bound, so a second batch
+// in the same launch costs far less than a second launch.
 constexpr int kMaxGroup = LMI_MAX_PIPES;
 struct HopGroup {
   HopArgs p[kMaxGroup];
@@ -136,7 +136,7 @@ static __global__ __launch_bounds__(256) void batch_generate_kernel(int64_t n_no
 template <int ITEMS>
 static __global__ __launch_bounds__(kScanBlock) void hop_count_scan_kernel(HopGroup g) {
   LMI_GRID_ROW(g.n);
-  const HopArgs &a = g.p[row];  // one pipe (mini-batch) per grid row
+  const HopArgs &a = g.p[row];  // this block's pipe (mini-batch)
   constexpr int TILE = kScanBlock * ITEMS;
   __shared__ int lds[kScanBlock / kWave + 1];
   __shared__ int s_prefix;
@@ -220,7 +220,7 @@ static __global__ __launch_bounds__(kScanBlock) void hop_count_scan_kernel(HopGr
 template <int G>
 static __global__ __launch_bounds__(256) void hop_sample_kernel(HopGroup g) {
   LMI_GRID_ROW(g.n);
-  const HopArgs &a = g.p[row];  // one pipe (mini-batch) per grid row
+  const HopArgs &a = g.p[row];  // this block's pipe (mini-batch)
   const DevState *st = a.st;
   const int64_t flat = (int64_t)bx * blockDim.x + threadIdx.x;
   scan_chain_reset(a.chain_edges, a.max_tiles, flat, (int64_t)gx * blockDim.x);
@@ -272,7 +272,7 @@ static __global__ __launch_bounds__(256) void hop_sample_kernel(HopGroup g) {
 template <int G>
 static __global__ __launch_bounds__(256) void hop_sample_lds_kernel(HopGroup g) {
   LMI_GRID_ROW(g.n);
-  const HopArgs &a = g.p[row];  // one pipe (mini-batch) per grid row
+  const HopArgs &a = g.p[row];  // this block's pipe (mini-batch)
   constexpr int TAB = 512;
   __shared__ int32_t lds_key[TAB];
   __shared__ int32_t lds_min[TAB];
@@ -357,7 +357,7 @@ static __global__ __launch_bounds__(256) void hop_sample_lds_kernel(HopGroup g) 
 template <int G, int NPB>
 static __global__ __launch_bounds__(256) void hop_count_sample_kernel(HopGroup g) {
   LMI_GRID_ROW(g.n);
-  const HopArgs &a = g.p[row];  // one pipe (mini-batch) per grid row
+  const HopArgs &a = g.p[row];  // this block's pipe (mini-batch)
   static_assert(NPB <= kWave && NPB >= 256 / G, "tile = one wavefront of nodes at most, one pass at least");
   __shared__ int32_t s_id[NPB];
   __shared__ int64_t s_beg[NPB], s_deg[NPB];
@@ -475,7 +475,7 @@ static __global__ __launch_bounds__(256) void hop_count_sample_kernel(HopGroup g
 template <int ITEMS>
 static __global__ __launch_bounds__(kScanBlock) void hop_flag_scan_kernel(HopGroup g) {
   LMI_GRID_ROW(g.n);
-  const HopArgs &a = g.p[row];  // one pipe (mini-batch) per grid row
+  const HopArgs &a = g.p[row];  // this block's pipe (mini-batch)
   constexpr int TILE = kScanBlock * ITEMS;
   __shared__ int lds[kScanBlock / kWave + 1];
   __shared__ int s_prefix;
