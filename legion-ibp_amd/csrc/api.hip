@@ -803,6 +803,7 @@ int lmi_tune(lmi_server *h, const char *key, int64_t value) {
   else if (!strcmp(key, "fuse_count")) s->fuse_count = (int)value;
   else if (!strcmp(key, "protect_hits")) s->protect_hits = (int)value;
   else if (!strcmp(key, "group_miss")) s->group_miss = (int)value;
+  else if (!strcmp(key, "lru_early_miss")) s->lru_early_miss = (int)value;
   else if (!strcmp(key, "table_epochs")) {
     s->table_epochs = std::max<int64_t>(0, value);
     for (auto &p : s->pipes) p.table_dirty = true;

@@ -374,9 +374,20 @@ static __global__ __launch_bounds__(kLookupBlock) void lookup_kernel(LookupGroup
       int slot = -1;
       if (id >= 0 && id < a.n_nodes) {
         if (a.kind == LMI_CACHE_LRU) {
-          const int64_t base = ((int64_t)id % a.lru_sets) * a.lru_ways;
-          for (int w = 0; w < a.lru_ways; ++w)
-            if (a.lru_keys[base + w] == id) slot = (int)(base + w);
+          // sets * ways < 2^31, so 32-bit arithmetic addresses every way
+          const int base = (int)((uint32_t)id % (uint32_t)a.lru_sets) * a.lru_ways;
+          if ((a.lru_ways & 3) == 0) {  // a set's keys start on a 16-byte boundary: four ways per load
+            for (int w = 0; w < a.lru_ways; w += 4) {
+              const int4 k = *reinterpret_cast<const int4 *>(a.lru_keys + base + w);
+              if (k.x == id) slot = base + w;
+              if (k.y == id) slot = base + w + 1;
+              if (k.z == id) slot = base + w + 2;
+              if (k.w == id) slot = base + w + 3;
+            }
+          } else {
+            for (int w = 0; w < a.lru_ways; ++w)
+              if (a.lru_keys[base + w] == id) slot = base + w;
+          }
           if (slot >= 0) a.lru_use[slot] = a.st->lru_tick;
           // a repeated seed keeps both rows, but the id is offered for insertion once, by its first row
           const bool repeat = i < a.st->n_seeds &&
@@ -595,8 +606,16 @@ int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int s
         s->side_busy = false;
       }
     }
-    LMI_TRY(launch_hits(s, pp, n, st, seg, seg_last));  // one launch for the group
+    // LRU batches are host-link-bound (a fifth of their rows miss): their host-link gather starts
+    // beside the HBM gather instead of behind it.  The insertion that follows it on the side stream
+    // only overwrites ways this batch's lookup did not touch, so the hits never read a row it writes.
+    const bool early = lru_lists > 0 && s->lru_early_miss;
     fork = nullptr;
+    if (early) {
+      fork = pp[0]->fork;
+      LMI_HIP(hipEventRecord(fork, st));
+    }
+    LMI_TRY(launch_hits(s, pp, n, st, seg, seg_last));  // one launch for the group
   }
   if (!fork) {  // one fork for the whole group
     fork = pp[0]->fork;
@@ -648,9 +667,10 @@ static __global__ __launch_bounds__(256) void lru_bid_kernel(LruArgs a) {
   for (int l = 0; l < a.n_lists; ++l) {
     const int n = a.st->n_miss[l];
     for (int j = blockIdx.x * blockDim.x + threadIdx.x; j < n; j += gridDim.x * blockDim.x) {
-      const int i = a.miss_list[l][j].x;
+      const int2 pr = a.miss_list[l][j];  // (row, id)
+      const int i = pr.x;
       if (a.fill[i] != -1) continue;  // the later row of a repeated seed
-      atomicMin(&a.claim_cur[(int64_t)a.ids[i] % a.sets], i);
+      atomicMin(&a.claim_cur[(uint32_t)pr.y % (uint32_t)a.sets], i);
     }
   }
 }
@@ -659,17 +679,28 @@ static __global__ __launch_bounds__(256) void lru_round_kernel(LruArgs a) {
   for (int l = 0; l < a.n_lists; ++l) {
     const int n = a.st->n_miss[l];
     for (int j = blockIdx.x * blockDim.x + threadIdx.x; j < n; j += gridDim.x * blockDim.x) {
-      const int i = a.miss_list[l][j].x;
+      const int2 pr = a.miss_list[l][j];  // (row, id)
+      const int i = pr.x;
       if (a.fill[i] != -1) continue;  // placed (>= 0) or refused (-2) earlier
-      const int32_t id = a.ids[i];
-      const int64_t set = (int64_t)id % a.sets;
+      const int32_t id = pr.y;
+      const int64_t set = (uint32_t)id % (uint32_t)a.sets;  // sets < 2^31
       if (a.claim_cur[set] == i) {
         const int64_t base = set * a.ways;
         int best = -1, best_use = kIntMax;
         const int tick = a.st->lru_tick;
-        for (int w = 0; w < a.ways; ++w) {
-          const int u = a.use[base + w];
-          if (u < tick && u < best_use) best = w, best_use = u;
+        if ((a.ways & 3) == 0) {  // four ways per load, same order of preference (lowest way wins a tie)
+          for (int w = 0; w < a.ways; w += 4) {
+            const int4 u = *reinterpret_cast<const int4 *>(a.use + base + w);
+            if (u.x < tick && u.x < best_use) best = w, best_use = u.x;
+            if (u.y < tick && u.y < best_use) best = w + 1, best_use = u.y;
+            if (u.z < tick && u.z < best_use) best = w + 2, best_use = u.z;
+            if (u.w < tick && u.w < best_use) best = w + 3, best_use = u.w;
+          }
+        } else {
+          for (int w = 0; w < a.ways; ++w) {
+            const int u = a.use[base + w];
+            if (u < tick && u < best_use) best = w, best_use = u;
+          }
         }
         if (best >= 0) {
           a.keys[base + best] = id;

@@ -161,6 +161,7 @@ struct Server {
   hipEvent_t side_idle = nullptr;  // recorded behind the last host-link gather issued on the side stream
   bool side_busy = false;
   int protect_hits = 0;            // 1: HBM gathers wait until earlier host-link gathers have drained
+  int lru_early_miss = 1;          // 1: with the LRU cache the host-link gather starts beside the HBM gather
   int group_miss = 1;              // 1: the host-link gathers of a group of batches are one launch
   hipEvent_t lru_ready = nullptr;  // recorded behind every LRU insertion: the next lookup waits for it
   bool lru_pending = false;        // an insertion may still be running
