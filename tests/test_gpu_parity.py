@@ -747,3 +747,61 @@ def test_rebuilding_cache_or_graph_after_graph_capture(lmi, oracle):
     finally:
         srv.close()
         feats.free()
+
+
+@pytest.mark.parametrize("cache", ["static", "int8", "lru"])
+@pytest.mark.parametrize("level,every", [(1, 1), (2, 1), (2, 3)])
+def test_profiled_batches_come_out_the_same_and_count_their_rows(lmi, oracle, level, every, cache):
+    """Profiling changes how kernels are launched (event-carrying launches, marker events between
+    phases, device row counters): the batches must not change, and the counters must add up to the
+    rows of the batches that were profiled (one in `every`)."""
+    rng = np.random.default_rng(level * 7 + every)
+    n_nodes, batch, dim, fanout = 4000, 120, 16, [8, 5]
+    indptr, indices = random_graph(rng, n_nodes, 12, hubs=4, hub_deg=400)
+    feats = make_features(lmi, rng, n_nodes, dim)
+    train = rng.permutation(n_nodes)[:3600].astype(np.int32)
+    group = 1 if cache == "lru" else 3
+    srv = lmi.Server(batch, fanout, dim, pipes=group, seed=4)
+    stream = lmi.stream_create()
+    try:
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        srv.load_idset(lmi.MODE_TRAIN, train)
+        if cache == "static":
+            srv.build_static_cache(1200, lmi.TABLE_RANK)
+        elif cache == "int8":
+            srv.build_int8_cache(1200, lmi.TABLE_RANK)
+        else:
+            srv.build_lru_cache(96, 4)
+        srv.tune("profile_every", every)
+        srv.profile_enable(level)
+        rows_profiled = hits_profiled = 0
+        n_calls = 6
+        for call in range(n_calls):
+            counters = [call * group + k for k in range(group)]
+            if group == 1:
+                srv.run_once(batch_counter=counters[0], pipe=0, stream=stream)
+            else:
+                srv.run_group(list(range(group)), counters, stream=stream)
+            for k, c in enumerate(counters):
+                g = srv.fetch(pipe=k, stream=stream)
+                o = oracle.sample_batch(indptr, indices, train[c * batch:(c + 1) * batch], fanout, 4 + c)
+                assert_batch_equal(g, o)
+                if cache != "int8":
+                    assert g.features.tobytes() == feats.array[o.ids].tobytes()
+                if call % every == 0:   # the first call after profile_enable is profiled, then one in `every`
+                    rows_profiled += len(o.ids)
+                    hits_profiled += int((g.cache_index >= 0).sum())
+        prof = srv.profile_read()
+        assert prof.gather_hit_rows + prof.gather_miss_rows == rows_profiled
+        assert prof.gather_hit_rows == hits_profiled
+        calls_profiled = len(range(0, n_calls, every))
+        assert prof.gather_hit_launches == calls_profiled          # one HBM gather launch per call
+        assert prof.gather_miss_launches == calls_profiled         # and one host-link gather launch
+        assert prof.gather_hit_ms > 0 and prof.gather_miss_ms > 0
+        if level == 1:
+            assert prof.sample_launches == calls_profiled and prof.sample_ms > 0
+        srv.profile_enable(0)
+    finally:
+        srv.close()
+        feats.free()
