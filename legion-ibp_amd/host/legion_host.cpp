@@ -174,8 +174,9 @@ class GPURunner : public Runner {
     } else {
       run_table(params, local, mode, false);
     }
-    LMI_MUST(lmi_batch_wait((lmi_server *)params->env, pipe_, stream_));
-    if (ipc && ipc->HandoffEnabled()) {
+    const bool handoff = ipc && ipc->HandoffEnabled();
+    if (handoff || !params->defer_join) LMI_MUST(lmi_batch_wait((lmi_server *)params->env, pipe_, stream_));
+    if (handoff) {
       LMI_MUST(lmi_stream_sync(stream_));  // the batch is complete before the trainer is told
       ipc->IPCPost(device_, pipe_);
     }
@@ -337,6 +338,9 @@ class GPUServer : public Server {
     const int32_t max_step = ipc_->GetMaxStep();
     const auto t0 = std::chrono::steady_clock::now();
     int64_t batches = 0;
+    // with nobody reading the batches as they come (no sink, no trainer), a batch's host-link
+    // gather may run on beside the next batch's sampling
+    params_.defer_join = !sink_ && !ipc_->HandoffEnabled();
     for (int32_t batch_id = 0; batch_id < max_step; ++batch_id) {
       params_.global_batch_id = batch_id;
       runner_->RunOnce(&params_);
@@ -347,6 +351,7 @@ class GPUServer : public Server {
       }
       ++batches;
     }
+    for (int pipe = 0; pipe < LEGION_INTERBATCH_CON; ++pipe) LMI_MUST(lmi_batch_wait(h_, pipe, runner_->Stream()));
     LMI_MUST(lmi_stream_sync(runner_->Stream()));
     const double sec = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
     std::printf("batches: %lld  time per sample: %.1f us  (%.1f batches/s)\n", (long long)batches,

@@ -54,6 +54,9 @@ struct RunnerParams {
                         // global_batch_id counts over the whole schedule and the mode and the
                         // batch's place in its id set come from it; when null, global_batch_id
                         // is the place in id set `mode`.
+  bool defer_join = false;  // true: RunOnce does not order the stream behind the batch's host-link
+                            // gather (nobody reads the batch yet); the pipe's next batch does, so the
+                            // gather overlaps the sampling of the batch in between
 };
 
 // Called once per finished batch with the pipe's device buffers; the stream has
