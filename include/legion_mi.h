@@ -32,7 +32,8 @@ extern "C" {
 #define LMI_ABI_VERSION 1
 #define LMI_MAX_HOPS    3   /* the 16-int headers hold 3 hops (INTRABATCH_CON, include/system_config.cuh:47-57) */
 #define LMI_MAX_FANOUT  64  /* one wavefront lane per slot; the reference asserts <= 32 (operator_impl.cu:504) */
-#define LMI_MAX_PIPES   8   /* output buffer sets; the reference uses INTERBATCH_CON = 2 */
+#define LMI_MAX_PIPES   16  /* output buffer sets; the reference uses INTERBATCH_CON = 2 */
+#define LMI_MAX_GROUP   8   /* mini-batches one lmi_run_group call can issue together */
 
 enum {
   LMI_OK = 0,
@@ -202,7 +203,7 @@ int lmi_op_io_complete(lmi_server *s, int pipe, void *stream);
 int lmi_run_once(lmi_server *s, int pipe, void *stream, const int32_t *seeds, int32_t n,
                  int seeds_location, int32_t batch_counter, int mode, uint64_t rng_seed);
 
-/* n_batches mini-batches at once, batch k into pipe pipes[k] (distinct pipes): the same as
+/* n_batches <= LMI_MAX_GROUP mini-batches at once, batch k into pipe pipes[k] (distinct pipes): the same as
  * n_batches calls of lmi_run_once, but every launch of the sampling phase serves all of them
  * (those kernels are latency-bound, so the batches after the first cost little).  seeds,
  * n_seeds and rng_seeds may be NULL (slices batch_counters[k] of id set `mode`, default RNG

@@ -13,7 +13,7 @@ import numpy as np
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "liblegion_mi.so")
 
-MAX_HOPS, MAX_FANOUT, MAX_PIPES = 3, 64, 4
+MAX_HOPS, MAX_FANOUT, MAX_PIPES, MAX_GROUP = 3, 64, 16, 8
 F32, F16 = 0, 1
 LOC_HOST, LOC_DEVICE = 0, 1
 MODE_TRAIN, MODE_VALID, MODE_TEST = 0, 1, 2

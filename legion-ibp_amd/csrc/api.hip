@@ -670,12 +670,12 @@ int lmi_run_group(lmi_server *h, int n_batches, const int32_t *pipes, void *stre
                   const uint64_t *rng_seeds) {
   Server *s = reinterpret_cast<Server *>(h);
   if (!s || !pipes || !batch_counters) LMI_FAIL(LMI_ERR_ARG, "null argument");
-  if (n_batches < 1 || n_batches > LMI_MAX_PIPES) LMI_FAIL(LMI_ERR_ARG, "a group holds 1..%d batches", LMI_MAX_PIPES);
+  if (n_batches < 1 || n_batches > LMI_MAX_GROUP) LMI_FAIL(LMI_ERR_ARG, "a group holds 1..%d batches", LMI_MAX_GROUP);
   if (!s->feat) LMI_FAIL(LMI_ERR_STATE, "no features attached");
   if (s->cache_kind == LMI_CACHE_LRU && n_batches > 1)
     LMI_FAIL(LMI_ERR_STATE, "the LRU cache takes one batch at a time (its state is batch-synchronous)");
-  Pipe *pp[LMI_MAX_PIPES];
-  BatchParams bps[LMI_MAX_PIPES];
+  Pipe *pp[LMI_MAX_GROUP];
+  BatchParams bps[LMI_MAX_GROUP];
   hipStream_t st = (hipStream_t)stream;
   for (int k = 0; k < n_batches; ++k) {
     LMI_TRY(check_pipe(s, pipes[k]));

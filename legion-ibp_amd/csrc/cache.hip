@@ -40,7 +40,7 @@ struct MoveRow {
   uint8_t *dst;
 };
 struct MoveGroup {
-  MoveRow p[LMI_MAX_PIPES];
+  MoveRow p[LMI_MAX_GROUP];
   int n;
 };
 
@@ -168,7 +168,7 @@ static int64_t auto_gather_blocks(const Server *s, int64_t want) {
 // power-of-two lane group that covers one row when possible.
 static int launch_move_rows(Server *s, hipStream_t st, const MoveArgs &a, bool nt) {
   if (a.n_max <= 0 || a.row_bytes <= 0) return LMI_OK;
-  if (a.g.n < 1 || a.g.n > LMI_MAX_PIPES) LMI_FAIL(LMI_ERR_ARG, "a row move serves 1..LMI_MAX_PIPES pipes");
+  if (a.g.n < 1 || a.g.n > LMI_MAX_GROUP) LMI_FAIL(LMI_ERR_ARG, "a row move serves 1..LMI_MAX_GROUP pipes");
   uintptr_t align = (uintptr_t)a.src | (uintptr_t)a.src_row_bytes | (uintptr_t)a.dst_row_bytes | (uintptr_t)a.row_bytes;
   for (int k = 0; k < a.g.n; ++k) align |= (uintptr_t)a.g.p[k].dst;
   int vec = (align % 16 == 0) ? 16 : (align % 8 == 0) ? 8 : 4;
@@ -347,7 +347,7 @@ __device__ __forceinline__ int32_t static_find(int table_kind, const HashSlot *s
 // schedules the host-link gather.
 constexpr int kLookupBlock = 1024;
 struct LookupGroup {  // blocks interleave over the pipes, as in the sampling kernels
-  LookupArgs p[LMI_MAX_PIPES];
+  LookupArgs p[LMI_MAX_GROUP];
   int n;
 };
 

@@ -54,7 +54,7 @@ struct HopArgs {
 // Several mini-batches (pipes) can share every launch of the sampling phase: block b
 // works on pipe b mod n (LMI_GRID_ROW).  The kernels are latency-bound, so a second batch
 // in the same launch costs far less than a second launch.
-constexpr int kMaxGroup = LMI_MAX_PIPES;
+constexpr int kMaxGroup = LMI_MAX_GROUP;
 struct HopGroup {
   HopArgs p[kMaxGroup];
   int n;
