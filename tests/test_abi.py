@@ -61,3 +61,12 @@ def test_missing_library_fails_loudly(lmi, monkeypatch):
     monkeypatch.setattr(lmi, "LIB_PATH", "/nonexistent/liblegion_mi.so")
     with pytest.raises(ImportError):
         lmi.lib()
+
+
+def test_bench_refuses_more_than_one_gpu():
+    import subprocess
+    import sys
+    r = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True,
+                       timeout=120)
+    assert r.returncode != 0
+    assert "ONE GPU" in r.stderr and r.stdout.strip() == ""
