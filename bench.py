@@ -362,6 +362,9 @@ def main():
                      peak=HOST_LINK_PEAK_GBS, unit="GB/s", rows_per_launch=round(miss_rows, 1),
                      batches_per_launch=miss_batches,
                      avg_launch_ms=round(miss_ms, 4))
+    # the sampling kernels are bound by cold random reads: what the device sustains on the neighbour array
+    rr_reads = 1 << 24
+    rr_ms = lmi.bench_random_read(info["d_indices"], info["n_edges"] * 4, rr_reads)
     total_rows = prof.gather_hit_rows + prof.gather_miss_rows
     profiled_batches = int(max(prof.gather_hit_launches * hit_batches, prof.gather_miss_launches * miss_batches))
     out = {
@@ -389,6 +392,8 @@ def main():
                                "gather_hit": round(hit_ms / hit_batches, 4),
                                "gather_miss_side_stream": round(miss_ms / miss_batches, 4)},
         "roofline": roofline, "host_link": host_link,
+        "random_read": {"measured_g_reads_per_s": round(rr_reads / (rr_ms * 1e-3) / 1e9, 1),
+                        "what": "independent 4-byte reads at random places of the neighbour array"},
     }
     if args.cpu_seconds > 0:
         cb, ok = cpu_baseline(lmi, srv, w, info, args.seed, args.cpu_seconds)

@@ -244,6 +244,10 @@ int lmi_bench_copy(size_t bytes, int repeats, double *ms_per_copy);
 /* Streaming zero-copy read of `bytes` bytes of pinned host memory (from lmi_host_alloc) into
  * HBM, repeated; returns mean ms per pass (the measured host-link ceiling). */
 int lmi_bench_host_read(const void *host_ptr, size_t bytes, int repeats, double *ms_per_pass);
+/* n_reads independent 4-byte reads at pseudo-random places of a device array of `bytes` bytes
+ * (e.g. the neighbour array), repeated; returns mean ms per pass: the rate of cold random reads
+ * this device sustains, which is what bounds the sampling kernels. */
+int lmi_bench_random_read(const void *device_ptr, size_t bytes, int64_t n_reads, int repeats, double *ms_per_pass);
 
 /* ---- synthetic inputs (stand-in for the reference's dataset tooling) ---- */
 /* Power-law graph generated in HBM: degree(v) by inverse-CDF lookup of a Philox

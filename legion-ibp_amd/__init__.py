@@ -32,7 +32,7 @@ ABI_SYMBOLS = [
     "lmi_cache_info_get", "lmi_cache_dump", "lmi_op_batch_generate", "lmi_op_random_sample",
     "lmi_op_cache_lookup", "lmi_op_io_submit", "lmi_op_io_complete", "lmi_run_once",
     "lmi_run_group", "lmi_batch_wait", "lmi_batch_view_get", "lmi_batch_counters", "lmi_steps_per_epoch", "lmi_profile_enable",
-    "lmi_profile_read", "lmi_tune", "lmi_bench_copy", "lmi_bench_host_read", "lmi_synth_graph", "lmi_synth_trainset",
+    "lmi_profile_read", "lmi_tune", "lmi_bench_copy", "lmi_bench_host_read", "lmi_bench_random_read", "lmi_synth_graph", "lmi_synth_trainset",
     "lmi_synth_features",
 ]
 
@@ -127,6 +127,7 @@ def lib():
         L.lmi_tune.argtypes = [C.c_void_p, C.c_char_p, C.c_int64]
         L.lmi_bench_copy.argtypes = [C.c_size_t, C.c_int, C.POINTER(C.c_double)]
         L.lmi_bench_host_read.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.POINTER(C.c_double)]
+        L.lmi_bench_random_read.argtypes = [C.c_void_p, C.c_size_t, C.c_int64, C.c_int, C.POINTER(C.c_double)]
         L.lmi_synth_graph.argtypes = [C.c_uint64, C.c_void_p, C.c_int32, C.c_int64, C.c_int32,
                                       C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.POINTER(C.c_int64)]
         L.lmi_synth_trainset.argtypes = [C.c_uint64, C.c_int64, C.c_int32, C.c_void_p]
@@ -354,6 +355,13 @@ class Server:
 def bench_copy(nbytes, repeats=10):
     ms = C.c_double()
     check(lib().lmi_bench_copy(nbytes, repeats, C.byref(ms)))
+    return ms.value
+
+
+def bench_random_read(device_ptr, nbytes, n_reads=1 << 24, repeats=5):
+    """Mean ms of n_reads independent random 4-byte reads of a device array of nbytes bytes."""
+    ms = C.c_double()
+    check(lib().lmi_bench_random_read(device_ptr, int(nbytes), int(n_reads), repeats, C.byref(ms)))
     return ms.value
 
 

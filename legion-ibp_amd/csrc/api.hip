@@ -840,6 +840,47 @@ int lmi_bench_host_read(const void *host_ptr, size_t bytes, int repeats, double 
   return LMI_OK;
 }
 
+// Four independent reads per thread at places drawn by a 64-bit mixer; the sum goes nowhere
+// unless it hits one particular value, which keeps the loads alive.
+static __global__ __launch_bounds__(256) void random_read_kernel(const uint32_t *a, uint64_t n_words, int64_t n_reads,
+                                                                uint64_t salt, uint32_t *sink) {
+  const int64_t t = ((int64_t)blockIdx.x * blockDim.x + threadIdx.x) * 4;
+  if (t >= n_reads) return;
+  uint32_t v[4];
+#pragma unroll
+  for (int k = 0; k < 4; ++k) {
+    uint64_t x = (uint64_t)(t + k) + salt;
+    x ^= x >> 33; x *= 0xff51afd7ed558ccdULL; x ^= x >> 33; x *= 0xc4ceb9fe1a85ec53ULL; x ^= x >> 33;
+    v[k] = a[x % n_words];
+  }
+  const uint32_t acc = v[0] + v[1] + v[2] + v[3];
+  if (acc == 0x9E3779B1u) *sink = acc;
+}
+
+int lmi_bench_random_read(const void *device_ptr, size_t bytes, int64_t n_reads, int repeats, double *ms_per_pass) {
+  if (!device_ptr || !ms_per_pass || repeats < 1 || bytes < 4 || n_reads < 4) LMI_FAIL(LMI_ERR_ARG, "bad argument");
+  uint32_t *sink = nullptr;
+  LMI_HIP(hipMalloc(&sink, 4));
+  hipEvent_t e0, e1;
+  LMI_HIP(hipEventCreate(&e0));
+  LMI_HIP(hipEventCreate(&e1));
+  const int grid = (int)std::min<int64_t>(ceil_div(ceil_div(n_reads, 4), 256), 1 << 30);
+  const uint64_t n_words = bytes / 4;
+  hipLaunchKernelGGL(random_read_kernel, dim3(grid), dim3(256), 0, 0, (const uint32_t *)device_ptr, n_words, n_reads, 1ull, sink);
+  LMI_HIP(hipEventRecord(e0, 0));
+  for (int r = 0; r < repeats; ++r)
+    hipLaunchKernelGGL(random_read_kernel, dim3(grid), dim3(256), 0, 0, (const uint32_t *)device_ptr, n_words, n_reads,
+                       (uint64_t)(r + 2) * 0x9E3779B97F4A7C15ull, sink);
+  LMI_HIP(hipEventRecord(e1, 0));
+  LMI_HIP(hipEventSynchronize(e1));
+  float ms = 0;
+  LMI_HIP(hipEventElapsedTime(&ms, e0, e1));
+  *ms_per_pass = ms / repeats;
+  (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
+  (void)hipFree(sink);
+  return LMI_OK;
+}
+
 int lmi_bench_copy(size_t bytes, int repeats, double *ms_per_copy) {
   if (!ms_per_copy || repeats < 1 || bytes < 16) LMI_FAIL(LMI_ERR_ARG, "bad argument");
   void *a = nullptr, *b = nullptr;
