@@ -135,3 +135,71 @@ def test_int8_workload(lmi, oracle):
     finally:
         srv.close()
         info["feats"].free()
+
+
+def _mem_available_gb():
+    try:
+        for line in open("/proc/meminfo"):
+            if line.startswith("MemAvailable:"):
+                return int(line.split()[1]) / 1e6
+    except OSError:
+        pass
+    return 0.0
+
+
+def test_paper100m_at_full_size_in_groups_of_four(lmi, oracle):
+    """The benchmark's own configuration at its real size (111 M nodes, 1.6 B edges, 57 GB of rows in
+    pinned host memory, 38 GB cache), four batches per launch as bench.py issues them: bit-exact
+    against the oracle, plus the properties that hold at any size."""
+    if _mem_available_gb() < 90:
+        pytest.skip("needs about 75 GB of host memory for the feature table and a host copy of the graph")
+    import bench
+    w = dict(bench.WORKLOADS["paper100m"])
+    srv, info = bench.build_workload(lmi, w, 20260101, 8, 64.0)
+    stream = lmi.stream_create()
+    feats = info["feats"].array
+    try:
+        indptr = lmi.to_host(info["d_indptr"], info["n_nodes"] + 1, np.int64)
+        indices = lmi.to_host(info["d_indices"], info["n_edges"], np.int32)
+        deg = np.diff(indptr)
+        B, fanout = w["batch"], w["fanout"]
+        counters = [3, 4, 5, 6]
+        srv.run_group([0, 1, 2, 3], counters, stream=stream)
+        got = [srv.fetch(pipe=k, stream=stream) for k in range(4)]
+        # the same batch issued alone, later, on another pipe: a batch depends on nothing but its seeds and RNG seed
+        srv.run_once(None, batch_counter=counters[1], pipe=5, stream=stream)
+        alone = srv.fetch(pipe=5, stream=stream)
+        check_batch(alone, got[1])
+        assert alone.features.tobytes() == got[1].features.tobytes()
+        for k, g in enumerate(got):
+            seeds = info["train"][counters[k] * B:(counters[k] + 1) * B]
+            o = oracle.sample_batch(indptr, indices, seeds, fanout, 20260101 + counters[k])
+            check_batch(g, o)
+            assert g.features.tobytes() == feats[g.ids].tobytes()
+            # closed forms and invariants
+            assert np.array_equal(g.ids[:len(seeds)], seeds) and len(np.unique(g.ids)) == len(g.ids)
+            n_prev = len(seeds)
+            for h in range(g.hops):
+                e0, e1 = g.edge_off[h], g.edge_off[h] + g.n_edges[h]
+                src, dst = g.agg_src_ids[e0:e1], g.agg_dst_off[e0:e1]
+                assert g.n_edges[h] == int(np.minimum(deg[g.ids[:n_prev]], fanout[h]).sum())
+                assert np.array_equal(g.ids[g.agg_src_off[e0:e1]], src) and dst.max() < n_prev
+                # new nodes are numbered by first appearance in edge order
+                new = src[~np.isin(src, g.ids[:n_prev])]
+                _, first = np.unique(new, return_index=True)
+                assert np.array_equal(g.ids[n_prev:g.n_nodes[h + 1]], new[np.sort(first)])
+                # a node of at most `fanout` neighbours contributes its whole row, in CSR order
+                small = np.flatnonzero(deg[g.ids[:n_prev]] <= fanout[h])[:2000]
+                rows = g.blk_indptr[h]
+                for v in small:
+                    assert np.array_equal(src[rows[v]:rows[v + 1]], indices[indptr[g.ids[v]]:indptr[g.ids[v] + 1]])
+                # sampled edges exist in the graph (a sample of them), without repeats inside a row
+                for e in np.linspace(0, len(src) - 1, 3000).astype(np.int64):
+                    d = g.ids[dst[e]]
+                    assert src[e] in indices[indptr[d]:indptr[d + 1]]
+                n_prev = g.n_nodes[h + 1]
+            hit = g.cache_index >= 0
+            assert deg[g.ids][hit].min() >= deg[g.ids][~hit].max()
+    finally:
+        srv.close()
+        info["feats"].free()
