@@ -1,7 +1,7 @@
 """The five target configurations (Cora-, products-, paper100m-, paper100m-LRU- and
 MAG240M-shaped) as parity cases: the synthetic workload
-builder of bench.py (graph generated on the GPU) at full size where that is
-cheap (cora, products) and at a stated fraction of the node count otherwise,
+builder of bench.py (graph generated on the GPU) at full size (cora, products,
+paper100m in groups of four) or at a stated fraction of the node count,
 compared with the CPU oracle batch by batch."""
 import os
 import sys
