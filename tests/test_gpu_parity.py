@@ -805,3 +805,38 @@ def test_profiled_batches_come_out_the_same_and_count_their_rows(lmi, oracle, le
     finally:
         srv.close()
         feats.free()
+
+
+@pytest.mark.parametrize("fanout,batch,n_nodes,deg", [([25, 10], 64, 1_000_000, 40), ([64, 64], 16, 2_000_000, 72),
+                                                      ([8, 8, 8], 128, 600_000, 160)])
+def test_batches_that_nearly_fill_their_buffers(lmi, oracle, fanout, batch, n_nodes, deg):
+    """Every node has more neighbours than the fan-out and they are spread over a graph far larger
+    than a batch, so almost every sampled edge brings a new node: the batch comes within a few
+    percent of the worst case the buffers and the dedup table are sized for, with both pipes of a
+    group at that size."""
+    rng = np.random.default_rng(len(fanout) * 1000 + batch)
+    indptr = np.arange(n_nodes + 1, dtype=np.int64) * deg
+    indices = rng.integers(0, n_nodes, n_nodes * deg, dtype=np.int32)
+    dim = 4
+    feats = lmi.HostBuffer((n_nodes, dim), np.float32)
+    feats.array[...] = np.arange(n_nodes, dtype=np.float32)[:, None]
+    worst = batch
+    for f in fanout:
+        worst *= 1 + f
+    srv = lmi.Server(batch, fanout, dim, pipes=2, seed=11)
+    stream = lmi.stream_create()
+    try:
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        srv.build_static_cache(n_nodes // 3, lmi.TABLE_RANK)
+        seeds = [rng.choice(n_nodes, batch, replace=False).astype(np.int32) for _ in range(2)]
+        srv.run_group([0, 1], [0, 0], seeds=seeds, rng_seeds=[5, 6], stream=stream)
+        for k in range(2):
+            g = srv.fetch(pipe=k, stream=stream)
+            o = oracle.sample_batch(indptr, indices, seeds[k], fanout, 5 + k)
+            assert_batch_equal(g, o)
+            assert g.n_nodes[-1] > 0.9 * worst
+            assert g.features.tobytes() == feats.array[o.ids].tobytes()
+    finally:
+        srv.close()
+        feats.free()
