@@ -343,11 +343,26 @@ def main():
     achieved = hit_rows * hit_bytes / (hit_ms * 1e-3) / 1e9 if hit_ms > 0 else 0.0
     copy_ms = lmi.bench_copy(1 << 30, 10)
     copy_gbs = 2 * (1 << 30) / (copy_ms * 1e-3) / 1e9
+    def mover(host_link):
+        # the instantiation the library picks for this row size: widest lane access that divides the
+        # row, smallest power-of-two lane group (8..64) that covers it
+        vec = 16 if rb % 16 == 0 else 8 if rb % 8 == 0 else 4
+        narrower = int(tunes.get("gather_vector_bytes", 0))
+        if narrower == 4 or (narrower == 8 and vec == 16):
+            vec = narrower
+        lanes = int(tunes.get("gather_lanes_per_row", 0))
+        if lanes not in (1, 4, 8, 16, 32, 64):
+            lanes = 8
+            while lanes < rb // vec and lanes < 64:
+                lanes *= 2
+        unroll = int(tunes.get("miss_unroll", 1) if host_link else tunes.get("gather_unroll", 1))
+        return "move_rows_kernel<%s,%d,%d,true,%s>" % ({16: "u32x4", 8: "u32x2", 4: "u32"}[vec], lanes, unroll,
+                                                     "true" if host_link else "false")
     if info["cache_kind"] == "int8":
         hit_kernel = "gather_int8_kernel<%s,%d> (HBM gather of cache hits, dequantisation fused)" % (
             "__half" if w["dtype"] == "f16" else "float", 32 if w["dim"] // 16 <= 32 else 64)
     else:
-        hit_kernel = "move_rows_kernel<u32x4,32,1,true,false> (HBM gather of cache hits)"
+        hit_kernel = mover(False) + " (HBM gather of cache hits)"
     roofline = dict(bound="hbm", kernel=hit_kernel, achieved=round(achieved, 1),
                     peak=HBM_PEAK_GBS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBS, 4),
                     traffic=recorded_traffic(args.workload) if args.scale == 1.0 else None,
@@ -356,7 +371,7 @@ def main():
                     measured_copy_gbs=round(copy_gbs, 1))
     link_bytes = min(1 << 28, info["feats"].nbytes)
     link_ms = lmi.bench_host_read(info["feats"], link_bytes)
-    host_link = dict(bound="host-link", kernel="move_rows_kernel<u32x4,32,1,true,true> (host-link gather of misses)",
+    host_link = dict(bound="host-link", kernel=mover(True) + " (host-link gather of misses)",
                      measured_stream_read_gbs=round(link_bytes // 16 * 16 / (link_ms * 1e-3) / 1e9, 2),
                      achieved=round(miss_rows * rb / (miss_ms * 1e-3) / 1e9, 2) if miss_ms > 0 else 0.0,
                      peak=HOST_LINK_PEAK_GBS, unit="GB/s", rows_per_launch=round(miss_rows, 1),
