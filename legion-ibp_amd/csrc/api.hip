@@ -223,6 +223,7 @@ int lmi_server_create(const lmi_config *cfg, lmi_server **out) {
   if (rc == LMI_OK && hipMalloc(&s->d_scalar, 64) != hipSuccess) rc = LMI_ERR_HIP;
   if (rc == LMI_OK && hipStreamCreateWithFlags(&s->side, hipStreamNonBlocking) != hipSuccess) rc = LMI_ERR_HIP;
   if (rc == LMI_OK && hipEventCreateWithFlags(&s->lru_ready, hipEventDisableTiming) != hipSuccess) rc = LMI_ERR_HIP;
+  if (rc == LMI_OK && hipEventCreateWithFlags(&s->lru_copied, hipEventDisableTiming) != hipSuccess) rc = LMI_ERR_HIP;
   if (rc == LMI_OK && hipEventCreateWithFlags(&s->side_idle, hipEventDisableTiming) != hipSuccess) rc = LMI_ERR_HIP;
   if (rc == LMI_OK && (hipMalloc(&s->d_prof_rows, 16) != hipSuccess || hipMemset(s->d_prof_rows, 0, 16) != hipSuccess))
     rc = LMI_ERR_HIP;
@@ -256,6 +257,7 @@ int lmi_server_destroy(lmi_server *h) {
   if (s->hot) (void)hipFree(s->hot);
   if (s->side) (void)hipStreamDestroy(s->side);
   if (s->lru_ready) (void)hipEventDestroy(s->lru_ready);
+  if (s->lru_copied) (void)hipEventDestroy(s->lru_copied);
   if (s->side_idle) (void)hipEventDestroy(s->side_idle);
   delete s;
   return LMI_OK;

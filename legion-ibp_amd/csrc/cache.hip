@@ -518,6 +518,7 @@ static int launch_hits_int8(Server *s, const MoveGroup &g, hipStream_t st, int s
 
 // HBM gather of the cache hits of rows [first, last) on stream `st`, for all n pipes in one launch.
 static int launch_hits(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg, int seg_last) {
+  LMI_TRY(lru_wait_copied(s, st));
   const int64_t n_max = s->node_cap[seg_last];
   MoveArgs m{};
   m.g.n = n;
@@ -741,6 +742,9 @@ int launch_lru_insert(Server *s, Pipe &p, hipStream_t st, int n_lists) {
     hipLaunchKernelGGL(lru_round_kernel, dim3(grid), dim3(256), 0, st, a);
   }
   LMI_HIP(hipGetLastError());
+  // keys and ticks are final: the next batch's lookup may start while the rows are still copied
+  LMI_HIP(hipEventRecord(s->lru_ready, st));
+  s->lru_pending = true;
   // copy the granted rows from the output buffer (already gathered) into the cache
   for (int l = 0; l < n_lists; ++l) {
     MoveArgs m{};
@@ -757,8 +761,8 @@ int launch_lru_insert(Server *s, Pipe &p, hipStream_t st, int n_lists) {
     m.n_max = s->node_cap[s->cfg.hops];
     LMI_TRY(launch_move_rows(s, st, m, false));
   }
-  LMI_HIP(hipEventRecord(s->lru_ready, st));
-  s->lru_pending = true;
+  LMI_HIP(hipEventRecord(s->lru_copied, st));
+  s->lru_copy_pending = true;
   return LMI_OK;
 }
 
@@ -772,6 +776,18 @@ int lru_wait_ready(Server *s, hipStream_t st) {
   }
   (void)hipGetLastError();  // "not ready" is an answer, not a failure
   LMI_HIP(hipStreamWaitEvent(st, s->lru_ready, 0));
+  return LMI_OK;
+}
+
+// The rows the previous batch's insertion granted must be in the cache before a gather reads it.
+int lru_wait_copied(Server *s, hipStream_t st) {
+  if (s->cache_kind != LMI_CACHE_LRU || !s->lru_copy_pending) return LMI_OK;
+  if (hipEventQuery(s->lru_copied) == hipSuccess) {
+    s->lru_copy_pending = false;
+    return LMI_OK;
+  }
+  (void)hipGetLastError();
+  LMI_HIP(hipStreamWaitEvent(st, s->lru_copied, 0));
   return LMI_OK;
 }
 
@@ -901,7 +917,7 @@ int launch_table_clear(Table &t, hipStream_t st) {
 
 void cache_free(Server *s) {
   (void)hipDeviceSynchronize();  // batches in flight (side stream included) still read the old cache
-  s->lru_pending = false;
+  s->lru_pending = s->lru_copy_pending = false;
   if (s->cache_data) (void)hipFree(s->cache_data);
   if (s->cache_scale) (void)hipFree(s->cache_scale);
   if (s->id_table.slots) (void)hipFree(s->id_table.slots);

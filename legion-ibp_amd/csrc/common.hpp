@@ -163,8 +163,10 @@ struct Server {
   int protect_hits = 0;            // 1: HBM gathers wait until earlier host-link gathers have drained
   int lru_early_miss = 1;          // 1: with the LRU cache the host-link gather starts beside the HBM gather
   int group_miss = 1;              // 1: the host-link gathers of a group of batches are one launch
-  hipEvent_t lru_ready = nullptr;  // recorded behind every LRU insertion: the next lookup waits for it
+  hipEvent_t lru_ready = nullptr;  // recorded when an LRU insertion has settled keys and ticks: the next lookup waits for it
   bool lru_pending = false;        // an insertion may still be running
+  hipEvent_t lru_copied = nullptr; // recorded when the granted rows are in the cache: the next HBM gather waits for it
+  bool lru_copy_pending = false;
   // pipes
   std::vector<Pipe> pipes;
   hipStream_t side = nullptr;  // server-owned second stream for gathers that must not hold up the caller's stream
@@ -245,7 +247,8 @@ int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last,
 // host-link gathers one after another on the side stream.
 int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg, int seg_last, int lru_lists);
 int launch_lru_insert(Server *s, Pipe &p, hipStream_t st, int n_lists);
-int lru_wait_ready(Server *s, hipStream_t st);  // orders `st` behind the last LRU insertion
+int lru_wait_ready(Server *s, hipStream_t st);
+int lru_wait_copied(Server *s, hipStream_t st);  // orders `st` behind the last LRU insertion
 int pipe_join(Pipe &p, hipStream_t st);  // make `st` wait for the pipe's side-stream work
 int cache_dump(Server *s, int32_t *slot_of, int64_t n, int32_t *aux);
 
