@@ -840,3 +840,68 @@ def test_batches_that_nearly_fill_their_buffers(lmi, oracle, fanout, batch, n_no
     finally:
         srv.close()
         feats.free()
+
+
+@pytest.mark.parametrize("case", range(48))
+def test_random_groups_sweep(lmi, oracle, case):
+    """Seeded sweep through lmi_run_group: random group sizes on random subsets of 2..16 pipes,
+    ragged seed lists, every launch shape and gather schedule the tuning keys select."""
+    rng = np.random.default_rng(31000 + case)
+    hops = int(rng.integers(1, 4))
+    fanout = [int(rng.choice([1, 2, 3, 5, 8, 16, 25, 33, 64])) for _ in range(hops)]
+    n_nodes = int(rng.choice([2, 50, 1000, 20000, 200000]))
+    batch = int(rng.choice([1, 7, 64, 500]))
+    hubs = int(rng.integers(0, 3)) if n_nodes >= 1000 else 0
+    indptr, indices = random_graph(rng, n_nodes, float(rng.choice([0, 1, 5, 40])), hubs=hubs,
+                                   hub_deg=int(rng.choice([300, 70000])), zero_frac=float(rng.choice([0.0, 0.3])))
+    dim = int(rng.choice([4, 20, 128]))
+    pipes = int(rng.choice([2, 4, 8, 16]))
+    worst = batch
+    for f in fanout:
+        worst *= 1 + f
+    while worst * (dim * 4 + 64) * pipes > 4e9 and batch > 1:   # keep the output buffers of all pipes modest
+        batch = max(1, batch // 4)
+        worst = batch
+        for f in fanout:
+            worst *= 1 + f
+    feats = make_features(lmi, rng, n_nodes, dim)
+    srv = lmi.Server(batch, fanout, dim, pipes=pipes, seed=5)
+    stream = lmi.stream_create() if case % 2 else None
+    kind = ["static", "int8", "none"][case % 3]
+    slot_ref = q = sc = None
+    try:
+        for key, vals in (("group_miss", [0, 1]), ("protect_hits", [0, 1]), ("fuse_count", [0, 1]),
+                          ("table_epochs", [0, 2, 1 << 30]), ("miss_blocks", [1, 8, 32]), ("split_miss", [0, 1, 2])):
+            srv.tune(key, int(rng.choice(vals)))
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        cap = int(rng.integers(1, n_nodes + 1))
+        if kind == "static":
+            srv.build_static_cache(cap, int(rng.integers(0, 3)))
+            slot_ref = oracle.static_cache_build(indptr, cap)
+        elif kind == "int8":
+            srv.build_int8_cache(cap, int(rng.integers(0, 3)))
+            slot_ref = oracle.static_cache_build(indptr, cap)
+            q, sc = oracle.quantize_rows(feats.array[np.flatnonzero(slot_ref >= 0)])
+        issued = 0
+        for rnd in range(4):
+            n = int(rng.integers(1, min(8, pipes) + 1))
+            plist = [int(x) for x in rng.choice(pipes, n, replace=False)]
+            seeds = [rng.integers(0, n_nodes, int(rng.integers(1, batch + 1))).astype(np.int32) for _ in plist]
+            rs = [500 + issued + k for k in range(n)]
+            issued += n
+            srv.run_group(plist, [0] * n, seeds=seeds, rng_seeds=rs, stream=stream)
+            for k, pipe in enumerate(plist):
+                g = srv.fetch(pipe=pipe, stream=stream)
+                o = oracle.sample_batch(indptr, indices, seeds[k], fanout, rs[k])
+                assert_batch_equal(g, o)
+                if kind == "int8":
+                    np.testing.assert_array_equal(g.cache_index, slot_ref[o.ids])
+                    assert g.features.tobytes() == oracle.gather_rows_int8(o.ids, slot_ref[o.ids], q, sc, feats.array).tobytes()
+                else:
+                    assert g.features.tobytes() == feats.array[o.ids].tobytes()
+                    if slot_ref is not None:
+                        np.testing.assert_array_equal(g.cache_index, slot_ref[o.ids])
+    finally:
+        srv.close()
+        feats.free()
