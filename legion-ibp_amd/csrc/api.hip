@@ -100,7 +100,7 @@ static int dmalloc(T **p, int64_t count) {
 static void pipe_free(Pipe &p) {
   void *ptrs[] = {p.ids, p.features, p.labels, p.agg_src_ids, p.agg_src_off, p.agg_dst_off, p.blk_indptr[0],
                   p.blk_indptr[1], p.blk_indptr[2], p.cache_index, p.st, p.dedup.slots, p.eslot[0], p.eslot[1],
-                  p.miss_list, p.lru_fill, p.seed_stage,
+                  p.miss_list, p.lru_fill, p.lru_next, p.seed_stage,
                   p.chain_status[0], p.chain_status[1]};
   for (void *q : ptrs)
     if (q) (void)hipFree(q);
@@ -144,6 +144,7 @@ static int pipe_alloc(Server *s, Pipe &p) {
   LMI_TRY(dmalloc(&p.chain_status[1], p.max_tiles));
   LMI_TRY(dmalloc(&p.miss_list, s->max_nodes));
   LMI_TRY(dmalloc(&p.lru_fill, s->max_nodes));
+  LMI_TRY(dmalloc(&p.lru_next, s->max_nodes));
   LMI_TRY(dmalloc(&p.seed_stage, s->cfg.batch_size));
   LMI_HIP(hipEventCreateWithFlags(&p.fork, hipEventDisableTiming));
   LMI_HIP(hipEventCreateWithFlags(&p.join, hipEventDisableTiming));

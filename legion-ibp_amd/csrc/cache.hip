@@ -649,46 +649,53 @@ int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last,
 }
 
 // --------------------------------------------------------------- LRU insert
-// Round r of the batch-synchronous insertion.  claim[r&1][set] holds the
-// smallest row index among the set's still-unplaced misses; that row takes the
-// way with the smallest (last_use, way) among ways not touched in this batch.
-// Losers bid for the next round in the other claim array.  After `ways` rounds
-// every set has granted all the ways it can.
+// Batch-synchronous insertion in two launches.  lru_chain_kernel threads the misses of
+// every set into a list (head[set] -> row -> next[row] ...; one atomic exchange per miss,
+// on as many addresses as there are sets).  lru_place_kernel: the thread of the row at a
+// list's head serves its set alone -- the set's misses in ascending row order each take
+// the way with the smallest (last_use, way) among ways not touched in this batch, until
+// no way is left; the rest are refused (-2).  A list is as long as the batch has misses
+// in that set (one or two for any useful geometry), and the walk is serial, so a cache of
+// very few sets pays for its collisions in time, not in correctness.
 struct LruArgs {
   const int32_t *ids;
   const int2 *miss_list[LMI_MAX_HOPS + 1];
   const DevState *st;
   int n_lists;
-  int32_t *keys, *use, *claim_cur, *claim_next, *fill;
+  int32_t *keys, *use, *head, *next, *fill;
   int64_t sets;
-  int ways, round, last_round;
+  int ways;
 };
 
-static __global__ __launch_bounds__(256) void lru_bid_kernel(LruArgs a) {
+static __global__ __launch_bounds__(256) void lru_chain_kernel(LruArgs a) {
   for (int l = 0; l < a.n_lists; ++l) {
     const int n = a.st->n_miss[l];
     for (int j = blockIdx.x * blockDim.x + threadIdx.x; j < n; j += gridDim.x * blockDim.x) {
       const int2 pr = a.miss_list[l][j];  // (row, id)
       const int i = pr.x;
       if (a.fill[i] != -1) continue;  // the later row of a repeated seed
-      atomicMin(&a.claim_cur[(uint32_t)pr.y % (uint32_t)a.sets], i);
+      a.next[i] = atomicExch(&a.head[(uint32_t)pr.y % (uint32_t)a.sets], i);
     }
   }
 }
 
-static __global__ __launch_bounds__(256) void lru_round_kernel(LruArgs a) {
+static __global__ __launch_bounds__(256) void lru_place_kernel(LruArgs a) {
+  const int tick = a.st->lru_tick;
   for (int l = 0; l < a.n_lists; ++l) {
     const int n = a.st->n_miss[l];
     for (int j = blockIdx.x * blockDim.x + threadIdx.x; j < n; j += gridDim.x * blockDim.x) {
       const int2 pr = a.miss_list[l][j];  // (row, id)
       const int i = pr.x;
-      if (a.fill[i] != -1) continue;  // placed (>= 0) or refused (-2) earlier
-      const int32_t id = pr.y;
-      const int64_t set = (uint32_t)id % (uint32_t)a.sets;  // sets < 2^31
-      if (a.claim_cur[set] == i) {
-        const int64_t base = set * a.ways;
+      const int64_t set = (uint32_t)pr.y % (uint32_t)a.sets;  // sets < 2^31
+      if (a.head[set] != i) continue;  // some other row's thread serves this set
+      const int64_t base = set * a.ways;
+      int last = -1;  // the row placed last; the next one is the smallest row above it
+      for (int placed = 0; placed < a.ways; ++placed) {
+        int row = kIntMax;
+        for (int r = i; r != -1; r = a.next[r])
+          if (r > last && r < row) row = r;
+        if (row == kIntMax) break;  // everybody is placed
         int best = -1, best_use = kIntMax;
-        const int tick = a.st->lru_tick;
         if ((a.ways & 3) == 0) {  // four ways per load, same order of preference (lowest way wins a tie)
           for (int w = 0; w < a.ways; w += 4) {
             const int4 u = *reinterpret_cast<const int4 *>(a.use + base + w);
@@ -703,17 +710,15 @@ static __global__ __launch_bounds__(256) void lru_round_kernel(LruArgs a) {
             if (u < tick && u < best_use) best = w, best_use = u;
           }
         }
-        if (best >= 0) {
-          a.keys[base + best] = id;
-          a.use[base + best] = tick;
-          a.fill[i] = (int)(base + best);
-        } else {
-          a.fill[i] = -2;
-        }
-        a.claim_cur[set] = kIntMax;
-      } else if (!a.last_round) {
-        atomicMin(&a.claim_next[set], i);
+        if (best < 0) break;  // every way was touched in this batch
+        a.keys[base + best] = a.ids[row];
+        a.use[base + best] = tick;
+        a.fill[row] = (int)(base + best);
+        last = row;
       }
+      for (int r = i; r != -1; r = a.next[r])
+        if (a.fill[r] == -1) a.fill[r] = -2;  // no way left for these
+      a.head[set] = -1;  // ready for the next batch
     }
   }
 }
@@ -728,19 +733,13 @@ int launch_lru_insert(Server *s, Pipe &p, hipStream_t st, int n_lists) {
   a.keys = s->lru_keys;
   a.use = s->lru_use;
   a.fill = p.lru_fill;
+  a.next = p.lru_next;
+  a.head = s->lru_head;
   a.sets = s->lru_sets;
   a.ways = s->lru_ways;
   const int grid = (int)std::max<int64_t>(1, std::min<int64_t>(ceil_div(s->max_nodes, 256), (int64_t)s->n_cu * 4));
-  a.claim_cur = s->lru_claim[0];
-  a.claim_next = s->lru_claim[1];
-  hipLaunchKernelGGL(lru_bid_kernel, dim3(grid), dim3(256), 0, st, a);
-  for (int r = 0; r < s->lru_ways; ++r) {
-    a.round = r;
-    a.last_round = (r == s->lru_ways - 1);
-    a.claim_cur = s->lru_claim[r & 1];
-    a.claim_next = s->lru_claim[(r + 1) & 1];
-    hipLaunchKernelGGL(lru_round_kernel, dim3(grid), dim3(256), 0, st, a);
-  }
+  hipLaunchKernelGGL(lru_chain_kernel, dim3(grid), dim3(256), 0, st, a);
+  hipLaunchKernelGGL(lru_place_kernel, dim3(grid), dim3(256), 0, st, a);
   LMI_HIP(hipGetLastError());
   // keys and ticks are final: the next batch's lookup may start while the rows are still copied
   LMI_HIP(hipEventRecord(s->lru_ready, st));
@@ -925,14 +924,13 @@ void cache_free(Server *s) {
   if (s->rank_tab) (void)hipFree(s->rank_tab);
   if (s->lru_keys) (void)hipFree(s->lru_keys);
   if (s->lru_use) (void)hipFree(s->lru_use);
-  if (s->lru_claim[0]) (void)hipFree(s->lru_claim[0]);
-  if (s->lru_claim[1]) (void)hipFree(s->lru_claim[1]);
+  if (s->lru_head) (void)hipFree(s->lru_head);
   s->cache_data = nullptr;
   s->cache_scale = nullptr;
   s->id_table = Table{};
   s->slot_of = nullptr;
   s->rank_tab = nullptr;
-  s->lru_keys = s->lru_use = s->lru_claim[0] = s->lru_claim[1] = nullptr;
+  s->lru_keys = s->lru_use = s->lru_head = nullptr;
   s->cache_kind = LMI_CACHE_NONE;
   s->cache_rows = 0;
 }
@@ -1066,14 +1064,12 @@ int cache_build_lru(Server *s, int64_t n_sets, int32_t ways) {
   const int64_t rows = n_sets * ways;
   LMI_HIP(hipMalloc(&s->lru_keys, rows * 4));
   LMI_HIP(hipMalloc(&s->lru_use, rows * 4));
-  LMI_HIP(hipMalloc(&s->lru_claim[0], n_sets * 4));
-  LMI_HIP(hipMalloc(&s->lru_claim[1], n_sets * 4));
+  LMI_HIP(hipMalloc(&s->lru_head, n_sets * 4));
   LMI_HIP(hipMalloc(&s->cache_data, (size_t)rows * s->row_bytes));
   const int g = 2048;
   hipLaunchKernelGGL(fill_i32_kernel, dim3(g), dim3(256), 0, 0, s->lru_keys, rows, -1);
   hipLaunchKernelGGL(fill_i32_kernel, dim3(g), dim3(256), 0, 0, s->lru_use, rows, 0);
-  hipLaunchKernelGGL(fill_i32_kernel, dim3(g), dim3(256), 0, 0, s->lru_claim[0], n_sets, kIntMax);
-  hipLaunchKernelGGL(fill_i32_kernel, dim3(g), dim3(256), 0, 0, s->lru_claim[1], n_sets, kIntMax);
+  hipLaunchKernelGGL(fill_i32_kernel, dim3(g), dim3(256), 0, 0, s->lru_head, n_sets, -1);
   LMI_HIP(hipDeviceSynchronize());
   s->lru_sets = n_sets;
   s->lru_ways = ways;

@@ -96,6 +96,7 @@ struct Pipe {
   int32_t max_tiles = 0;
   int2 *miss_list = nullptr;   // [max_nodes] (row, id) pairs of cache misses
   int32_t *lru_fill = nullptr;                        // [max_nodes] slot granted to a miss
+  int32_t *lru_next = nullptr;                        // [max_nodes] next row in the list of misses of the same LRU set
   hipEvent_t fork = nullptr, join = nullptr;
   bool side_pending = false;   // the side stream still owes this pipe's miss rows (join not yet waited on)
   int32_t *seed_stage = nullptr;  // [batch_size] host seeds land here
@@ -157,7 +158,8 @@ struct Server {
   int64_t lru_sets = 0;
   int32_t lru_ways = 0;
   int32_t lru_tick = 0;
-  int32_t *lru_keys = nullptr, *lru_use = nullptr, *lru_claim[2] = {nullptr, nullptr};
+  int32_t *lru_keys = nullptr, *lru_use = nullptr;
+  int32_t *lru_head = nullptr;  // [sets] first row of the set's list of misses while a batch is inserted, else -1
   hipEvent_t side_idle = nullptr;  // recorded behind the last host-link gather issued on the side stream
   bool side_busy = false;
   int protect_hits = 0;            // 1: HBM gathers wait until earlier host-link gathers have drained
