@@ -374,21 +374,27 @@ static __global__ __launch_bounds__(kLookupBlock) void lookup_kernel(LookupGroup
       int slot = -1;
       if (id >= 0 && id < a.n_nodes) {
         if (a.kind == LMI_CACHE_LRU) {
-          // sets * ways < 2^31, so 32-bit arithmetic addresses every way
-          const int base = (int)((uint32_t)id % (uint32_t)a.lru_sets) * a.lru_ways;
+          // a set's record is its keys followed by its ticks (one 64-byte line for 8 ways), so the
+          // tick of a hit is written into the line its key was just read from
+          const int set = (int)((uint32_t)id % (uint32_t)a.lru_sets);
+          const int64_t rec = (int64_t)set * 2 * a.lru_ways;
+          int way = -1;
           if ((a.lru_ways & 3) == 0) {  // a set's keys start on a 16-byte boundary: four ways per load
             for (int w = 0; w < a.lru_ways; w += 4) {
-              const int4 k = *reinterpret_cast<const int4 *>(a.lru_keys + base + w);
-              if (k.x == id) slot = base + w;
-              if (k.y == id) slot = base + w + 1;
-              if (k.z == id) slot = base + w + 2;
-              if (k.w == id) slot = base + w + 3;
+              const int4 k = *reinterpret_cast<const int4 *>(a.lru_keys + rec + w);
+              if (k.x == id) way = w;
+              if (k.y == id) way = w + 1;
+              if (k.z == id) way = w + 2;
+              if (k.w == id) way = w + 3;
             }
           } else {
             for (int w = 0; w < a.lru_ways; ++w)
-              if (a.lru_keys[base + w] == id) slot = base + w;
+              if (a.lru_keys[rec + w] == id) way = w;
           }
-          if (slot >= 0) a.lru_use[slot] = a.st->lru_tick;
+          if (way >= 0) {
+            slot = set * a.lru_ways + way;  // sets * ways < 2^31
+            a.lru_use[rec + way] = a.st->lru_tick;
+          }
           // a repeated seed keeps both rows, but the id is offered for insertion once, by its first row
           const bool repeat = i < a.st->n_seeds &&
                               table_find(a.dedup, a.dedup_log2cap, id, a.st->table_tag, a.st->table_mask) != i;
@@ -688,7 +694,8 @@ static __global__ __launch_bounds__(256) void lru_place_kernel(LruArgs a) {
       const int i = pr.x;
       const int64_t set = (uint32_t)pr.y % (uint32_t)a.sets;  // sets < 2^31
       if (a.head[set] != i) continue;  // some other row's thread serves this set
-      const int64_t base = set * a.ways;
+      const int64_t base = set * a.ways;     // the set's first slot (row of the cache)
+      const int64_t rec = set * 2 * a.ways;  // the set's record: keys, then ticks
       int last = -1;  // the row placed last; the next one is the smallest row above it
       for (int placed = 0; placed < a.ways; ++placed) {
         int row = kIntMax;
@@ -698,7 +705,7 @@ static __global__ __launch_bounds__(256) void lru_place_kernel(LruArgs a) {
         int best = -1, best_use = kIntMax;
         if ((a.ways & 3) == 0) {  // four ways per load, same order of preference (lowest way wins a tie)
           for (int w = 0; w < a.ways; w += 4) {
-            const int4 u = *reinterpret_cast<const int4 *>(a.use + base + w);
+            const int4 u = *reinterpret_cast<const int4 *>(a.use + rec + w);
             if (u.x < tick && u.x < best_use) best = w, best_use = u.x;
             if (u.y < tick && u.y < best_use) best = w + 1, best_use = u.y;
             if (u.z < tick && u.z < best_use) best = w + 2, best_use = u.z;
@@ -706,13 +713,13 @@ static __global__ __launch_bounds__(256) void lru_place_kernel(LruArgs a) {
           }
         } else {
           for (int w = 0; w < a.ways; ++w) {
-            const int u = a.use[base + w];
+            const int u = a.use[rec + w];
             if (u < tick && u < best_use) best = w, best_use = u;
           }
         }
         if (best < 0) break;  // every way was touched in this batch
-        a.keys[base + best] = a.ids[row];
-        a.use[base + best] = tick;
+        a.keys[rec + best] = a.ids[row];
+        a.use[rec + best] = tick;
         a.fill[row] = (int)(base + best);
         last = row;
       }
@@ -922,8 +929,7 @@ void cache_free(Server *s) {
   if (s->id_table.slots) (void)hipFree(s->id_table.slots);
   if (s->slot_of) (void)hipFree(s->slot_of);
   if (s->rank_tab) (void)hipFree(s->rank_tab);
-  if (s->lru_keys) (void)hipFree(s->lru_keys);
-  if (s->lru_use) (void)hipFree(s->lru_use);
+  if (s->lru_keys) (void)hipFree(s->lru_keys);  // one allocation: lru_use points into it
   if (s->lru_head) (void)hipFree(s->lru_head);
   s->cache_data = nullptr;
   s->cache_scale = nullptr;
@@ -1056,19 +1062,24 @@ int cache_build_static(Server *s, int64_t capacity_rows, int table_kind, bool in
   return LMI_OK;
 }
 
+// Empty LRU records: key -1 and tick 0 in every way.
+static __global__ __launch_bounds__(256) void lru_init_kernel(int32_t *rec, int64_t n_words, int ways) {
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_words; i += (int64_t)gridDim.x * blockDim.x)
+    rec[i] = ((i / ways) & 1) ? 0 : -1;
+}
+
 int cache_build_lru(Server *s, int64_t n_sets, int32_t ways) {
   if (!s->feat) LMI_FAIL(LMI_ERR_STATE, "attach features before building a cache");
   if (n_sets < 1 || ways < 1 || ways > 64 || n_sets * ways >= (int64_t(1) << 31))
     LMI_FAIL(LMI_ERR_ARG, "bad LRU geometry (sets=%lld ways=%d)", (long long)n_sets, ways);
   cache_free(s);
   const int64_t rows = n_sets * ways;
-  LMI_HIP(hipMalloc(&s->lru_keys, rows * 4));
-  LMI_HIP(hipMalloc(&s->lru_use, rows * 4));
+  LMI_HIP(hipMalloc(&s->lru_keys, rows * 8));  // per set: `ways` keys, then `ways` ticks
+  s->lru_use = s->lru_keys + ways;
   LMI_HIP(hipMalloc(&s->lru_head, n_sets * 4));
   LMI_HIP(hipMalloc(&s->cache_data, (size_t)rows * s->row_bytes));
   const int g = 2048;
-  hipLaunchKernelGGL(fill_i32_kernel, dim3(g), dim3(256), 0, 0, s->lru_keys, rows, -1);
-  hipLaunchKernelGGL(fill_i32_kernel, dim3(g), dim3(256), 0, 0, s->lru_use, rows, 0);
+  hipLaunchKernelGGL(lru_init_kernel, dim3(g), dim3(256), 0, 0, s->lru_keys, rows * 2, ways);
   hipLaunchKernelGGL(fill_i32_kernel, dim3(g), dim3(256), 0, 0, s->lru_head, n_sets, -1);
   LMI_HIP(hipDeviceSynchronize());
   s->lru_sets = n_sets;
@@ -1091,8 +1102,14 @@ int cache_dump(Server *s, int32_t *slot_of, int64_t n, int32_t *aux) {
   LMI_HIP(hipDeviceSynchronize());
   if (s->cache_kind == LMI_CACHE_LRU) {
     if (n != s->cache_rows) LMI_FAIL(LMI_ERR_ARG, "LRU dump needs n == sets*ways");
-    LMI_HIP(hipMemcpy(slot_of, s->lru_keys, n * 4, hipMemcpyDeviceToHost));
-    if (aux) LMI_HIP(hipMemcpy(aux, s->lru_use, n * 4, hipMemcpyDeviceToHost));
+    std::vector<int32_t> rec((size_t)n * 2);
+    LMI_HIP(hipMemcpy(rec.data(), s->lru_keys, (size_t)n * 8, hipMemcpyDeviceToHost));
+    const int64_t ways = s->lru_ways;
+    for (int64_t slot = 0; slot < n; ++slot) {  // slot = set * ways + way
+      const int64_t at = slot / ways * 2 * ways + slot % ways;
+      slot_of[slot] = rec[at];
+      if (aux) aux[slot] = rec[at + ways];
+    }
     return LMI_OK;
   }
   if (n != s->n_nodes) LMI_FAIL(LMI_ERR_ARG, "dump needs n == n_nodes");

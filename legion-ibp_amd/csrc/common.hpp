@@ -158,7 +158,8 @@ struct Server {
   int64_t lru_sets = 0;
   int32_t lru_ways = 0;
   int32_t lru_tick = 0;
-  int32_t *lru_keys = nullptr, *lru_use = nullptr;
+  int32_t *lru_keys = nullptr, *lru_use = nullptr;  // one array of per-set records: `ways` keys, then `ways` ticks;
+                                                    // way w of set s: lru_keys[(s * 2) * ways + w], lru_use[same]
   int32_t *lru_head = nullptr;  // [sets] first row of the set's list of misses while a batch is inserted, else -1
   hipEvent_t side_idle = nullptr;  // recorded behind the last host-link gather issued on the side stream
   bool side_busy = false;
