@@ -404,6 +404,11 @@ def main():
                    "note": info["note"]},
         "feature_gather_gbs": round(achieved, 1),
         "feature_gather_frac_hbm_peak": round(achieved / HBM_PEAK_GBS, 4),
+        # hits and misses together: all bytes moved into the output rows over the time of both kernels
+        # (they run on different streams, so this is a lower bound on what the batch sees)
+        "feature_gather_blended_gbs": round((hit_rows / hit_batches * hit_bytes + miss_rows / miss_batches * (2 * rb + 8)) /
+                                            ((hit_ms / hit_batches + miss_ms / miss_batches) * 1e-3) / 1e9, 1)
+        if hit_ms + miss_ms > 0 else None,
         "cache_hit_rate": round(prof.gather_hit_rows / total_rows, 4) if total_rows else None,
         "rows_per_batch": round(total_rows / max(profiled_batches, 1), 1),
         "profiled_batches": profiled_batches,
