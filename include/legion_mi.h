@@ -213,6 +213,30 @@ int lmi_run_group(lmi_server *s, int n_batches, const int32_t *pipes, void *stre
                   const int32_t *const *seeds, const int32_t *n_seeds, int seeds_location,
                   const int32_t *batch_counters, int mode, const uint64_t *rng_seeds);
 
+/* ---- one batch without any allocation ---------------------------------- */
+/* Limits of lmi_run_once_static: the server's worst-case rows per batch (max_nodes of its
+ * batch view) and worst-case edges of its largest hop, e.g. batch 800 with fan-out [25, 10]. */
+#define LMI_STATIC_MAX_NODES      (1 << 18)
+#define LMI_STATIC_MAX_HOP_EDGES  (1 << 18)
+/* bytes of device memory the library holds per GPU for it, from load to process end */
+#define LMI_STATIC_SCRATCH_BYTES  ((size_t)10 << 20)
+/* No counterpart in the reference.  For callers that cannot allocate device memory: code under
+ * HIP graph capture, tight serving loops, harnesses that forbid it.  The same batch as
+ * lmi_run_once (all hops, one lookup, one gather over all rows; hits and misses both on
+ * `stream`, no side stream, nothing left pending), but every output goes into buffers the CALLER
+ * owns -- `out` names them, all device memory, sized for the server's worst case:
+ * ids / cache_index [max_nodes], features [max_nodes][feat_dim], labels [batch_size],
+ * agg_* [max_edges], blk_indptr[k] [n_k + 1], node_counter / edge_counter [16] -- and the
+ * kernels' scratch (dedup table, per-edge slots, scan status words, miss list, batch state)
+ * lives in one file-scope device array of LMI_STATIC_SCRATCH_BYTES per GPU instead of a pipe.
+ * Calls no hipMalloc / hipFree and nothing else that allocates.  `seeds` is device memory.
+ * Servers whose worst case exceeds the limits above, and servers with the LRU cache (whose
+ * insertion needs per-pipe state), get LMI_ERR_CAPACITY / LMI_ERR_STATE.  Every call on a GPU
+ * shares that GPU's array: calls that overlap on one GPU (two streams, two threads, two
+ * servers) race; calls that follow each other on one stream do not. */
+int lmi_run_once_static(lmi_server *s, void *stream, const int32_t *seeds, int32_t n,
+                        uint64_t rng_seed, const lmi_batch_view *out);
+
 /* ---- outputs ----------------------------------------------------------- */
 /* Makes `stream` wait until every output of the pipe's last batch is complete,
  * including rows still being fetched over the host link on the server's own side

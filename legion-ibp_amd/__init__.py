@@ -14,6 +14,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "liblegion_mi.so")
 
 MAX_HOPS, MAX_FANOUT, MAX_PIPES, MAX_GROUP = 3, 64, 16, 8
+STATIC_MAX_NODES, STATIC_MAX_HOP_EDGES = 1 << 18, 1 << 18   # limits of lmi_run_once_static
 F32, F16 = 0, 1
 LOC_HOST, LOC_DEVICE = 0, 1
 MODE_TRAIN, MODE_VALID, MODE_TEST = 0, 1, 2
@@ -31,7 +32,7 @@ ABI_SYMBOLS = [
     "lmi_cache_policy", "lmi_cache_build_static", "lmi_cache_build_lru", "lmi_cache_build_int8",
     "lmi_cache_info_get", "lmi_cache_dump", "lmi_op_batch_generate", "lmi_op_random_sample",
     "lmi_op_cache_lookup", "lmi_op_io_submit", "lmi_op_io_complete", "lmi_run_once",
-    "lmi_run_group", "lmi_batch_wait", "lmi_batch_view_get", "lmi_batch_counters", "lmi_steps_per_epoch", "lmi_profile_enable",
+    "lmi_run_group", "lmi_run_once_static", "lmi_batch_wait", "lmi_batch_view_get", "lmi_batch_counters", "lmi_steps_per_epoch", "lmi_profile_enable",
     "lmi_profile_read", "lmi_tune", "lmi_bench_copy", "lmi_bench_host_read", "lmi_bench_random_read", "lmi_synth_graph", "lmi_synth_trainset",
     "lmi_synth_features",
 ]
@@ -121,6 +122,8 @@ def lib():
         L.lmi_batch_counters.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         L.lmi_run_group.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
                                     C.c_void_p, C.c_int, C.c_void_p]
+        L.lmi_run_once_static.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int32, C.c_uint64,
+                                          C.POINTER(BatchView)]
         L.lmi_steps_per_epoch.argtypes = [C.c_void_p, C.c_int, C.POINTER(C.c_int32)]
         L.lmi_profile_enable.argtypes = [C.c_void_p, C.c_int]
         L.lmi_profile_read.argtypes = [C.c_void_p, C.POINTER(Profile), C.c_int]
@@ -294,6 +297,11 @@ class Server:
             sp = (C.c_void_p * n)(*[x.ctypes.data for x in keep])
             ns = (C.c_int32 * n)(*[len(x) for x in keep])
         check(lib().lmi_run_group(self.h, n, pa, stream, sp, ns, LOC_HOST, bc, mode, rs))
+
+    def run_once_static(self, seeds_dev, n, view, rng_seed=0, stream=None):
+        """lmi_run_once_static: `seeds_dev` is device memory holding n seed ids, `view` a BatchView of
+        caller-owned device buffers; nothing is allocated by the call."""
+        check(lib().lmi_run_once_static(self.h, stream, seeds_dev, n, rng_seed, C.byref(view)))
 
     # outputs -----------------------------------------------------------------
     def batch_wait(self, pipe=0, stream=None):

@@ -3,6 +3,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstring>
+#include <mutex>
 #include <new>
 
 #include "common.hpp"
@@ -111,6 +112,27 @@ static void pipe_free(Pipe &p) {
   p = Pipe{};
 }
 
+// Size of a batch's dedup table: load factor <= 2/3 in the worst case (every sampled edge a new
+// node); real batches fill a few percent, and a smaller table is cheaper to clear and to probe.
+static int dedup_log2cap(const Server *s) {
+  int lg = 4;
+  while ((int64_t(1) << lg) * 2 < 3 * s->max_nodes) ++lg;
+  return lg;
+}
+
+// Status words a look-back scan chain needs: the finest tiling any scan kernel uses, 256 items
+// per tile over nodes or edges, or the node tiles of the fused count-and-sample kernel.
+static int32_t scan_max_tiles(const Server *s) {
+  const int64_t scan_n = std::max(s->max_nodes, s->max_edges_hop);
+  int64_t tiles = ceil_div(scan_n, 256);
+  for (int k = 0; k < s->cfg.hops; ++k) {
+    int G = 4;
+    while (G < s->cfg.fanout[k]) G <<= 1;
+    tiles = std::max(tiles, ceil_div(s->node_cap[k], (int64_t)std::min(64, 256 / G)));  // smallest tile
+  }
+  return (int32_t)tiles + 1;
+}
+
 static int pipe_alloc(Server *s, Pipe &p) {
   LMI_TRY(dmalloc(&p.ids, s->max_nodes));
   LMI_HIP(hipMalloc(&p.features, (size_t)s->max_nodes * s->row_bytes));
@@ -122,24 +144,12 @@ static int pipe_alloc(Server *s, Pipe &p) {
   LMI_TRY(dmalloc(&p.cache_index, s->max_nodes));
   LMI_TRY(dmalloc(&p.st, 1));
   LMI_HIP(hipMemset(p.st, 0, sizeof(DevState)));
-  // load factor <= 2/3 in the worst case (every sampled edge a new node); real batches
-  // fill a few percent, and a smaller table is cheaper to clear and to probe
-  int lg = 4;
-  while ((int64_t(1) << lg) * 2 < 3 * s->max_nodes) ++lg;
+  const int lg = dedup_log2cap(s);
   p.dedup.log2cap = lg;
   LMI_HIP(hipMalloc(&p.dedup.slots, size_t(8) << lg));
   LMI_TRY(dmalloc(&p.eslot[0], s->max_edges_hop));
   LMI_TRY(dmalloc(&p.eslot[1], s->max_edges_hop));
-  const int64_t scan_n = std::max(s->max_nodes, s->max_edges_hop);
-  // the finest tiling any scan kernel uses: 256 items per tile over nodes or edges, or the
-  // node tiles of the fused count-and-sample kernel
-  int64_t tiles = ceil_div(scan_n, 256);
-  for (int k = 0; k < s->cfg.hops; ++k) {
-    int G = 4;
-    while (G < s->cfg.fanout[k]) G <<= 1;
-    tiles = std::max(tiles, ceil_div(s->node_cap[k], (int64_t)std::min(64, 256 / G)));  // smallest tile
-  }
-  p.max_tiles = (int32_t)tiles + 1;
+  p.max_tiles = scan_max_tiles(s);
   LMI_TRY(dmalloc(&p.chain_status[0], p.max_tiles));
   LMI_TRY(dmalloc(&p.chain_status[1], p.max_tiles));
   LMI_TRY(dmalloc(&p.miss_list, s->max_nodes));
@@ -170,6 +180,58 @@ static __global__ __launch_bounds__(256) void copy_kernel(const cp_u32x4 *__rest
   }
 }
 
+// ------------------------------------------- scratch of lmi_run_once_static
+// One array per GPU: every device that loads this code object holds its own copy at its own
+// address, from load until the process ends.  It stands in for the scratch a Pipe allocates at
+// server creation, carved at fixed offsets and sized for the limits in the header.  In host code
+// the array's NAME is only a handle for hipGetSymbolAddress; what kernels, fills and copies get
+// is the device address that call returned for the device in use (StaticScratch::ptr).
+constexpr int64_t kStaticLog2Cap = 19;  // 2^19 slots hold 1.5 x LMI_STATIC_MAX_NODES keys
+constexpr int64_t kStaticMaxTiles = LMI_STATIC_MAX_NODES / 4 + 32;  // smallest tile: 4 nodes (fan-out 64)
+constexpr size_t kOffState = 0;
+constexpr size_t kOffTable = 256;
+constexpr size_t kOffEslot0 = kOffTable + (size_t(8) << kStaticLog2Cap);
+constexpr size_t kOffEslot1 = kOffEslot0 + size_t(4) * LMI_STATIC_MAX_HOP_EDGES;
+constexpr size_t kOffChain0 = kOffEslot1 + size_t(4) * LMI_STATIC_MAX_HOP_EDGES;
+constexpr size_t kOffChain1 = kOffChain0 + size_t(8) * kStaticMaxTiles;
+constexpr size_t kOffMiss = kOffChain1 + size_t(8) * kStaticMaxTiles;
+constexpr size_t kStaticUsed = kOffMiss + size_t(8) * LMI_STATIC_MAX_NODES;
+static_assert(sizeof(DevState) <= 256, "the batch state has a 256-byte slot at the head of the scratch");
+static_assert(kStaticUsed <= LMI_STATIC_SCRATCH_BYTES, "the scratch array is too small for its pieces");
+static_assert(kOffEslot0 % 256 == 0 && kOffChain0 % 256 == 0 && kOffChain1 % 256 == 0 && kOffMiss % 256 == 0,
+              "every piece starts on a 256-byte boundary");
+
+static __device__ __align__(256) unsigned char scratch[LMI_STATIC_SCRATCH_BYTES];
+
+constexpr int kMaxDevices = 16;
+struct StaticScratch {
+  unsigned char *ptr = nullptr;  // device address of `scratch` on this device
+  Pipe pipe;                     // host-side bookkeeping of the one "pipe" that lives in it
+};
+static StaticScratch g_static[kMaxDevices];
+static std::mutex g_static_mu;
+
+// Once per device, with that device current (lmi_server_create).
+static int static_scratch_setup(int device) {
+  if (device < 0 || device >= kMaxDevices) return LMI_OK;  // such a device simply has no static entry point
+  std::lock_guard<std::mutex> lock(g_static_mu);
+  StaticScratch &sc = g_static[device];
+  if (sc.ptr) return LMI_OK;
+  unsigned char *ptr = nullptr;
+  LMI_HIP(hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch)));
+  if (!ptr) LMI_FAIL(LMI_ERR_HIP, "hipGetSymbolAddress gave no address for the static scratch");
+  sc.ptr = ptr;
+  return LMI_OK;
+}
+
+// The two 16-int headers live in the batch state; the caller of the static entry point owns
+// separate arrays for them.
+static __global__ void copy_headers_kernel(const DevState *st, int32_t *node_counter, int32_t *edge_counter) {
+  const int t = threadIdx.x;
+  if (t < 16) node_counter[t] = st->node_counter[t];
+  else if (t < 32) edge_counter[t - 16] = st->edge_counter[t - 16];
+}
+
 }  // namespace lmi
 
 using namespace lmi;
@@ -193,6 +255,7 @@ int lmi_server_create(const lmi_config *cfg, lmi_server **out) {
   LMI_HIP(hipGetDeviceCount(&n_dev));
   if (cfg->device_id < 0 || cfg->device_id >= n_dev) LMI_FAIL(LMI_ERR_ARG, "device %d not present", cfg->device_id);
   LMI_HIP(hipSetDevice(cfg->device_id));
+  LMI_TRY(static_scratch_setup(cfg->device_id));
   Server *s = new (std::nothrow) Server;
   if (!s) LMI_FAIL(LMI_ERR_HIP, "out of host memory");
   s->cfg = *cfg;
@@ -691,6 +754,79 @@ int lmi_run_group(lmi_server *h, int n_batches, const int32_t *pipes, void *stre
     LMI_TRY(batch_params(s, *pp[k], st, seeds ? seeds[k] : nullptr, (seeds && n_seeds) ? n_seeds[k] : 0, seeds_location,
                          batch_counters[k], mode, rng_seeds ? rng_seeds[k] : 0, &bps[k]));
   return run_group(s, pp, bps, n_batches, st);
+}
+
+int lmi_run_once_static(lmi_server *h, void *stream, const int32_t *seeds, int32_t n, uint64_t rng_seed,
+                        const lmi_batch_view *out) {
+  Server *s = reinterpret_cast<Server *>(h);
+  if (!s || !out || !seeds) LMI_FAIL(LMI_ERR_ARG, "null argument");
+  if (!s->feat) LMI_FAIL(LMI_ERR_STATE, "no features attached");
+  if (s->cache_kind == LMI_CACHE_LRU)
+    LMI_FAIL(LMI_ERR_STATE, "the LRU cache keeps per-pipe insertion state: use lmi_run_once");
+  if (s->max_nodes > LMI_STATIC_MAX_NODES || s->max_edges_hop > LMI_STATIC_MAX_HOP_EDGES)
+    LMI_FAIL(LMI_ERR_CAPACITY,
+             "this server's worst case (%lld rows per batch, %lld edges in a hop) exceeds the static scratch "
+             "(%d rows, %d edges): use lmi_run_once", (long long)s->max_nodes, (long long)s->max_edges_hop,
+             LMI_STATIC_MAX_NODES, LMI_STATIC_MAX_HOP_EDGES);
+  const int lg = dedup_log2cap(s);
+  const int32_t tiles = scan_max_tiles(s);
+  if (lg > kStaticLog2Cap || tiles > kStaticMaxTiles)
+    LMI_FAIL(LMI_ERR_CAPACITY, "this server's scan tiles or dedup table exceed the static scratch");
+  bool have = out->ids && out->features && out->labels && out->agg_src_ids && out->agg_src_off && out->agg_dst_off &&
+              out->node_counter && out->edge_counter && out->cache_index;
+  for (int k = 0; k < s->cfg.hops; ++k) have = have && out->blk_indptr[k];
+  if (!have) LMI_FAIL(LMI_ERR_ARG, "every output buffer of the view must be given");
+  if (out->max_nodes < s->max_nodes || out->max_edges < s->max_edges)
+    LMI_FAIL(LMI_ERR_CAPACITY, "the output buffers must hold the worst case: %lld rows, %lld edges",
+             (long long)s->max_nodes, (long long)s->max_edges);
+  if ((uintptr_t)out->features % 16 != 0) LMI_FAIL(LMI_ERR_ARG, "the feature buffer must be 16-byte aligned");
+  const int device = s->cfg.device_id;
+  if (device < 0 || device >= kMaxDevices || !g_static[device].ptr)
+    LMI_FAIL(LMI_ERR_STATE, "no static scratch on device %d", device);
+  LMI_HIP(hipSetDevice(device));
+  unsigned char *ptr = g_static[device].ptr;
+  Pipe &p = g_static[device].pipe;
+  // another server (another table size, other tilings) may have used the array last
+  if (p.dedup.log2cap != lg || p.max_tiles != tiles) p.table_dirty = true;
+  p.ids = out->ids;
+  p.features = out->features;
+  p.labels = out->labels;
+  p.agg_src_ids = out->agg_src_ids;
+  p.agg_src_off = out->agg_src_off;
+  p.agg_dst_off = out->agg_dst_off;
+  for (int k = 0; k < LMI_MAX_HOPS; ++k) p.blk_indptr[k] = out->blk_indptr[k];
+  p.cache_index = out->cache_index;
+  p.st = reinterpret_cast<DevState *>(ptr + kOffState);
+  p.dedup.slots = reinterpret_cast<HashSlot *>(ptr + kOffTable);
+  p.dedup.log2cap = lg;
+  p.eslot[0] = reinterpret_cast<int32_t *>(ptr + kOffEslot0);
+  p.eslot[1] = reinterpret_cast<int32_t *>(ptr + kOffEslot1);
+  p.chain_status[0] = reinterpret_cast<unsigned long long *>(ptr + kOffChain0);
+  p.chain_status[1] = reinterpret_cast<unsigned long long *>(ptr + kOffChain1);
+  p.max_tiles = tiles;
+  p.miss_list = reinterpret_cast<int2 *>(ptr + kOffMiss);
+  p.fill_pending = -1;
+  p.side_pending = false;
+  hipStream_t st = (hipStream_t)stream;
+  Pipe *pp[1] = {&p};
+  BatchParams bp{};
+  const bool prof = s->prof_on;
+  s->prof_on = false;  // profiling creates events: not here
+  int rc = batch_params(s, p, st, seeds, n, LMI_LOC_DEVICE, 0, LMI_MODE_TRAIN, rng_seed, &bp);
+  if (rc == LMI_OK) rc = launch_batch_generate(s, pp, &bp, 1, st, false);
+  for (int k = 0; rc == LMI_OK && k < s->cfg.hops; ++k) rc = launch_hop(s, pp, 1, st, k, true, true);
+  if (rc == LMI_OK) rc = launch_lookup(s, pp, 1, st, 0, s->cfg.hops);
+  if (rc == LMI_OK) rc = launch_gather_group(s, pp, 1, st, 0, s->cfg.hops, 0, true);
+  if (rc == LMI_OK) {
+    hipLaunchKernelGGL(copy_headers_kernel, dim3(1), dim3(64), 0, st, p.st, out->node_counter, out->edge_counter);
+    if (hipGetLastError() != hipSuccess) {
+      set_error("launch of the header copy failed");
+      rc = LMI_ERR_HIP;
+    }
+  }
+  if (rc != LMI_OK) p.table_dirty = true;  // a batch cut short may have left half an epoch behind
+  s->prof_on = prof;
+  return rc;
 }
 
 int lmi_batch_wait(lmi_server *h, int pipe, void *stream) {

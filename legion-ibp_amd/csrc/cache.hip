@@ -587,9 +587,10 @@ static int launch_misses(Server *s, Pipe *const *pp, int n, hipStream_t st, int 
 //      is done.
 // With 1 and 2 the caller's stream does not wait here: the next call on this pipe,
 // or lmi_batch_wait, joins.  The LRU cache joins at once (its insert copies the rows).
-int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg, int seg_last, int lru_lists) {
+int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg, int seg_last, int lru_lists,
+                        bool same_stream) {
   const bool have_cache = s->cache_kind != LMI_CACHE_NONE;
-  int mode = (s->feat_loc == LMI_LOC_HOST && have_cache) ? s->split_miss : 0;
+  int mode = (s->feat_loc == LMI_LOC_HOST && have_cache && !same_stream) ? s->split_miss : 0;
   // The gather kernels carry their own profiling events (prof_kernel_events); a bracket
   // left open by the sampling phase ends here.
   hipEvent_t closing = prof_phase(s, st, &s->prof_open, -1);

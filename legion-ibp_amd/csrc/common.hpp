@@ -248,7 +248,9 @@ int launch_hotness(Server *s, Pipe &p, hipStream_t st);
 int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last, int lru_lists);
 // The same for n pipes in step: the HBM gathers one after another, one fork, then the
 // host-link gathers one after another on the side stream.
-int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg, int seg_last, int lru_lists);
+// same_stream: hits then misses on `st` whatever the schedule knob says (nothing is left pending).
+int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg, int seg_last, int lru_lists,
+                        bool same_stream = false);
 int launch_lru_insert(Server *s, Pipe &p, hipStream_t st, int n_lists);
 int lru_wait_ready(Server *s, hipStream_t st);
 int lru_wait_copied(Server *s, hipStream_t st);  // orders `st` behind the last LRU insertion

@@ -1,0 +1,175 @@
+"""The entry point that allocates nothing (lmi_run_once_static): same outputs as lmi_run_once,
+bit for bit, on two calls in a row, the second with a smaller input; plus its refusals."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from conftest import random_graph
+
+pytestmark = pytest.mark.gpu
+
+
+class DeviceOutputs:
+    """Caller-owned device buffers for one batch, as an lmi_batch_view."""
+
+    def __init__(self, lmi, srv, poison=0xA5):
+        v0 = srv.view(0)   # only for the worst-case sizes
+        self.lmi, self.max_nodes, self.max_edges = lmi, int(v0.max_nodes), int(v0.max_edges)
+        self.dim, self.np_dtype = srv.cfg.feat_dim, srv.np_dtype
+        esz = np.dtype(self.np_dtype).itemsize
+        hops, batch = srv.cfg.hops, srv.cfg.batch_size
+        caps = [batch]
+        for k in range(hops):
+            caps.append(caps[-1] * (1 + srv.fanout[k]))
+        sizes = dict(ids=self.max_nodes * 4, features=self.max_nodes * self.dim * esz, labels=batch * 4,
+                     agg_src_ids=self.max_edges * 4, agg_src_off=self.max_edges * 4, agg_dst_off=self.max_edges * 4,
+                     node_counter=64, edge_counter=64, cache_index=self.max_nodes * 4)
+        for k in range(hops):
+            sizes["blk%d" % k] = (caps[k] + 1) * 4
+        self.ptr = {}
+        for name, nbytes in sizes.items():
+            p = C.c_void_p()
+            lmi.check(lmi.lib().lmi_device_alloc(nbytes, C.byref(p)))
+            junk = np.full(nbytes, poison, np.uint8)   # whatever a caller's buffer held before
+            lmi.check(lmi.lib().lmi_copy_to_device(p, junk.ctypes.data, nbytes))
+            self.ptr[name] = p
+        v = lmi.BatchView()
+        for name in ("ids", "features", "labels", "agg_src_ids", "agg_src_off", "agg_dst_off", "node_counter",
+                     "edge_counter", "cache_index"):
+            setattr(v, name, self.ptr[name])
+        for k in range(hops):
+            v.blk_indptr[k] = self.ptr["blk%d" % k]
+        v.max_nodes, v.max_edges = self.max_nodes, self.max_edges
+        self.view = v
+
+    def fetch(self):
+        lmi = self.lmi
+        nc = lmi.to_host(self.ptr["node_counter"], 16, np.int32)
+        ec = lmi.to_host(self.ptr["edge_counter"], 16, np.int32)
+        hops = int(nc[8])
+        b = lmi.Batch()
+        b.node_counter, b.edge_counter = nc, ec
+        b.n_nodes = [int(nc[9 + k]) for k in range(hops + 1)]
+        n, e = b.n_nodes[-1], int(sum(ec[9 + k] for k in range(1, hops + 1)))
+        b.ids = lmi.to_host(self.ptr["ids"], n, np.int32)
+        b.labels = lmi.to_host(self.ptr["labels"], b.n_nodes[0], np.int32)
+        for name in ("agg_src_ids", "agg_src_off", "agg_dst_off"):
+            setattr(b, name, lmi.to_host(self.ptr[name], e, np.int32))
+        b.blk_indptr = [lmi.to_host(self.ptr["blk%d" % k], b.n_nodes[k] + 1, np.int32) for k in range(hops)]
+        b.cache_index = lmi.to_host(self.ptr["cache_index"], n, np.int32)
+        b.features = lmi.to_host(self.ptr["features"], n * self.dim, self.np_dtype).reshape(n, self.dim)
+        return b
+
+    def free(self):
+        for p in self.ptr.values():
+            self.lmi.check(self.lmi.lib().lmi_device_free(p))
+
+
+def device_seeds(lmi, seeds):
+    p = C.c_void_p()
+    lmi.check(lmi.lib().lmi_device_alloc(max(4, seeds.nbytes), C.byref(p)))
+    if len(seeds):
+        lmi.check(lmi.lib().lmi_copy_to_device(p, seeds.ctypes.data, seeds.nbytes))
+    return p
+
+
+def assert_same(a, b):
+    assert list(a.node_counter) == list(b.node_counter) and list(a.edge_counter) == list(b.edge_counter)
+    for name in ("ids", "labels", "agg_src_ids", "agg_src_off", "agg_dst_off", "cache_index"):
+        assert np.array_equal(getattr(a, name), getattr(b, name)), name
+    for x, y in zip(a.blk_indptr, b.blk_indptr):
+        assert np.array_equal(x, y)
+    assert a.features.tobytes() == b.features.tobytes()
+
+
+@pytest.mark.parametrize("cache,dim,dtype,fanout,batch", [
+    ("static", 128, np.float32, [25, 10], 300),
+    ("int8", 768, np.float16, [25, 15], 64),
+    ("static", 100, np.float32, [5, 4, 3], 700),
+    ("none", 64, np.float32, [64, 2], 128),
+])
+def test_static_entry_point_matches_run_once_twice_in_a_row(lmi, oracle, cache, dim, dtype, fanout, batch):
+    rng = np.random.default_rng(11)
+    n_nodes = 30_000
+    indptr, indices = random_graph(rng, n_nodes, 14, hubs=8, hub_deg=3000)
+    feats = lmi.HostBuffer((n_nodes, dim), dtype)
+    feats.array[...] = rng.standard_normal((n_nodes, dim)).astype(dtype)
+    srv = lmi.Server(batch, fanout, dim, feat_dtype=lmi.F16 if dtype == np.float16 else lmi.F32, pipes=1, seed=5)
+    stream = lmi.stream_create()
+    outs, dseeds = None, []
+    try:
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        if cache == "static":
+            srv.build_static_cache(9000, lmi.TABLE_RANK)
+        elif cache == "int8":
+            srv.build_int8_cache(9000, lmi.TABLE_HASH)
+        outs = DeviceOutputs(lmi, srv)
+        # two calls in a row on the same scratch, the second with a smaller input, then a third
+        # as large as the first again
+        for call, n in enumerate([batch, max(1, batch // 5), batch]):
+            seeds = rng.choice(n_nodes, n, replace=False).astype(np.int32)
+            d = device_seeds(lmi, seeds)
+            dseeds.append(d)
+            srv.run_once_static(d, n, outs.view, rng_seed=100 + call, stream=stream)
+            lmi.check(lmi.lib().lmi_stream_sync(stream))
+            got = outs.fetch()
+            srv.run_once(seeds, rng_seed=100 + call, pipe=0, stream=stream)
+            ref = srv.fetch(pipe=0, stream=stream)
+            assert_same(got, ref)
+            # and both are what the oracle says
+            o = oracle.sample_batch(indptr, indices, seeds, fanout, 100 + call)
+            assert np.array_equal(got.ids, o.ids) and np.array_equal(got.agg_src_off, o.agg_src_off)
+            assert len(got.ids) > n
+    finally:
+        srv.close()
+        if outs:
+            outs.free()
+        for d in dseeds:
+            lmi.check(lmi.lib().lmi_device_free(d))
+        feats.free()
+
+
+def test_static_entry_point_refuses_what_it_cannot_hold(lmi):
+    rng = np.random.default_rng(3)
+    n_nodes, dim = 5000, 32
+    indptr, indices = random_graph(rng, n_nodes, 10)
+    feats = lmi.HostBuffer((n_nodes, dim), np.float32)
+    feats.array[...] = 1.0
+    seeds = np.arange(10, dtype=np.int32)
+    d = device_seeds(lmi, seeds)
+    try:
+        # worst case beyond the scratch: 8000 x 26 x 11 rows
+        big = lmi.Server(8000, [25, 10], dim, pipes=1)
+        try:
+            big.load_graph(indptr, indices)
+            big.attach_features(feats)
+            with pytest.raises(lmi.LegionError) as e:
+                big.run_once_static(d, 10, big.view(0))
+            assert e.value.code == -4 and "static scratch" in str(e.value)
+        finally:
+            big.close()
+        small = lmi.Server(64, [5, 5], dim, pipes=1)
+        try:
+            small.load_graph(indptr, indices)
+            small.attach_features(feats)
+            v = small.view(0)
+            v.max_nodes = 10   # buffers said to be too small
+            with pytest.raises(lmi.LegionError) as e:
+                small.run_once_static(d, 10, v)
+            assert e.value.code == -4
+            v = small.view(0)
+            v.cache_index = None
+            with pytest.raises(lmi.LegionError) as e:
+                small.run_once_static(d, 10, v)
+            assert e.value.code == -1
+            small.build_lru_cache(16, 4)
+            with pytest.raises(lmi.LegionError) as e:
+                small.run_once_static(d, 10, small.view(0))
+            assert e.value.code == -3
+        finally:
+            small.close()
+    finally:
+        lmi.check(lmi.lib().lmi_device_free(d))
+        feats.free()
