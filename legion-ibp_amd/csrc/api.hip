@@ -957,26 +957,45 @@ int lmi_tune(lmi_server *h, const char *key, int64_t value) {
   return LMI_OK;
 }
 
+// Buffers and events of a measurement, released on every return path.
+namespace {
+struct BenchScratch {
+  void *a = nullptr, *b = nullptr;
+  hipEvent_t e0 = nullptr, e1 = nullptr;
+  ~BenchScratch() {
+    if (e0) (void)hipEventDestroy(e0);
+    if (e1) (void)hipEventDestroy(e1);
+    if (a) (void)hipFree(a);
+    if (b) (void)hipFree(b);
+  }
+  int events() {
+    LMI_HIP(hipEventCreate(&e0));
+    LMI_HIP(hipEventCreate(&e1));
+    return LMI_OK;
+  }
+  int elapsed(int repeats, double *ms_out) {
+    LMI_HIP(hipEventRecord(e1, 0));
+    LMI_HIP(hipEventSynchronize(e1));
+    float ms = 0;
+    LMI_HIP(hipEventElapsedTime(&ms, e0, e1));
+    *ms_out = ms / repeats;
+    return LMI_OK;
+  }
+};
+}  // namespace
+
 int lmi_bench_host_read(const void *host_ptr, size_t bytes, int repeats, double *ms_per_pass) {
   if (!host_ptr || !ms_per_pass || repeats < 1 || bytes < 16) LMI_FAIL(LMI_ERR_ARG, "bad argument");
-  void *b = nullptr;
-  LMI_HIP(hipMalloc(&b, bytes));
-  hipEvent_t e0, e1;
-  LMI_HIP(hipEventCreate(&e0));
-  LMI_HIP(hipEventCreate(&e1));
+  BenchScratch m;
+  LMI_HIP(hipMalloc(&m.b, bytes));
+  LMI_TRY(m.events());
   const size_t n = bytes / 16;
-  hipLaunchKernelGGL(copy_kernel<true>, dim3(1024), dim3(256), 0, 0, (const cp_u32x4 *)host_ptr, (cp_u32x4 *)b, n);
-  LMI_HIP(hipEventRecord(e0, 0));
+  hipLaunchKernelGGL(copy_kernel<true>, dim3(1024), dim3(256), 0, 0, (const cp_u32x4 *)host_ptr, (cp_u32x4 *)m.b, n);
+  LMI_HIP(hipEventRecord(m.e0, 0));
   for (int r = 0; r < repeats; ++r)
-    hipLaunchKernelGGL(copy_kernel<true>, dim3(1024), dim3(256), 0, 0, (const cp_u32x4 *)host_ptr, (cp_u32x4 *)b, n);
-  LMI_HIP(hipEventRecord(e1, 0));
-  LMI_HIP(hipEventSynchronize(e1));
-  float ms = 0;
-  LMI_HIP(hipEventElapsedTime(&ms, e0, e1));
-  *ms_per_pass = ms / repeats;
-  (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
-  (void)hipFree(b);
-  return LMI_OK;
+    hipLaunchKernelGGL(copy_kernel<true>, dim3(1024), dim3(256), 0, 0, (const cp_u32x4 *)host_ptr, (cp_u32x4 *)m.b, n);
+  LMI_HIP(hipGetLastError());
+  return m.elapsed(repeats, ms_per_pass);
 }
 
 // Four independent reads per thread at places drawn by a 64-bit mixer; the sum goes nowhere
@@ -998,50 +1017,35 @@ static __global__ __launch_bounds__(256) void random_read_kernel(const uint32_t 
 
 int lmi_bench_random_read(const void *device_ptr, size_t bytes, int64_t n_reads, int repeats, double *ms_per_pass) {
   if (!device_ptr || !ms_per_pass || repeats < 1 || bytes < 4 || n_reads < 4) LMI_FAIL(LMI_ERR_ARG, "bad argument");
-  uint32_t *sink = nullptr;
-  LMI_HIP(hipMalloc(&sink, 4));
-  hipEvent_t e0, e1;
-  LMI_HIP(hipEventCreate(&e0));
-  LMI_HIP(hipEventCreate(&e1));
+  BenchScratch m;
+  LMI_HIP(hipMalloc(&m.a, 4));
+  uint32_t *sink = (uint32_t *)m.a;
+  LMI_TRY(m.events());
   const int grid = (int)std::min<int64_t>(ceil_div(ceil_div(n_reads, 4), 256), 1 << 30);
   const uint64_t n_words = bytes / 4;
   hipLaunchKernelGGL(random_read_kernel, dim3(grid), dim3(256), 0, 0, (const uint32_t *)device_ptr, n_words, n_reads, 1ull, sink);
-  LMI_HIP(hipEventRecord(e0, 0));
+  LMI_HIP(hipEventRecord(m.e0, 0));
   for (int r = 0; r < repeats; ++r)
     hipLaunchKernelGGL(random_read_kernel, dim3(grid), dim3(256), 0, 0, (const uint32_t *)device_ptr, n_words, n_reads,
                        (uint64_t)(r + 2) * 0x9E3779B97F4A7C15ull, sink);
-  LMI_HIP(hipEventRecord(e1, 0));
-  LMI_HIP(hipEventSynchronize(e1));
-  float ms = 0;
-  LMI_HIP(hipEventElapsedTime(&ms, e0, e1));
-  *ms_per_pass = ms / repeats;
-  (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
-  (void)hipFree(sink);
-  return LMI_OK;
+  LMI_HIP(hipGetLastError());
+  return m.elapsed(repeats, ms_per_pass);
 }
 
 int lmi_bench_copy(size_t bytes, int repeats, double *ms_per_copy) {
   if (!ms_per_copy || repeats < 1 || bytes < 16) LMI_FAIL(LMI_ERR_ARG, "bad argument");
-  void *a = nullptr, *b = nullptr;
-  LMI_HIP(hipMalloc(&a, bytes));
-  LMI_HIP(hipMalloc(&b, bytes));
-  LMI_HIP(hipMemset(a, 1, bytes));
-  hipEvent_t e0, e1;
-  LMI_HIP(hipEventCreate(&e0));
-  LMI_HIP(hipEventCreate(&e1));
+  BenchScratch m;
+  LMI_HIP(hipMalloc(&m.a, bytes));
+  LMI_HIP(hipMalloc(&m.b, bytes));
+  LMI_HIP(hipMemset(m.a, 1, bytes));
+  LMI_TRY(m.events());
   const size_t n = bytes / 16;
-  hipLaunchKernelGGL(copy_kernel<false>, dim3(16384), dim3(256), 0, 0, (const cp_u32x4 *)a, (cp_u32x4 *)b, n);
-  LMI_HIP(hipEventRecord(e0, 0));
+  hipLaunchKernelGGL(copy_kernel<false>, dim3(16384), dim3(256), 0, 0, (const cp_u32x4 *)m.a, (cp_u32x4 *)m.b, n);
+  LMI_HIP(hipEventRecord(m.e0, 0));
   for (int r = 0; r < repeats; ++r)
-    hipLaunchKernelGGL(copy_kernel<false>, dim3(16384), dim3(256), 0, 0, (const cp_u32x4 *)a, (cp_u32x4 *)b, n);
-  LMI_HIP(hipEventRecord(e1, 0));
-  LMI_HIP(hipEventSynchronize(e1));
-  float ms = 0;
-  LMI_HIP(hipEventElapsedTime(&ms, e0, e1));
-  *ms_per_copy = ms / repeats;
-  (void)hipEventDestroy(e0); (void)hipEventDestroy(e1);
-  (void)hipFree(a); (void)hipFree(b);
-  return LMI_OK;
+    hipLaunchKernelGGL(copy_kernel<false>, dim3(16384), dim3(256), 0, 0, (const cp_u32x4 *)m.a, (cp_u32x4 *)m.b, n);
+  LMI_HIP(hipGetLastError());
+  return m.elapsed(repeats, ms_per_copy);
 }
 
 }  // extern "C"

@@ -1,4 +1,11 @@
-// Device-wide exclusive scan in three phases over fixed 2048-item tiles:
+// Device-wide exclusive scans, two kinds.
+//
+// On the per-batch path: a single-pass scan with decoupled look-back (ScanChain,
+// scan_tile_prefix, further down) that lives inside the producing kernel, so a hop needs
+// no scan launches of its own.
+//
+// At cache-build time, where launch count does not matter: a three-phase scan over fixed
+// 2048-item tiles --
 //   1. the producer kernel writes cnt[i] and one sum per tile (tile_reduce_store),
 //   2. scan_tiles_kernel (one block) turns tile sums into tile offsets and
 //      publishes the total,

@@ -294,8 +294,7 @@ void *orc_lru_create(int64_t n_sets, int32_t ways, int64_t row_bytes) {
   c->sets = n_sets; c->ways = ways; c->row_bytes = row_bytes; c->tick = 0;
   c->keys.assign((size_t)(n_sets * ways), -1);
   c->last_use.assign((size_t)(n_sets * ways), 0);
-  c->rows.assign((size_t)(n_sets * ways * row_bytes), 0);
-  return c;
+  return c;  // the row store is set up by the first access that brings host rows
 }
 void orc_lru_destroy(void *lru) { delete (Lru *)lru; }
 
@@ -304,6 +303,8 @@ void orc_lru_access(void *lru, const int32_t *ids, int64_t n, int32_t *hit_slot,
   Lru *c = (Lru *)lru;
   const int32_t t = ++c->tick;
   const int64_t rb = c->row_bytes;
+  // policy-only use (host_rows == NULL) never pays for sets * ways * row_bytes of rows
+  if (host_rows && c->rows.empty()) c->rows.assign((size_t)(c->sets * c->ways * rb), 0);
   for (int64_t i = 0; i < n; ++i) {
     const int64_t base = ((int64_t)ids[i] % c->sets) * c->ways;
     hit_slot[i] = -1;

@@ -15,7 +15,9 @@
  * Pinning status (what independent check fixes each function):
  *   orc_philox4x32_10      Random123 known-answer vectors (3 KATs)
  *   orc_sample_positions   closed forms (deg<=f, deg=0), exact-subset
- *                          enumeration + chi-square over seeds, invariants
+ *                          enumeration + chi-square over seeds, invariants; for
+ *                          deg>f every pick against Floyd's rule stated in plain
+ *                          Python on orc_draw words (itself pinned by the KATs)
  *   orc_sample_batch       invariants against a brute-force python pass
  *                          (dict first-occurrence relabel, adjacency membership),
  *                          closed-form counter identities
@@ -25,7 +27,9 @@
  *                          model + invariants (occupancy, key uniqueness)
  *   orc_quantize/dequant   numpy float32/float16 arithmetic (IEEE, same ops)
  *   orc_f32_to_f16 etc.    numpy.float16 conversion (exhaustive over fp16)
- *   orc_gather_*           memcmp against numpy fancy indexing
+ *   orc_gather_rows        memcmp against numpy fancy indexing
+ *   orc_gather_rows_int8   numpy: hits = float32(q) * scale rounded to the row type,
+ *                          misses = the host rows, byte for byte
  */
 #ifndef LEGION_ORACLE_H
 #define LEGION_ORACLE_H
@@ -80,7 +84,9 @@ void  orc_lru_destroy(void *lru);
  * fill_slot[i] = slot a missing id was inserted into, or -1.  An id that appears
  * more than once in the batch is inserted once, by its first position.
  * If host_rows/out are non-null, also gathers: hits from the cache's own row
- * store, misses from host_rows, and copies inserted rows into the store. */
+ * store, misses from host_rows, and copies inserted rows into the store.  The
+ * store (n_sets * ways * row_bytes) is only allocated by the first call that
+ * brings host_rows; use either every call with host_rows or none. */
 void  orc_lru_access(void *lru, const int32_t *ids, int64_t n,
                      int32_t *hit_slot, int32_t *fill_slot,
                      const void *host_rows, void *out);

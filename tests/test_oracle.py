@@ -57,6 +57,34 @@ def test_long_rows_give_distinct_in_range_positions(oracle):
         assert pos.min() >= 0 and pos.max() < deg
 
 
+def python_floyd(oracle, seed, hop, node, deg, fanout):
+    """Floyd's sampling of `fanout` of `deg` positions, slot by slot, on the oracle's draw words."""
+    picks = []
+    for s in range(fanout):
+        j = deg - fanout + s
+        t = (oracle.draw(seed, hop, node, s) * (j + 1)) >> 32     # mulhi32: a position in [0, j]
+        picks.append(j if t in picks else t)
+    return picks
+
+
+@pytest.mark.parametrize("fanout", [1, 2, 5, 10, 25, 64])
+def test_long_rows_follow_floyd_pick_for_pick(oracle, fanout):
+    rng = np.random.default_rng(fanout)
+    collisions = 0
+    for _ in range(400):
+        seed = int(rng.integers(1, 2 ** 63))
+        hop, node = int(rng.integers(0, 3)), int(rng.integers(0, 2 ** 31 - 1))
+        # just above the fan-out (many collisions), moderate, and hub-sized rows
+        deg = int(rng.choice([fanout + 1, fanout + 2, 2 * fanout + 3, 1000, 100_000, 2 ** 31 - 1]))
+        want = python_floyd(oracle, seed, hop, node, deg, fanout)
+        got = oracle.sample_positions(seed, hop, node, deg, fanout)
+        assert list(got) == want
+        raw = [(oracle.draw(seed, hop, node, s) * (deg - fanout + s + 1)) >> 32 for s in range(fanout)]
+        collisions += int(raw != want)
+    if fanout >= 5:
+        assert collisions > 0    # the replacement branch was exercised
+
+
 def test_positions_depend_only_on_seed_hop_node(oracle):
     a = oracle.sample_positions(123, 1, 42, 900, 10)
     assert np.array_equal(a, oracle.sample_positions(123, 1, 42, 900, 10))
@@ -308,6 +336,47 @@ def test_gather_rows_is_fancy_indexing(oracle):
 
 
 # ------------------------------------------------------- synthetic generator
+@pytest.mark.parametrize("dtype,dim", [(np.float32, 100), (np.float16, 768), (np.float16, 6)])
+def test_gather_rows_int8_against_numpy(oracle, dtype, dim):
+    rng = np.random.default_rng(dim)
+    n_nodes, n_cached = 500, 120
+    host = (rng.standard_normal((n_nodes, dim)) * 3).astype(dtype)
+    q = rng.integers(-127, 128, (n_cached, dim)).astype(np.int8)
+    sc = np.abs(rng.standard_normal(n_cached)).astype(np.float32)
+    sc[:3] = [0.0, 2.0 ** -20, 517.25]            # a zero scale, a tiny one, a large one
+    ids = rng.integers(0, n_nodes, 900).astype(np.int32)
+    slot = np.where(rng.random(900) < 0.6, rng.integers(0, n_cached, 900), -1).astype(np.int32)
+    slot[:3] = [0, 1, 2]
+    got = oracle.gather_rows_int8(ids, slot, q, sc, host)
+    hit = slot >= 0
+    want = host[ids].copy()
+    y = q[slot[hit]].astype(np.float32) * sc[slot[hit]][:, None]     # one float32 multiply per element
+    assert y.dtype == np.float32
+    with np.errstate(over="ignore"):                                  # 127 x 517.25 is beyond fp16: inf on both sides
+        want[hit] = y.astype(dtype)                                   # round-to-nearest-even for fp16
+    assert got.dtype == host.dtype and got.tobytes() == want.tobytes()
+    assert hit.any() and (~hit).any()
+
+
+def test_lru_policy_needs_no_row_store(oracle):
+    """Without host rows the model tracks keys and ticks only (sets * ways * row_bytes is never
+    allocated), and decides exactly as it does with rows."""
+    rng = np.random.default_rng(9)
+    rows = rng.integers(0, 255, (2000, 16)).astype(np.uint8)
+    a, b = oracle.Lru(32, 4, 16), oracle.Lru(1 << 22, 8, 1 << 20)    # b would need 32 TiB of rows
+    c = oracle.Lru(32, 4, 16)
+    for _ in range(20):
+        ids = rng.choice(2000, 150, replace=False).astype(np.int32)
+        hit_a, fill_a, out = a.access(ids, rows)
+        hit_c, fill_c, none = c.access(ids)
+        assert none is None and np.array_equal(hit_a, hit_c) and np.array_equal(fill_a, fill_c)
+        assert out.tobytes() == rows[ids].tobytes()
+        b.access(ids)
+    ka, ua = a.state()
+    kc, uc = c.state()
+    assert np.array_equal(ka, kc) and np.array_equal(ua, uc)
+
+
 def test_synth_graph_properties(oracle, lmi):
     cdf = lmi.zipf_cdf(2.0, 2000, 12.0)
     assert cdf[0] == 0 and cdf[-1] == 0xFFFFFFFF and (np.diff(cdf.astype(np.int64)) >= 0).all()
