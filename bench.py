@@ -73,21 +73,53 @@ def log(msg):
     print("[bench] " + msg, file=sys.stderr, flush=True)
 
 
-def build_workload(lmi, w, seed, pipes, host_budget_gb, table=2, policy="degree"):
-    """Generate the graph, features, train set and cache; returns (server, info)."""
+def mem_available_gb():
+    """MemAvailable of the box in GB (0 when /proc/meminfo cannot be read)."""
+    try:
+        for line in open("/proc/meminfo"):
+            if line.startswith("MemAvailable:"):
+                return int(line.split()[1]) * 1024 / 1e9
+    except OSError:
+        pass
+    return 0.0
+
+
+def pinned_table(lmi, w, host_budget_gb):
+    """The feature table in pinned host memory, as large as this box allows: the full node count
+    when it fits, otherwise the largest node count whose table (a) stays under the budget -- by
+    default 70 % of the box's available RAM, the rest being for the host copy of the graph the
+    CPU baseline needs -- and (b) hipHostMalloc actually grants (the driver's limit on pinned
+    memory can be far below the RAM).  Returns (HostBuffer, n_nodes, note)."""
     np_dtype = np.float16 if w["dtype"] == "f16" else np.float32
-    esz = np.dtype(np_dtype).itemsize
-    n_nodes = w["nodes"]
+    row_bytes = w["dim"] * np.dtype(np_dtype).itemsize
+    ram_gb = mem_available_gb()
+    budget_gb = host_budget_gb if host_budget_gb > 0 else (0.70 * ram_gb if ram_gb > 0 else 64.0)
+    full_gb = w["nodes"] * row_bytes / 1e9
+    n_nodes, refused = w["nodes"], 0
+    if full_gb > budget_gb:
+        n_nodes = int(w["nodes"] * budget_gb / full_gb)
+    while True:
+        try:
+            feats = lmi.HostBuffer((n_nodes, w["dim"]), np_dtype)
+            break
+        except lmi.LegionError:
+            refused += 1
+            if n_nodes < 1000 or refused > 200:
+                raise
+            n_nodes = int(n_nodes * 0.95)   # a refusal costs nothing: step down until one is granted
     note = None
-    feat_gb = n_nodes * w["dim"] * esz / 1e9
-    if feat_gb > host_budget_gb:
-        # the feature table must fit in pinned host memory on this box
-        scale = host_budget_gb / feat_gb
-        n_nodes = int(n_nodes * scale)
-        if w["cache"][0] in ("static", "lru", "int8"):
-            w = dict(w, cache=(w["cache"][0], w["cache"][1] * scale))   # keep the cached fraction
-        note = "node count and cache budget down-scaled x%.3f so the %.0f GB feature table fits pinned host memory" % (scale, feat_gb)
+    if n_nodes != w["nodes"]:
+        note = ("box: %.0f GB RAM available, hipHostMalloc grants a %.1f GB table%s; the full table is %.0f GB, so node "
+                "count and cache budget are down-scaled x%.3f" % (
+                    ram_gb, n_nodes * row_bytes / 1e9,
+                    " (%d larger requests refused)" % refused if refused else "", full_gb, n_nodes / w["nodes"]))
         log(note)
+    return feats, n_nodes, note
+
+
+def build_inputs(lmi, w, seed, host_budget_gb, neighbours="degree"):
+    """Graph (HBM), feature table (pinned host memory) and train set of a workload."""
+    feats, n_nodes, note = pinned_table(lmi, w, host_budget_gb)
     t0 = time.time()
     if w["alpha"] is None:   # Erdos-Renyi-like: Poisson degrees, uniform neighbours
         from math import exp
@@ -100,20 +132,37 @@ def build_workload(lmi, w, seed, pipes, host_budget_gb, table=2, policy="degree"
         t[-1] = 4294967295
         cdf_u32, mode = t.astype(np.uint32), 0
     else:
-        cdf_u32, mode = lmi.zipf_cdf(w["alpha"], w["d_max"], w["mean_deg"]), 1
+        cdf_u32, mode = lmi.zipf_cdf(w["alpha"], w["d_max"], w["mean_deg"]), (0 if neighbours == "uniform" else 1)
     d_indptr, d_indices, n_edges = lmi.synth_graph(seed, cdf_u32, n_nodes, mode)
     log("graph: %d nodes, %d edges in HBM (%.1f s)" % (n_nodes, n_edges, time.time() - t0))
     t0 = time.time()
-    feats = lmi.HostBuffer((n_nodes, w["dim"]), np_dtype)
     lmi.synth_features(seed + 1, feats)
     log("features: %.2f GB in pinned host memory (%.1f s)" % (feats.nbytes / 1e9, time.time() - t0))
-    srv = lmi.Server(w["batch"], w["fanout"], w["dim"], feat_dtype=lmi.F16 if w["dtype"] == "f16" else lmi.F32,
-                     pipes=pipes, seed=seed)
-    srv.attach_graph_device(d_indptr, d_indices, n_nodes, n_edges)
-    srv.attach_features(feats)
     n_train = min(w["train"], n_nodes)
     train = lmi.synth_trainset(seed + 2, n_nodes, n_train)
-    srv.load_idset(lmi.MODE_TRAIN, train)
+    return dict(n_nodes=n_nodes, n_edges=n_edges, n_train=n_train, note=note, feats=feats, d_indptr=d_indptr,
+                d_indices=d_indices, train=train, scale=n_nodes / w["nodes"],
+                graph="%s degrees%s, %s neighbours" % (
+                    "Poisson" if w["alpha"] is None else "Zipf-Mandelbrot", "" if w["alpha"] is None else " alpha=%s" % w["alpha"],
+                    "uniform" if mode == 0 else "degree-proportional"))
+
+
+def free_inputs(lmi, inputs):
+    inputs["feats"].free()
+    for k in ("d_indptr", "d_indices"):
+        lmi.check(lmi.lib().lmi_device_free(inputs[k]))
+
+
+def build_server(lmi, w, inputs, seed, pipes, table=2, policy="degree"):
+    """A server over prepared inputs, with the workload's cache; returns (server, info)."""
+    np_dtype = np.float16 if w["dtype"] == "f16" else np.float32
+    esz = np.dtype(np_dtype).itemsize
+    n_nodes, n_train, scale = inputs["n_nodes"], inputs["n_train"], inputs["scale"]
+    srv = lmi.Server(w["batch"], w["fanout"], w["dim"], feat_dtype=lmi.F16 if w["dtype"] == "f16" else lmi.F32,
+                     pipes=pipes, seed=seed)
+    srv.attach_graph_device(inputs["d_indptr"], inputs["d_indices"], n_nodes, inputs["n_edges"])
+    srv.attach_features(inputs["feats"])
+    srv.load_idset(lmi.MODE_TRAIN, inputs["train"])
     if policy == "presampled":
         # the reference's policy: one presampling pass over the training set, rank by sampled frequency
         t0 = time.time()
@@ -123,6 +172,8 @@ def build_workload(lmi, w, seed, pipes, host_budget_gb, table=2, policy="degree"
         log("presampled one epoch (%.2f s)" % (time.time() - t0))
     t0 = time.time()
     kind, amount = w["cache"]
+    if kind in ("static", "lru", "int8"):
+        amount = amount * scale   # a down-scaled table keeps its cached fraction
     row_bytes = w["dim"] * esz
     if kind == "static":
         rows = min(n_nodes, int(amount // row_bytes))
@@ -140,10 +191,14 @@ def build_workload(lmi, w, seed, pipes, host_budget_gb, table=2, policy="degree"
     ci = srv.cache_info()
     log("cache: kind=%d rows=%d (%.2f GB) table %.2f GB (%.1f s)" % (
         ci.kind, ci.capacity_rows, ci.capacity_rows * ci.row_bytes / 1e9, ci.table_bytes / 1e9, time.time() - t0))
-    info = dict(n_nodes=n_nodes, n_edges=n_edges, n_train=n_train, note=note, feats=feats, d_indptr=d_indptr,
-                d_indices=d_indices, train=train, row_bytes=row_bytes, cache_rows=int(ci.capacity_rows),
-                cache_kind=kind)
+    info = dict(inputs, row_bytes=row_bytes, cache_rows=int(ci.capacity_rows), cache_kind=kind)
     return srv, info
+
+
+def build_workload(lmi, w, seed, pipes, host_budget_gb, table=2, policy="degree", neighbours="degree"):
+    """Generate the graph, features, train set and cache; returns (server, info)."""
+    inputs = build_inputs(lmi, w, seed, host_budget_gb, neighbours)
+    return build_server(lmi, w, inputs, seed, pipes, table, policy)
 
 
 def record_seed_plan(lmi, srv, w, info, n_batches, seed):
@@ -196,8 +251,13 @@ def cpu_baseline(lmi, srv, w, info, seed, budget_s):
         if info["cache_kind"] != "int8":
             same = same and g.features.tobytes() == out.tobytes()
         else:
-            miss = g.cache_index < 0
-            same = same and g.features[miss].tobytes() == out[miss].tobytes()
+            # misses are the host rows; hits are the oracle's codec applied to the host rows of the ids
+            # that hit (the codec works row by row, so quantising just these rows is the cached content)
+            hit = g.cache_index >= 0
+            same = same and g.features[~hit].tobytes() == out[~hit].tobytes()
+            if hit.any():
+                q, sc = orc.quantize_rows(out[hit])
+                same = same and g.features[hit].tobytes() == orc.dequant_rows(q, sc, out.dtype).tobytes()
         # threshold property of the degree-ordered static cache
         if info["cache_kind"] in ("static", "static_frac", "int8") and len(o.ids):
             deg = indptr[o.ids + 1] - indptr[o.ids]
@@ -228,6 +288,67 @@ def cpu_baseline(lmi, srv, w, info, seed, budget_s):
                 gather_rows_per_s=rows / spent), parity_ok
 
 
+def gather_variants(lmi, srv, info, w):
+    """Sweeps the memory-access choices of the feature gather on the loaded workload -- bytes per
+    lane access, lanes per row (thread per row .. wavefront per row), rows in flight per lane,
+    store policy, grid of the host-link gather -- one batch per launch on two pipes, timed by HIP
+    events inside the library.  Every variant is a tuning key; each is a different
+    move_rows_kernel<V, LPR, U, NT, HOSTLINK> instantiation, so the same run under
+    `rocprofv3 --kernel-trace --stats` (or --pmc) lists them one by one."""
+    stream = lmi.stream_create()
+    spe = -(-info["n_train"] // w["batch"])
+    rb = info["row_bytes"]
+    hit_bytes = (w["dim"] + 4 + rb + 8) if info["cache_kind"] == "int8" else 2 * rb + 8
+
+    def run(label, steps=60):
+        for i in range(3):
+            srv.run_once(None, batch_counter=i % spe, rng_seed=100 + i, pipe=i % 2, stream=stream)
+        lmi.check(lmi.lib().lmi_device_sync())
+        srv.profile_read(True)
+        srv.profile_enable(1)
+        t0 = time.perf_counter()
+        for i in range(steps):
+            srv.run_once(None, batch_counter=i % spe, rng_seed=100 + i, pipe=i % 2, stream=stream)
+        lmi.check(lmi.lib().lmi_device_sync())
+        t1 = time.perf_counter()
+        srv.profile_enable(0)
+        p = srv.profile_read(True)
+        hit_ms = p.gather_hit_ms / max(p.gather_hit_launches, 1)
+        rows = p.gather_hit_rows / max(p.gather_hit_launches, 1)
+        miss_ms = p.gather_miss_ms / max(p.gather_miss_launches, 1)
+        mrows = p.gather_miss_rows / max(p.gather_miss_launches, 1)
+        gbs = rows * hit_bytes / (hit_ms * 1e-3) / 1e9 if hit_ms else 0.0
+        print("%-68s hit %6.1f us %5.0f GB/s (%4.1f%% of 8 TB/s) | miss %6.1f us %5.1f GB/s | sample %6.1f us | %6.1f us/batch" % (
+            label, hit_ms * 1e3, gbs, gbs / 80, miss_ms * 1e3, mrows * rb / (miss_ms * 1e-3) / 1e9 if miss_ms else 0.0,
+            p.sample_ms / max(p.sample_launches, 1) * 1e3, (t1 - t0) * 1e6 / steps), flush=True)
+
+    print("feature-gather access variants, %d-byte rows, %d algorithmic bytes per hit row" % (rb, hit_bytes), flush=True)
+    run("default")
+    if info["cache_kind"] != "int8":
+        for vb in (4, 8):
+            srv.tune("gather_vector_bytes", vb)
+            run("vector %2d B per lane (lanes per row auto)" % vb)
+        srv.tune("gather_vector_bytes", 0)
+    for lpr in (1, 4, 8, 16, 32, 64):
+        srv.tune("gather_lanes_per_row", lpr)
+        run("lanes per row %2d%s" % (lpr, "  = thread per row" if lpr == 1 else "  = wavefront per row" if lpr == 64 else ""))
+    srv.tune("gather_lanes_per_row", 0)
+    for u in (2, 4, 8):
+        srv.tune("gather_unroll", u)
+        run("rows in flight per lane %d" % u)
+    srv.tune("gather_unroll", 1)
+    srv.tune("gather_nontemporal", 0)
+    run("plain (temporal) output stores")
+    srv.tune("gather_nontemporal", 1)
+    for mb in (8, 16, 64, 256):
+        srv.tune("miss_blocks", mb)
+        run("host-link gather on %3d blocks" % mb)
+    srv.tune("miss_blocks", 32)
+    srv.tune("split_miss", 0)
+    run("host-link gather on the caller's stream (no overlap)")
+    srv.tune("split_miss", 1)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -241,7 +362,18 @@ def main():
                     help="mini-batches issued together with lmi_run_group (their sampling kernels share launches)")
     ap.add_argument("--seed", type=int, default=20260101)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget (0 = skip)")
-    ap.add_argument("--host-gb", type=float, default=64.0, help="pinned host memory budget for the feature table")
+    ap.add_argument("--host-gb", type=float, default=0.0,
+                    help="pinned host memory budget for the feature table; 0 = 70 %% of the box's available RAM, "
+                         "stepping down to what hipHostMalloc grants")
+    ap.add_argument("--neighbours", default="degree", choices=["degree", "uniform"],
+                    help="how the synthetic graph draws neighbours: degree-proportional (in-degree follows the "
+                         "out-degree law, default) or uniform over the nodes")
+    ap.add_argument("--steady-steps", type=int, default=200,
+                    help="when --steps is smaller, an extra untimed-for-`value` leg of this many steps gives "
+                         "steady_state_batches_s (0 = skip)")
+    ap.add_argument("--gather-variants", action="store_true",
+                    help="instead of the benchmark line, sweep the feature gather's access patterns on this "
+                         "workload and print one line per variant")
     ap.add_argument("--table", default="rank", choices=["hash", "direct", "rank"], help="id->slot table layout")
     ap.add_argument("--policy", default="degree", choices=["degree", "presampled"],
                     help="ranking of the static hot set: out-degree (the configs' choice) or presampled frequency")
@@ -263,8 +395,14 @@ def main():
     if w["cache"][0] == "lru":
         args.group = 1                      # the LRU cache takes one batch at a time
         args.pipes = min(args.pipes, 2)
+    if args.gather_variants:
+        args.pipes = 2
     srv, info = build_workload(lmi, w, args.seed, args.pipes, args.host_gb,
-                               {"hash": 0, "direct": 1, "rank": 2}[args.table], args.policy)
+                               {"hash": 0, "direct": 1, "rank": 2}[args.table], args.policy, args.neighbours)
+    if args.gather_variants:
+        gather_variants(lmi, srv, info, w)
+        srv.close()
+        return
     tunes = {k: str(v) for k, v in w.get("tune", {}).items()}   # the workload's own settings, then --tune
     tunes.update(kv.split("=") for kv in args.tune)
     # host-link gather grid (miss_blocks, library default 32), measured on paper100m-shaped in groups
@@ -277,7 +415,8 @@ def main():
     plan = None
     if w.get("locality"):
         t0 = time.time()
-        plan = record_seed_plan(lmi, srv, w, info, args.warmup + args.steps + min(args.steps, 20), args.seed)
+        extra = args.steady_steps if args.steps < args.steady_steps else 0
+        plan = record_seed_plan(lmi, srv, w, info, args.warmup + args.steps + extra + min(args.steps, 20), args.seed)
         ci = srv.cache_info()
         srv.build_lru_cache(int(ci.n_sets), int(ci.ways))   # start the replay from an empty cache again
         log("recorded %d seed batches with temporal locality (%.1f s)" % (len(plan), time.time() - t0))
@@ -302,9 +441,12 @@ def main():
                           seeds=[plan[k] for k in ks] if plan else None, rng_seeds=[args.seed + k for k in ks],
                           stream=streams[(p // group) % len(streams)])
 
-    args.warmup = -(-args.warmup // group) * group   # whole groups, so that the timed region starts on pipe 0
-    for i in range(0, args.warmup, group):
-        step(i)
+    def run_steps(first, count):
+        """Batches first .. first+count-1 in groups (the last group may be a partial one)."""
+        for i in range(first, first + count, group):
+            step(i, min(group, first + count - i))
+
+    run_steps(0, args.warmup)
     lmi.check(lmi.lib().lmi_device_sync())
     srv.profile_read(reset=True)
     # timed region: the two gather kernels of every 4th batch carry HIP start / stop events
@@ -313,19 +455,36 @@ def main():
     srv.tune("profile_every", args.profile_every)
     srv.profile_enable(2)
     t0 = time.perf_counter()
-    for i in range(args.warmup, args.warmup + args.steps, group):
-        step(i, min(group, args.warmup + args.steps - i))   # exactly --steps batches
+    run_steps(args.warmup, args.steps)   # exactly --steps batches
+    t_issued = time.perf_counter()
     lmi.check(lmi.lib().lmi_device_sync())
     t1 = time.perf_counter()
+    srv.status()   # a batch a kernel flagged (bad seed id, scan that gave up) voids the measurement
     srv.profile_enable(0)
     prof = srv.profile_read(reset=True)
     ms_per_step = (t1 - t0) * 1e3 / args.steps
+    drain_ms = (t1 - t_issued) * 1e3   # what was still running when the last batch had been issued
+    done = args.warmup + args.steps
+    # Short runs are dominated by their tail: the last group's host-link gather has nothing to
+    # overlap with.  A longer leg of the same loop gives the rate a serving loop sustains.
+    steady = None
+    if args.steps >= args.steady_steps or args.steady_steps <= 0:
+        steady = dict(batches_s=round(args.steps / (t1 - t0), 2), steps=args.steps, drain_ms=round(drain_ms, 3),
+                      same_run_as="value")
+    else:
+        s0 = time.perf_counter()
+        run_steps(done, args.steady_steps)
+        s_issued = time.perf_counter()
+        lmi.check(lmi.lib().lmi_device_sync())
+        s1 = time.perf_counter()
+        srv.status()
+        steady = dict(batches_s=round(args.steady_steps / (s1 - s0), 2), steps=args.steady_steps,
+                      drain_ms=round((s1 - s_issued) * 1e3, 3), same_run_as=None)
+        done += args.steady_steps
     # untimed extra leg with every phase of every batch bracketed (level 1), for the per-phase breakdown only
     srv.tune("profile_every", 1)
     srv.profile_enable(1)
-    leg = -(-(args.warmup + args.steps) // group) * group
-    for i in range(leg, leg + -(-min(args.steps, 20) // group) * group, group):
-        step(i)
+    run_steps(done, -(-min(args.steps, 20) // group) * group)
     srv.profile_enable(0)
     phases = srv.profile_read(reset=True)
 
@@ -347,6 +506,13 @@ def main():
     achieved = hit_rows * hit_bytes / (hit_ms * 1e-3) / 1e9 if hit_ms > 0 else 0.0
     copy_ms = lmi.bench_copy(1 << 30, 10)
     copy_gbs = 2 * (1 << 30) / (copy_ms * 1e-3) / 1e9
+    # the plain copy kernel moving as many bytes as one launch of the hit gather does: what a launch of
+    # this size can reach at all (a launch of a few hundred MB is over before the device is warm)
+    launch_bytes = int(hit_rows * hit_bytes) // 32 * 16
+    same_copy_gbs = None
+    if launch_bytes >= 1 << 16:
+        same_ms = lmi.bench_copy(launch_bytes, 20)
+        same_copy_gbs = 2 * launch_bytes / (same_ms * 1e-3) / 1e9
     def mover(host_link):
         # the instantiation the library picks for this row size: widest lane access that divides the
         # row, smallest power-of-two lane group (8..64) that covers it
@@ -367,12 +533,20 @@ def main():
             "__half" if w["dtype"] == "f16" else "float", 32 if w["dim"] // 16 <= 32 else 64)
     else:
         hit_kernel = mover(False) + " (HBM gather of cache hits)"
+    # HBM bytes per launch as the counters saw them: not collected by this run (rocprofv3 --pmc needs runs of
+    # its own), but recorded from the same command in the file named beside it
+    traffic = recorded_traffic(args.workload) if (args.scale == 1.0 and info["scale"] == 1.0 and
+                                                  args.neighbours == "degree") else None
+    traffic_source = ("recorded: profiles/%s_hit_gather_hbm_traffic.txt (rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE of "
+                      "this command, calibrated on the copy kernel; not counted during this run)" % args.workload
+                      ) if traffic is not None else None
     roofline = dict(bound="hbm", kernel=hit_kernel, achieved=round(achieved, 1),
                     peak=HBM_PEAK_GBS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBS, 4),
-                    traffic=recorded_traffic(args.workload) if args.scale == 1.0 else None,
+                    traffic=traffic, traffic_source=traffic_source,
                     rows_per_launch=round(hit_rows, 1), batches_per_launch=hit_batches, bytes_per_row=hit_bytes,
                     avg_launch_ms=round(hit_ms, 4),
-                    measured_copy_gbs=round(copy_gbs, 1))
+                    measured_copy_gbs=round(copy_gbs, 1),
+                    same_bytes_copy_gbs=round(same_copy_gbs, 1) if same_copy_gbs else None)
     link_bytes = min(1 << 28, info["feats"].nbytes)
     link_ms = lmi.bench_host_read(info["feats"], link_bytes)
     host_link = dict(bound="host-link", kernel=mover(True) + " (host-link gather of misses)",
@@ -389,6 +563,8 @@ def main():
     out = {
         "metric": "sampled mini-batches/sec", "value": round(args.steps / (t1 - t0), 2), "unit": "batches/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),
+        "drain_ms": round(drain_ms, 3),
+        "steady_state_batches_s": steady["batches_s"] if steady else None, "steady_state": steady,
         "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int32", "feature_dtype": "fp16" if w["dtype"] == "f16" else "fp32",
         "data": "synthetic",
@@ -397,7 +573,7 @@ def main():
                    "cache": "%s, %d rows, %s id->slot table" % (info["cache_kind"], info["cache_rows"], args.table),
                    "pipes": args.pipes, "streams": args.streams, "group": group, "tune": tunes,
                    "cache_policy": args.policy,
-                   "graph": "Zipf-Mandelbrot degrees alpha=%s, degree-proportional neighbours" % w["alpha"],
+                   "graph": info["graph"],
                    "seeds": ("%d %% of a batch from the frontiers of the previous %d batches, the rest uniform from the "
                              "train set" % (w["locality"][0] * 100, w["locality"][1])) if w.get("locality")
                    else "consecutive slices of the train set",

@@ -244,6 +244,15 @@ int lmi_run_once_static(lmi_server *s, void *stream, const int32_t *seeds, int32
  * operator's event and posts the batch (engine/server.cu:356-361,377).  Any other
  * call on the same pipe waits in the same way first. */
 int lmi_batch_wait(lmi_server *s, int pipe, void *stream);
+/* What the reference answers with printf + exit(EXIT_FAILURE) (cudaCheckError,
+ * engine/memorypool.cuh:9-17; soft failures operator_impl.cu:144-151): a condition raised
+ * by a kernel of ANY batch since the server was created (or since the last call with
+ * clear != 0) -- a seed id outside [0, n_nodes) (LMI_ERR_BAD_ID; the id was skipped) or a
+ * device scan that gave up waiting (LMI_ERR_HIP; that batch is incomplete).  The kernels
+ * record it in pinned host memory, so this call reads no device memory and synchronises
+ * nothing; a condition of a batch still running shows once that batch is done.
+ * lmi_batch_wait returns the same code. */
+int lmi_server_status(lmi_server *s, int clear);
 int lmi_batch_view_get(lmi_server *s, int pipe, lmi_batch_view *out);
 /* Synchronises `stream`, copies both headers to the host, reports a bad seed id. */
 int lmi_batch_counters(lmi_server *s, int pipe, void *stream, int32_t node_counter[16],

@@ -32,7 +32,7 @@ ABI_SYMBOLS = [
     "lmi_cache_policy", "lmi_cache_build_static", "lmi_cache_build_lru", "lmi_cache_build_int8",
     "lmi_cache_info_get", "lmi_cache_dump", "lmi_op_batch_generate", "lmi_op_random_sample",
     "lmi_op_cache_lookup", "lmi_op_io_submit", "lmi_op_io_complete", "lmi_run_once",
-    "lmi_run_group", "lmi_run_once_static", "lmi_batch_wait", "lmi_batch_view_get", "lmi_batch_counters", "lmi_steps_per_epoch", "lmi_profile_enable",
+    "lmi_run_group", "lmi_run_once_static", "lmi_batch_wait", "lmi_server_status", "lmi_batch_view_get", "lmi_batch_counters", "lmi_steps_per_epoch", "lmi_profile_enable",
     "lmi_profile_read", "lmi_tune", "lmi_bench_copy", "lmi_bench_host_read", "lmi_bench_random_read", "lmi_synth_graph", "lmi_synth_trainset",
     "lmi_synth_features",
 ]
@@ -118,6 +118,7 @@ def lib():
         L.lmi_run_once.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int32, C.c_int, C.c_int32,
                                    C.c_int, C.c_uint64]
         L.lmi_batch_wait.argtypes = [C.c_void_p, C.c_int, C.c_void_p]
+        L.lmi_server_status.argtypes = [C.c_void_p, C.c_int]
         L.lmi_batch_view_get.argtypes = [C.c_void_p, C.c_int, C.POINTER(BatchView)]
         L.lmi_batch_counters.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p]
         L.lmi_run_group.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p, C.c_int,
@@ -306,6 +307,10 @@ class Server:
     # outputs -----------------------------------------------------------------
     def batch_wait(self, pipe=0, stream=None):
         check(lib().lmi_batch_wait(self.h, pipe, stream))
+
+    def status(self, clear=False):
+        """Raises if a kernel of any batch so far reported a bad seed id or a scan that gave up."""
+        check(lib().lmi_server_status(self.h, int(clear)))
 
     def counters(self, pipe=0, stream=None):
         nc = np.zeros(16, np.int32)

@@ -291,6 +291,16 @@ int lmi_server_create(const lmi_config *cfg, lmi_server **out) {
   if (rc == LMI_OK && hipEventCreateWithFlags(&s->side_idle, hipEventDisableTiming) != hipSuccess) rc = LMI_ERR_HIP;
   if (rc == LMI_OK && (hipMalloc(&s->d_prof_rows, 16) != hipSuccess || hipMemset(s->d_prof_rows, 0, 16) != hipSuccess))
     rc = LMI_ERR_HIP;
+  if (rc == LMI_OK) {  // sticky fault words: pinned host memory the kernels write and the host reads without a copy
+    void *fh = nullptr, *fd = nullptr;
+    if (hipHostMalloc(&fh, 64, hipHostMallocMapped) != hipSuccess) rc = LMI_ERR_HIP;
+    if (rc == LMI_OK) {
+      memset(fh, 0, 64);
+      s->fault_host = (volatile int32_t *)fh;
+      if (hipHostGetDevicePointer(&fd, fh, 0) != hipSuccess) rc = LMI_ERR_HIP;
+      s->fault_dev = (int32_t *)fd;
+    }
+  }
   if (rc != LMI_OK) {
     lmi_server_destroy(reinterpret_cast<lmi_server *>(s));
     return rc;
@@ -323,6 +333,7 @@ int lmi_server_destroy(lmi_server *h) {
   if (s->lru_ready) (void)hipEventDestroy(s->lru_ready);
   if (s->lru_copied) (void)hipEventDestroy(s->lru_copied);
   if (s->side_idle) (void)hipEventDestroy(s->side_idle);
+  if (s->fault_host) (void)hipHostFree((void *)s->fault_host);
   delete s;
   return LMI_OK;
 }
@@ -569,6 +580,7 @@ static int batch_params(Server *s, Pipe &p, hipStream_t st, const int32_t *seeds
   p.id_bits = id_bits;
   bp->table_tag = max_epoch > 0 ? (int32_t)((uint32_t)p.epoch << id_bits) : 0;
   bp->table_mask = max_epoch > 0 ? (int32_t)(0xFFFFFFFFu << id_bits) : kUntaggedMask;
+  bp->fault = s->fault_dev;
   bp->rng_seed = rng_seed ? rng_seed : s->cfg.seed + (uint64_t)(uint32_t)batch_counter;
   if (s->cache_kind == LMI_CACHE_LRU) ++s->lru_tick;
   bp->lru_tick = s->lru_tick;
@@ -829,10 +841,28 @@ int lmi_run_once_static(lmi_server *h, void *stream, const int32_t *seeds, int32
   return rc;
 }
 
+// What the sticky fault words say, as an error code (no device access, no synchronisation).
+static int fault_status(Server *s, int clear) {
+  if (!s->fault_host) return LMI_OK;
+  const int32_t bad = s->fault_host[kFaultBadId], scan = s->fault_host[kFaultScan];
+  if (clear) s->fault_host[kFaultBadId] = s->fault_host[kFaultScan] = 0;
+  if (scan) LMI_FAIL(LMI_ERR_HIP, "a device scan timed out waiting for an earlier tile: that batch is incomplete");
+  if (bad)
+    LMI_FAIL(LMI_ERR_BAD_ID, "a seed id outside [0, %lld) was seen on the device and skipped", (long long)s->n_nodes);
+  return LMI_OK;
+}
+
+int lmi_server_status(lmi_server *h, int clear) {
+  Server *s = reinterpret_cast<Server *>(h);
+  if (!s) LMI_FAIL(LMI_ERR_ARG, "null server");
+  return fault_status(s, clear);
+}
+
 int lmi_batch_wait(lmi_server *h, int pipe, void *stream) {
   Server *s = reinterpret_cast<Server *>(h);
   LMI_TRY(check_pipe(s, pipe));
-  return pipe_join(s->pipes[pipe], (hipStream_t)stream);
+  LMI_TRY(pipe_join(s->pipes[pipe], (hipStream_t)stream));
+  return fault_status(s, 0);
 }
 
 // ------------------------------------------------------------------ outputs
@@ -938,6 +968,9 @@ int lmi_tune(lmi_server *h, const char *key, int64_t value) {
   else if (!strcmp(key, "gather_vector_bytes")) s->gather_vec = (int)value;
   else if (!strcmp(key, "gather_blocks")) s->gather_blocks = (int)value;
   else if (!strcmp(key, "gather_nontemporal")) s->gather_nt = (int)value;
+  else if (!strcmp(key, "gather_flat")) s->gather_flat = (int)value;
+  else if (!strcmp(key, "gather_tile_rows")) s->gather_tile_rows = (int)value;
+  else if (!strcmp(key, "int8_elements_per_lane")) s->int8_epl = (int)value;
   else if (!strcmp(key, "lds_dedup")) s->lds_dedup = (int)value;
   else if (!strcmp(key, "fuse_count")) s->fuse_count = (int)value;
   else if (!strcmp(key, "protect_hits")) s->protect_hits = (int)value;

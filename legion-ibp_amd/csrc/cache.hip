@@ -100,6 +100,141 @@ static __global__ __launch_bounds__(256) void move_rows_kernel(
 
 typedef uint32_t u32x4 __attribute__((ext_vector_type(4)));
 typedef uint32_t u32x2 __attribute__((ext_vector_type(2)));
+typedef u32x4 u32x4_a4 __attribute__((aligned(4)));  // a 16-byte access at a 4-byte-aligned address
+
+// Row mover for rows that a power-of-two lane group does not fit: 400-byte rows (25 chunks of
+// 16 bytes would leave 7 of 32 lanes idle), rows that are no multiple of 16 bytes, rows whose
+// start is only 4-byte aligned.  A row is `cpr` 16-byte units followed by `tail` 4-byte units.
+// A block takes a tile of TILE consecutive work items in two steps.  Staging: one thread per
+// work item resolves it (list entry, source row, destination row: the only dependent loads)
+// and the items that have something to move -- cache hits, when the source index is the
+// cache slot -- are compacted into LDS by ballot + prefix popcount, as (source offset,
+// destination offset) pairs.  Moving: the 256 threads walk the units of the staged rows in
+// flat order, unit f = staged row f / units, place f % units inside it, offsets from LDS, so
+// every lane of every pass but the last has a unit, misses cost no lanes, and the row loads
+// of a pass depend on nothing but LDS.  Consecutive lanes touch consecutive bytes of a row,
+// and of the next row when the destination rows are contiguous.  V16 says whether the 16-byte
+// accesses may assume 16-byte alignment.  Work items, lists and index arrays mean what they
+// mean in move_rows_kernel.
+constexpr int kTileWaves = 4;  // wavefronts of a 256-thread block
+template <typename V16, int TILE, int U, bool NT, bool HOSTLINK>
+static __global__ __launch_bounds__(256) void move_rows_tiled_kernel(
+    MoveGroup g, int src_from_list, const uint8_t *src, int cpr, int tail, int tile_rows, int64_t src_row_bytes,
+    int64_t dst_row_bytes, unsigned long long *row_counter) {
+  static_assert(TILE == 64 || TILE == 256, "a tile is at most one work item per lane of one wavefront, or of the block");
+  __shared__ int64_t s_src[TILE], s_dst[TILE];
+  __shared__ int s_cnt[kTileWaves];
+  LMI_GRID_ROW(g.n);
+  const MoveRow &r = g.p[row];
+  const int2 *list = r.list;
+  const int32_t *src_index = r.src_index, *dst_index = r.dst_index;
+  uint8_t *dst = r.dst;
+  const int n = *r.n_ptr;
+  const int first = r.first_ptr ? *r.first_ptr : 0;
+  if (row_counter && bx == 0 && threadIdx.x == 0 && n > first)
+    atomicAdd(row_counter, (unsigned long long)(n - first));  // work items offered to this launch (profiling)
+  const int units = cpr + tail;
+  const int dq = 256 / units, dr = 256 % units;  // what 256 units further means in (row, place)
+  const int r0 = (int)threadIdx.x / units, u0 = (int)threadIdx.x % units;
+  const int lane = threadIdx.x & (kWave - 1), wid = threadIdx.x / kWave;
+  const int n_tiles = (n - first + tile_rows - 1) / tile_rows;  // tile_rows <= TILE
+  for (int tile = bx; tile < n_tiles; tile += gx) {
+    // ---- staging
+    bool ok = false;
+    int64_t so = 0, dof = 0;
+    if ((int)threadIdx.x < tile_rows) {
+      const int j = first + tile * tile_rows + (int)threadIdx.x;
+      if (j < n) {
+        int i = j, si;
+        if (list) {
+          const int2 pr = list[j];
+          i = pr.x;
+          si = pr.y;
+        }
+        if (!list || !src_from_list) si = src_index ? src_index[i] : i;
+        const int di = dst_index ? dst_index[i] : i;
+        ok = si >= 0 && di >= 0;
+        so = (int64_t)si * src_row_bytes;
+        dof = (int64_t)di * dst_row_bytes;
+      }
+    }
+    int n_rows;
+    if (TILE == 64) {
+      if (wid == 0) {
+        const uint64_t m = __ballot(ok);
+        if (ok) {
+          const int pos = __popcll(m & lanemask_lt());
+          s_src[pos] = so;
+          s_dst[pos] = dof;
+        }
+        if (lane == 0) s_cnt[0] = __popcll(m);
+      }
+      __syncthreads();
+      n_rows = s_cnt[0];
+    } else {
+      const uint64_t m = __ballot(ok);
+      if (lane == 0) s_cnt[wid] = __popcll(m);
+      __syncthreads();
+      int base = 0, total = 0;
+#pragma unroll
+      for (int w = 0; w < kTileWaves; ++w) {
+        const int c = s_cnt[w];
+        if (w < wid) base += c;
+        total += c;
+      }
+      if (ok) {
+        const int pos = base + __popcll(m & lanemask_lt());
+        s_src[pos] = so;
+        s_dst[pos] = dof;
+      }
+      __syncthreads();
+      n_rows = total;
+    }
+    // ---- moving
+    const int lim = n_rows * units;
+    int rr = r0, uu = u0;
+    for (int f0 = threadIdx.x; f0 < lim; f0 += 256 * U) {
+      int64_t sa[U], da[U];
+      int kind[U];  // 0: nothing, 1: 16 bytes, 2: 4 bytes
+#pragma unroll
+      for (int q = 0; q < U; ++q) {
+        kind[q] = 0;
+        if (f0 + q * 256 < lim) {
+          const int off = uu < cpr ? 16 * uu : 16 * cpr + 4 * (uu - cpr);
+          sa[q] = s_src[rr] + off;
+          da[q] = s_dst[rr] + off;
+          kind[q] = uu < cpr ? 1 : 2;
+        }
+        uu += dr;
+        rr += dq;
+        if (uu >= units) {
+          uu -= units;
+          ++rr;
+        }
+      }
+      V16 v[U];
+      uint32_t w[U];
+#pragma unroll
+      for (int q = 0; q < U; ++q) {
+        if (kind[q] == 1) v[q] = __builtin_nontemporal_load(reinterpret_cast<const V16 *>(src + sa[q]));
+        else if (kind[q] == 2) w[q] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(src + sa[q]));
+      }
+#pragma unroll
+      for (int q = 0; q < U; ++q) {
+        if (kind[q] == 1) {
+          V16 *d = reinterpret_cast<V16 *>(dst + da[q]);
+          if (NT) __builtin_nontemporal_store(v[q], d);
+          else *d = v[q];
+        } else if (kind[q] == 2) {
+          uint32_t *d = reinterpret_cast<uint32_t *>(dst + da[q]);
+          if (NT) __builtin_nontemporal_store(w[q], d);
+          else *d = w[q];
+        }
+      }
+    }
+    __syncthreads();  // the next tile's staging overwrites the offsets
+  }
+}
 
 struct MoveArgs {
   MoveGroup g;     // per pipe: work list, bounds, index arrays, destination
@@ -164,8 +299,67 @@ static int64_t auto_gather_blocks(const Server *s, int64_t want) {
   return std::min<int64_t>(std::max<int64_t>(want / 16, (int64_t)s->n_cu * 8), (int64_t)s->n_cu * 64);
 }
 
+template <typename V16, int TILE, int U>
+static void launch_tiled_vtu(hipStream_t st, const MoveArgs &a, int grid, bool nt, int cpr, int tail, int tile_rows) {
+#define LMI_TILED(NT_, HL_)                                                                                         \
+  if (a.ev_start)                                                                                                   \
+    hipExtLaunchKernelGGL((move_rows_tiled_kernel<V16, TILE, U, NT_, HL_>), dim3(grid * a.g.n), dim3(256), 0, st,    \
+                          a.ev_start, a.ev_stop, 0, a.g, a.src_from_list, a.src, cpr, tail, tile_rows,              \
+                          a.src_row_bytes, a.dst_row_bytes, a.row_counter);                                          \
+  else                                                                                                              \
+    hipLaunchKernelGGL((move_rows_tiled_kernel<V16, TILE, U, NT_, HL_>), dim3(grid * a.g.n), dim3(256), 0, st, a.g,  \
+                       a.src_from_list, a.src, cpr, tail, tile_rows, a.src_row_bytes, a.dst_row_bytes, a.row_counter)
+  if (a.host_link) {
+    LMI_TILED(true, true);
+  } else if (nt) {
+    LMI_TILED(true, false);
+  } else {
+    LMI_TILED(false, false);
+  }
+#undef LMI_TILED
+}
+
+template <typename V16, int TILE>
+static void launch_tiled_vt(hipStream_t st, const MoveArgs &a, int grid, bool nt, int cpr, int tail, int tile_rows,
+                            int unroll) {
+  if (unroll >= 4) launch_tiled_vtu<V16, TILE, 4>(st, a, grid, nt, cpr, tail, tile_rows);
+  else if (unroll >= 2) launch_tiled_vtu<V16, TILE, 2>(st, a, grid, nt, cpr, tail, tile_rows);
+  else launch_tiled_vtu<V16, TILE, 1>(st, a, grid, nt, cpr, tail, tile_rows);
+}
+
+// Rows of a tile of the tiled movers: about 8 KB of rows, so that a batch of long rows still
+// makes thousands of tiles and short tiles even out the blocks that run beside host-link reads;
+// between 2 and 64 (a wavefront stages them), or the block's 256 when rows are so short that 64
+// of them do not give every thread a unit.  Measured, share of HBM peak: 400-byte rows 16 rows
+// 47 %, 32 44 %, 64 42 %; 5 732-byte rows 2 rows 52 %, 4 48 %, 8 49 %, 16 41 %.
+static int tiled_tile_rows(Server *s, int64_t row_bytes) {
+  if (s->gather_tile_rows > 0) return std::min(s->gather_tile_rows, row_bytes < 128 ? 256 : 64);
+  if (row_bytes < 128) return 256;
+  int t = 64;
+  while (t > 2 && (int64_t)t * row_bytes > 8192) t >>= 1;
+  return t;
+}
+
+static int launch_move_rows_tiled(Server *s, hipStream_t st, const MoveArgs &a, bool nt, bool aligned16) {
+  const int cpr = (int)(a.row_bytes / 16), tail = (int)(a.row_bytes % 16) / 4;
+  const int tile = tiled_tile_rows(s, a.row_bytes);
+  const int64_t want = ceil_div(a.n_max, tile);
+  const int64_t cap = a.max_blocks > 0 ? a.max_blocks : s->gather_blocks > 0 ? s->gather_blocks : auto_gather_blocks(s, want);
+  const int grid = (int)std::max<int64_t>(1, std::min(want, cap));
+  // two units in flight per lane unless the caller or the knob says otherwise (400-byte rows: 1 -> 42 %
+  // of HBM peak, 2 -> 44 %, 4 -> 34 %)
+  const int unroll = a.unroll > 0 ? a.unroll : s->gather_unroll > 0 ? s->gather_unroll : 2;
+  if (aligned16 && tile <= 64) launch_tiled_vt<u32x4, 64>(st, a, grid, nt, cpr, tail, tile, unroll);
+  else if (aligned16) launch_tiled_vt<u32x4, 256>(st, a, grid, nt, cpr, tail, tile, unroll);
+  else if (tile <= 64) launch_tiled_vt<u32x4_a4, 64>(st, a, grid, nt, cpr, tail, tile, unroll);
+  else launch_tiled_vt<u32x4_a4, 256>(st, a, grid, nt, cpr, tail, tile, unroll);
+  LMI_HIP(hipGetLastError());
+  return LMI_OK;
+}
+
 // Picks the widest vector that divides the row and all base addresses, and a
-// power-of-two lane group that covers one row when possible.
+// power-of-two lane group that covers one row when possible; rows such a group does not
+// fit exactly go to the tiled mover.
 static int launch_move_rows(Server *s, hipStream_t st, const MoveArgs &a, bool nt) {
   if (a.n_max <= 0 || a.row_bytes <= 0) return LMI_OK;
   if (a.g.n < 1 || a.g.n > LMI_MAX_GROUP) LMI_FAIL(LMI_ERR_ARG, "a row move serves 1..LMI_MAX_GROUP pipes");
@@ -173,14 +367,22 @@ static int launch_move_rows(Server *s, hipStream_t st, const MoveArgs &a, bool n
   for (int k = 0; k < a.g.n; ++k) align |= (uintptr_t)a.g.p[k].dst;
   int vec = (align % 16 == 0) ? 16 : (align % 8 == 0) ? 8 : 4;
   if (align % 4 != 0) LMI_FAIL(LMI_ERR_ARG, "feature rows must be 4-byte aligned");
+  {
+    // a lane group fits exactly when the row is 8, 16, 32 or 64 aligned 16-byte chunks (128 .. 1024 bytes)
+    const int64_t c16 = a.row_bytes / 16;
+    const bool exact = vec == 16 && (c16 == 8 || c16 == 16 || c16 == 32 || c16 == 64);
+    const bool knobs = s->gather_vec != 0 || (s->gather_lpr != 0 && !a.host_link);  // measurement knobs of the lane-group mover
+    if (a.row_bytes >= 16 && (s->gather_flat == 1 || (s->gather_flat == 0 && !exact && !knobs)))
+      return launch_move_rows_tiled(s, st, a, nt, vec == 16);
+  }
   if (s->gather_vec == 4 || (s->gather_vec == 8 && vec == 16)) vec = s->gather_vec;  // narrower on request
   const int64_t chunks = a.row_bytes / vec;
-  int lpr = s->gather_lpr;
+  int lpr = a.host_link ? 0 : s->gather_lpr;  // the knob is about the HBM gather
   if (lpr != 1 && lpr != 4 && lpr != 8 && lpr != 16 && lpr != 32 && lpr != 64) {
     lpr = 8;
     while (lpr < chunks && lpr < 64) lpr <<= 1;
   }
-  const int unroll = a.unroll > 0 ? a.unroll : s->gather_unroll;
+  const int unroll = a.unroll > 0 ? a.unroll : s->gather_unroll > 0 ? s->gather_unroll : 1;
   const int64_t groups_per_block = 256 / lpr;
   int64_t want = ceil_div(a.n_max, groups_per_block * (unroll > 0 ? unroll : 1));
   // Many small blocks rather than one resident wave of them: blocks that run beside host-link reads
@@ -228,6 +430,25 @@ static __global__ __launch_bounds__(256) void quantize_rows_kernel(
   }
 }
 
+// y = float(q) * scale for the four int8 values packed in `w`, bit for bit what
+// __fmul_rn((float)q, scale) gives, in two instructions per element instead of three:
+// the byte, biased by 128, converts as an unsigned byte in one instruction, and one fused
+// multiply-add takes the bias out again -- (q + 128) * scale - 128 * scale is q * scale
+// exactly before the single rounding, because 128 * scale is exact (a power of two; the
+// caller takes the plain path when it would overflow).
+__device__ __forceinline__ void dequant4(uint32_t w, float sc, float bias /* -128 * sc */, bool plain, float y[4]) {
+  if (plain) {
+#pragma unroll
+    for (int e = 0; e < 4; ++e) y[e] = __fmul_rn((float)(int8_t)((w >> (e * 8)) & 0xFF), sc);
+    return;
+  }
+  const uint32_t u = w ^ 0x80808080u;
+  y[0] = __fmaf_rn((float)(u & 0xFFu), sc, bias);
+  y[1] = __fmaf_rn((float)((u >> 8) & 0xFFu), sc, bias);
+  y[2] = __fmaf_rn((float)((u >> 16) & 0xFFu), sc, bias);
+  y[3] = __fmaf_rn((float)(u >> 24), sc, bias);
+}
+
 // Dequantising gather for hits of the int8 cache, 16 elements per lane:
 // y = float(q) * scale, rounded to the output type (RNE for fp16).
 // Like the row mover, one launch serves several pipes (MoveGroup: src_index = slot per row,
@@ -250,25 +471,128 @@ static __global__ __launch_bounds__(256) void gather_int8_kernel(MoveGroup g, co
     const int slot = cache_index[i];
     if (slot < 0) continue;
     const float sc = scale[slot];
+    const bool plain = !(sc < 1.0e30f);  // 128 * scale must stay finite (also catches a NaN scale)
+    const float bias = -128.0f * sc;
     const int8_t *src = q + (int64_t)slot * dim;
     OUT *dst = out + (int64_t)i * dim;
     for (int c = lane; c < chunks; c += LPR) {
-      const u32x4 w = *reinterpret_cast<const u32x4 *>(src + c * 16);
+      const u32x4 w = __builtin_nontemporal_load(reinterpret_cast<const u32x4 *>(src + c * 16));
       union alignas(16) {
         OUT y[16];
         u32x4 v[sizeof(OUT)];
       } pk;
 #pragma unroll
-      for (int k = 0; k < 16; ++k) {
-        const int8_t b = (int8_t)((w[k >> 2] >> ((k & 3) * 8)) & 0xFF);
-        const float f = __fmul_rn((float)b, sc);
-        if constexpr (sizeof(OUT) == 2) pk.y[k] = __float2half_rn(f);
-        else pk.y[k] = f;
+      for (int k = 0; k < 4; ++k) {
+        float f[4];
+        dequant4(w[k], sc, bias, plain, f);
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+          if constexpr (sizeof(OUT) == 2) pk.y[4 * k + e] = __float2half_rn(f[e]);
+          else pk.y[4 * k + e] = f[e];
+        }
       }
       u32x4 *d4 = reinterpret_cast<u32x4 *>(dst + c * 16);
 #pragma unroll
       for (int k = 0; k < (int)sizeof(OUT); ++k) __builtin_nontemporal_store(pk.v[k], d4 + k);
     }
+  }
+}
+
+// The same gather in the shape of move_rows_tiled_kernel: the hits of a tile of 64 rows are
+// staged in LDS as (output row, slot, scale), then the block walks their EPL-element units in
+// flat order.  EPL = 16 / sizeof(OUT) makes every lane's output one 16-byte store and a
+// wavefront's store one contiguous kilobyte.  U units in flight per lane.
+template <int BYTES> struct RawVec;
+template <> struct RawVec<16> { typedef u32x4 type; };
+template <> struct RawVec<8> { typedef u32x2 type; };
+template <> struct RawVec<4> { typedef uint32_t type; };
+
+template <typename OUT, int EPL, int U>
+static __global__ __launch_bounds__(256) void gather_int8_tiled_kernel(MoveGroup g, const int8_t *q, const float *scale,
+                                                                       int dim, int tile_rows,
+                                                                       unsigned long long *row_counter) {
+  typedef typename RawVec<EPL>::type IN;
+  constexpr int OUT_VECS = EPL * (int)sizeof(OUT) / 16;
+  constexpr int TILE = 64;
+  __shared__ int s_row[TILE], s_slot[TILE];
+  __shared__ float s_scale[TILE];
+  __shared__ int s_cnt;
+  LMI_GRID_ROW(g.n);
+  const int32_t *cache_index = g.p[row].src_index;
+  OUT *out = reinterpret_cast<OUT *>(g.p[row].dst);
+  const int n = *g.p[row].n_ptr;
+  const int first = g.p[row].first_ptr ? *g.p[row].first_ptr : 0;
+  if (row_counter && bx == 0 && threadIdx.x == 0 && n > first)
+    atomicAdd(row_counter, (unsigned long long)(n - first));
+  const int units = dim / EPL;
+  const int dq = 256 / units, dr = 256 % units;
+  const int r0 = (int)threadIdx.x / units, u0 = (int)threadIdx.x % units;
+  const int n_tiles = (n - first + tile_rows - 1) / tile_rows;  // tile_rows <= TILE
+  for (int tile = bx; tile < n_tiles; tile += gx) {
+    if (threadIdx.x < TILE) {
+      const int i = first + tile * tile_rows + (int)threadIdx.x;
+      const int slot = ((int)threadIdx.x < tile_rows && i < n) ? cache_index[i] : -1;
+      const uint64_t m = __ballot(slot >= 0);
+      if (slot >= 0) {
+        const int pos = __popcll(m & lanemask_lt());
+        s_row[pos] = i;
+        s_slot[pos] = slot;
+        s_scale[pos] = scale[slot];
+      }
+      if (threadIdx.x == 0) s_cnt = __popcll(m);
+    }
+    __syncthreads();
+    const int lim = s_cnt * units;
+    int rr = r0, uu = u0;
+    for (int f0 = threadIdx.x; f0 < lim; f0 += 256 * U) {
+      int at[U], c[U];
+      bool on[U];
+#pragma unroll
+      for (int k = 0; k < U; ++k) {
+        on[k] = f0 + k * 256 < lim;
+        at[k] = rr;
+        c[k] = uu;
+        uu += dr;
+        rr += dq;
+        if (uu >= units) {
+          uu -= units;
+          ++rr;
+        }
+      }
+      union {
+        IN v;
+        uint32_t w[EPL / 4];
+      } in[U];
+#pragma unroll
+      for (int k = 0; k < U; ++k)
+        if (on[k])
+          in[k].v = __builtin_nontemporal_load(reinterpret_cast<const IN *>(q + (int64_t)s_slot[at[k]] * dim + c[k] * EPL));
+#pragma unroll
+      for (int k = 0; k < U; ++k)
+        if (on[k]) {
+          union alignas(16) {
+            OUT y[EPL];
+            u32x4 v[OUT_VECS];
+          } pk;
+          const float sc = s_scale[at[k]];
+          const bool plain = !(sc < 1.0e30f);
+          const float bias = -128.0f * sc;
+#pragma unroll
+          for (int e4 = 0; e4 < EPL / 4; ++e4) {
+            float f[4];
+            dequant4(in[k].w[e4], sc, bias, plain, f);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+              if constexpr (sizeof(OUT) == 2) pk.y[4 * e4 + e] = __float2half_rn(f[e]);
+              else pk.y[4 * e4 + e] = f[e];
+            }
+          }
+          u32x4 *d4 = reinterpret_cast<u32x4 *>(out + (int64_t)s_row[at[k]] * dim + c[k] * EPL);
+#pragma unroll
+          for (int e = 0; e < OUT_VECS; ++e) __builtin_nontemporal_store(pk.v[e], d4 + e);
+        }
+    }
+    __syncthreads();
   }
 }
 
@@ -501,17 +825,65 @@ static int launch_hits_int8(Server *s, const MoveGroup &g, hipStream_t st, int s
   else                                                                                                   \
     hipLaunchKernelGGL((KERN), dim3(grid), dim3(256), 0, st, g, q, s->cache_scale, dim, rc)
   const bool half = s->cfg.feat_dtype == LMI_F16;
-  if (dim % 16 == 0) {
-    const bool narrow = dim / 16 <= 32;
-    if (half && narrow) {
-      LMI_INT8((gather_int8_kernel<__half, 32>));
+  if (dim % 16 == 0 && s->gather_flat != 2) {
+    // elements per lane: by default as many as make one 16-byte store (8 fp16, 4 fp32)
+    int epl = s->int8_epl > 0 ? s->int8_epl : (half ? 8 : 4);
+    if (epl != 16 && epl != 8 && epl != 4) epl = half ? 8 : 4;
+    if (half && epl == 4) epl = 8;  // fewer than 16 output bytes per lane are not offered
+    // 768-element fp16 rows, share of HBM peak: 8 rows per tile 45 %, 16 51 %, 32 54 %, 64 52 %
+    const int tile_rows = s->gather_tile_rows > 0 ? std::min(64, s->gather_tile_rows) : 32;
+    const int64_t want_f = ceil_div(n_max, tile_rows);
+    const int64_t cap_f = s->gather_blocks > 0 ? s->gather_blocks : auto_gather_blocks(s, want_f);
+    const int grid_f = g.n * (int)std::max<int64_t>(1, std::min<int64_t>(want_f, cap_f));
+#define LMI_INT8_FLAT(KERN)                                                                                   \
+  if (e0)                                                                                                     \
+    hipExtLaunchKernelGGL((KERN), dim3(grid_f), dim3(256), 0, st, e0, e1, 0, g, q, s->cache_scale, dim,        \
+                          tile_rows, rc);                                                                     \
+  else                                                                                                        \
+    hipLaunchKernelGGL((KERN), dim3(grid_f), dim3(256), 0, st, g, q, s->cache_scale, dim, tile_rows, rc)
+#define LMI_INT8_FLAT_U(OUT_, EPL_)                                    \
+  if (s->gather_unroll >= 4) {                                         \
+    LMI_INT8_FLAT((gather_int8_tiled_kernel<OUT_, EPL_, 4>));           \
+  } else if (s->gather_unroll != 1) {                                  \
+    LMI_INT8_FLAT((gather_int8_tiled_kernel<OUT_, EPL_, 2>));           \
+  } else {                                                             \
+    LMI_INT8_FLAT((gather_int8_tiled_kernel<OUT_, EPL_, 1>));           \
+  }
+    if (half && epl == 16) {
+      LMI_INT8_FLAT_U(__half, 16)
     } else if (half) {
-      LMI_INT8((gather_int8_kernel<__half, 64>));
-    } else if (narrow) {
-      LMI_INT8((gather_int8_kernel<float, 32>));
+      LMI_INT8_FLAT_U(__half, 8)
+    } else if (epl == 16) {
+      LMI_INT8_FLAT_U(float, 16)
+    } else if (epl == 8) {
+      LMI_INT8_FLAT_U(float, 8)
     } else {
-      LMI_INT8((gather_int8_kernel<float, 64>));
+      LMI_INT8_FLAT_U(float, 4)
     }
+#undef LMI_INT8_FLAT_U
+#undef LMI_INT8_FLAT
+  } else if (dim % 16 == 0) {
+    // lanes per row: 16 or 32, several 16-element chunks per lane when the row is longer (768-d rows,
+    // beside the host-link gather: 64 lanes, 48 of them busy, 39 % of HBM peak; 32 lanes x 2 steps 48 %;
+    // 16 lanes x 3 steps 49 %; 8 lanes x 6 steps 46 %), or what the measurement knob asks for
+    int lpr = s->gather_lpr;
+    if (lpr != 8 && lpr != 16 && lpr != 32 && lpr != 64) lpr = dim / 16 <= 16 ? 16 : 32;
+#define LMI_INT8_L(OUT_)                                   \
+  if (lpr == 8) {                                          \
+    LMI_INT8((gather_int8_kernel<OUT_, 8>));               \
+  } else if (lpr == 16) {                                  \
+    LMI_INT8((gather_int8_kernel<OUT_, 16>));              \
+  } else if (lpr == 32) {                                  \
+    LMI_INT8((gather_int8_kernel<OUT_, 32>));              \
+  } else {                                                 \
+    LMI_INT8((gather_int8_kernel<OUT_, 64>));              \
+  }
+    if (half) {
+      LMI_INT8_L(__half)
+    } else {
+      LMI_INT8_L(float)
+    }
+#undef LMI_INT8_L
   } else if (half) {
     LMI_INT8((gather_int8_generic_kernel<__half>));
   } else {

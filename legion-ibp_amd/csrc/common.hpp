@@ -25,6 +25,7 @@ void set_error(const char *fmt, ...);
     if (e_ != hipSuccess) {                                                              \
       lmi::set_error("%s failed: %s (%s:%d)", #call, hipGetErrorString(e_), __FILE__,    \
                      __LINE__);                                                          \
+      (void)hipGetLastError(); /* reported here: a later launch check must not see it */ \
       return LMI_ERR_HIP;                                                                \
     }                                                                                    \
   } while (0)
@@ -61,7 +62,10 @@ struct DevState {
   int32_t table_tag, table_mask;  // epoch tag of this batch's dedup-table keys (table_insert_min)
   const int32_t *seeds;      // device address of this batch's seed ids
   const int32_t *labels_in;  // device address of their labels (or null)
+  int32_t *fault;            // the server's sticky fault words in pinned host memory (raise_fault), or null
 };
+
+enum { kFaultBadId = 0, kFaultScan = 1 };  // index of a condition in the server's sticky fault words
 
 struct HashSlot {  // 8-byte open-addressing slot: one 64-bit load per probe
   int32_t key;
@@ -118,6 +122,7 @@ struct BatchParams {
   uint64_t rng_seed;
   const int32_t *seeds;
   const int32_t *labels;
+  int32_t *fault;  // device-visible address of the server's sticky fault words
 };
 
 struct EventPair {  // device time between two recorded events, attributed to `kind`
@@ -170,15 +175,23 @@ struct Server {
   bool lru_pending = false;        // an insertion may still be running
   hipEvent_t lru_copied = nullptr; // recorded when the granted rows are in the cache: the next HBM gather waits for it
   bool lru_copy_pending = false;
+  // sticky fault words in pinned + mapped host memory, written by kernels, never cleared by a batch:
+  // [0] a seed id outside [0, n_nodes), [1] a look-back scan gave up
+  volatile int32_t *fault_host = nullptr;
+  int32_t *fault_dev = nullptr;  // the same words as the device addresses them
   // pipes
   std::vector<Pipe> pipes;
   hipStream_t side = nullptr;  // server-owned second stream for gathers that must not hold up the caller's stream
   // tuning
   int gather_lpr = 0;     // lanes per row (0 = auto)
   int gather_vec = 0;     // bytes per lane access (0 = widest that fits: 16)
-  int gather_unroll = 1;  // rows in flight per lane (1 measured best, a few percent ahead of 4)
+  int gather_unroll = 0;  // rows (units) in flight per lane; 0 = the mover's own best: 1 for the lane-group mover
+                          // (a few percent ahead of 4), 2 for the tiled movers
+  int gather_tile_rows = 0;  // tiled movers: rows per tile (0 = about 32 KB worth, 4..64)
   int gather_blocks = 0;  // blocks per pipe; 0 = auto (auto_gather_blocks)
   int gather_nt = 1;      // non-temporal output stores
+  int gather_flat = 0;    // 0: rows that a lane group does not fit exactly use the tiled mover; 1: every row; 2: none
+  int int8_epl = 0;       // tiled int8 gather: elements per lane (0 = one 16-byte store per lane: 8 fp16 or 4 fp32)
   int64_t fuse_small_max = 32768;  // hops of at most this many nodes use the small tile of hop_tile_nodes
   int64_t table_epochs = int64_t(1) << 30;  // batches a dedup table serves between wipes, less one (also
                                             // bounded by the key bits the node ids leave free)

@@ -34,6 +34,16 @@ __device__ __forceinline__ uint32_t sample_draw(uint64_t seed, uint32_t hop, uin
   return philox4x32_10(node, hop, slot, 0u, (uint32_t)seed, (uint32_t)(seed >> 32)).x;
 }
 
+// ------------------------------------------------------------------ faults
+// A condition the host must hear about: recorded in the batch state (read back by
+// lmi_batch_counters) and in the server's sticky fault word, which lives in pinned host
+// memory and is never cleared by a later batch, so the host sees it without reading the
+// device (lmi_server_status).
+__device__ __forceinline__ void raise_fault(DevState *st, int which) {
+  if (which == kFaultBadId) st->bad_id = 1; else st->scan_fault = 1;
+  if (st->fault) __hip_atomic_store(&st->fault[which], 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+}
+
 // -------------------------------------------------------------- hash table
 __device__ __forceinline__ uint32_t hash_id(int32_t key, int log2cap) {
   return ((uint32_t)key * 0x9E3779B1u) >> (32 - log2cap);

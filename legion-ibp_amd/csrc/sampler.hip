@@ -109,6 +109,7 @@ static __global__ __launch_bounds__(256) void batch_begin_kernel(BeginGroup g, i
     st->table_mask = bp.table_mask;
     st->seeds = bp.seeds;
     st->labels_in = bp.labels;
+    st->fault = bp.fault;
   }
 }
 
@@ -122,7 +123,7 @@ static __global__ __launch_bounds__(256) void batch_generate_kernel(int64_t n_no
   ids[i] = id;
   labels[i] = st->labels_in ? st->labels_in[i] : -1;
   if (id < 0 || id >= n_nodes) {
-    st->bad_id = 1;
+    raise_fault(st, kFaultBadId);
     return;
   }
   table_insert_min(slots, log2cap, id, i, st->table_tag, st->table_mask);
@@ -168,7 +169,7 @@ static __global__ __launch_bounds__(kScanBlock) void hop_count_scan_kernel(HopGr
           id[j] = a.ids[i];
         }
         if (id[j] < 0 || id[j] >= a.n_nodes) {
-          if (a.stage_seeds) st->bad_id = 1;
+          if (a.stage_seeds) raise_fault(st, kFaultBadId);
           id[j] = -1;
         }
       }
@@ -197,7 +198,8 @@ static __global__ __launch_bounds__(kScanBlock) void hop_count_scan_kernel(HopGr
     }
     int total;
     const int ex = block_exclusive_scan<kScanBlock>(sum, lds, total);
-    const int prefix = scan_tile_prefix(a.chain_nodes, tile, total, &s_prefix, &st->scan_fault);
+    const int prefix = scan_tile_prefix(a.chain_nodes, tile, total, &s_prefix, st);
+    if (prefix == kScanFaultPrefix) return;  // the whole block: no offset, no writes
     int run = prefix + ex;
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {
@@ -398,7 +400,7 @@ static __global__ __launch_bounds__(256) void hop_count_sample_kernel(HopGroup g
         id = a.ids[my];
       }
       if (id < 0 || id >= a.n_nodes) {
-        if (a.stage_seeds) st->bad_id = 1;
+        if (a.stage_seeds) raise_fault(st, kFaultBadId);
         id = -1;
       }
     }
@@ -413,7 +415,8 @@ static __global__ __launch_bounds__(256) void hop_count_sample_kernel(HopGroup g
     ex = inc - cnt;
     total = __shfl(inc, kWave - 1, kWave);
   }
-  const int prefix = scan_tile_prefix(a.chain_nodes, tile, total, &s_prefix, &st->scan_fault);
+  const int prefix = scan_tile_prefix(a.chain_nodes, tile, total, &s_prefix, st);
+  if (prefix == kScanFaultPrefix) return;  // the whole block: no offset, no writes
   if (t < NPB) {
     s_id[t] = id;
     s_beg[t] = lo;
@@ -509,7 +512,8 @@ static __global__ __launch_bounds__(kScanBlock) void hop_flag_scan_kernel(HopGro
     }
     int total;
     const int ex = block_exclusive_scan<kScanBlock>(sum, lds, total);
-    const int prefix = scan_tile_prefix(a.chain_edges, tile, total, &s_prefix, &st->scan_fault);
+    const int prefix = scan_tile_prefix(a.chain_edges, tile, total, &s_prefix, st);
+    if (prefix == kScanFaultPrefix) return;  // the whole block: no ranks, no writes
     int run = prefix + ex;
 #pragma unroll
     for (int j = 0; j < ITEMS; ++j) {

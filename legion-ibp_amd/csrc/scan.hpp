@@ -14,6 +14,7 @@
 #pragma once
 
 #include "device.hpp"
+#include "lookback.hpp"
 
 namespace lmi {
 
@@ -124,7 +125,12 @@ struct ScanChain {
 };
 
 constexpr unsigned long long kScanAggregate = 1ull << 32, kScanInclusive = 2ull << 32;
-constexpr int kScanSpinLimit = 1 << 16;  // look-back re-reads before a tile gives up and raises DevState::scan_fault
+// A tile that waits longer than this for an earlier tile gives up, raises DevState::scan_fault
+// (and the server's sticky fault word) and writes nothing.  Wall-clock ticks, not re-reads: a
+// legitimate wait is microseconds, whatever else shares the device (wall_clock64 counts at a
+// constant 100 MHz: a quarter of a second).  The clock is read once per 1024 re-reads.
+constexpr long long kScanWaitTicks = 25000000;
+constexpr int kScanFaultPrefix = -1;  // what scan_tile_prefix returns to a tile that gave up
 
 // Zeroes a chain for a later kernel; call from any grid with a flat thread index.
 __device__ __forceinline__ void scan_chain_reset(ScanChain c, int max_tiles, int64_t tid, int64_t n_threads) {
@@ -136,10 +142,12 @@ __device__ __forceinline__ void scan_publish(ScanChain c, int tile, unsigned lon
 }
 
 // Publishes this tile's aggregate and returns the exclusive prefix of the tile
-// (sum of all earlier tiles) to every thread of the block.  Wavefront 0 looks back
-// 64 tiles per step.  lds_prefix is one shared int.  Contains __syncthreads.
+// (sum of all earlier tiles) to every thread of the block, or kScanFaultPrefix to every
+// thread when the wait ran out: the tile then has no valid offset and must write nothing.
+// Wavefront 0 looks back 64 tiles per step (lookback_window).  lds_prefix is one shared int.
+// Contains __syncthreads.
 __device__ __forceinline__ int scan_tile_prefix(ScanChain c, int tile, int aggregate, int *lds_prefix,
-                                                int32_t *fault) {
+                                                DevState *st) {
   if (threadIdx.x < kWave) {
     const int lane = threadIdx.x;
     int prefix = 0;
@@ -149,30 +157,32 @@ __device__ __forceinline__ int scan_tile_prefix(ScanChain c, int tile, int aggre
       if (lane == 0) scan_publish(c, tile, kScanAggregate | (unsigned int)aggregate);
       int base = tile - 1;
       int spins = 0;
-      // a legitimate wait is a few hundred re-reads (one tile's worth of loads); after a first
-      // fault every later tile gives up almost at once, so a broken chain drains in milliseconds
-      const int spin_limit = *fault ? 64 : kScanSpinLimit;
+      // after a first fault every later tile gives up almost at once, so a broken chain drains
+      // in milliseconds
+      const bool broken = st->scan_fault != 0;
+      const long long t0 = wall_clock64();
       while (true) {
         const int j = base - lane;
         unsigned long long w = kScanInclusive;  // before tile 0: an inclusive prefix of 0
         if (j >= 0) w = __hip_atomic_load(&c.status[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         const unsigned flag = (unsigned)(w >> 32);
-        const unsigned long long inc = __ballot(flag == 2u), inv = __ballot(flag == 0u);
-        const int first_inc = inc ? (__ffsll((long long)inc) - 1) : (kWave - 1);
-        const unsigned long long window = (first_inc >= kWave - 1) ? ~0ull : ((1ull << (first_inc + 1)) - 1ull);
-        if (inv & window) {  // a tile we need has not published yet: read again
-          if (++spins < spin_limit) continue;
-          if (lane == 0) *fault = 1;  // never expected; bounded so that the grid always drains
+        const LookbackWindow win = lookback_window(__ballot(flag == 2u), __ballot(flag == 0u));
+        if (win.wait) {  // a tile we need has not published yet: read again
+          ++spins;
+          const bool out_of_time = broken ? spins >= 64 : ((spins & 1023) == 0 && wall_clock64() - t0 > kScanWaitTicks);
+          if (!out_of_time) continue;
+          if (lane == 0) raise_fault(st, kFaultScan);  // never expected; bounded so that the grid always drains
+          prefix = kScanFaultPrefix;
           break;
         }
-        int contrib = (lane <= first_inc) ? (int)(unsigned)w : 0;
+        int contrib = ((win.take >> lane) & 1ull) ? (int)(unsigned)w : 0;
 #pragma unroll
         for (int d = kWave / 2; d > 0; d >>= 1) contrib += __shfl_xor(contrib, d, kWave);
         prefix += contrib;
-        if (inc) break;
+        if (win.done) break;
         base -= kWave;
       }
-      if (lane == 0) scan_publish(c, tile, kScanInclusive | (unsigned int)(prefix + aggregate));
+      if (lane == 0 && prefix != kScanFaultPrefix) scan_publish(c, tile, kScanInclusive | (unsigned int)(prefix + aggregate));
     }
     if (lane == 0) *lds_prefix = prefix;
   }

@@ -178,6 +178,9 @@ class GPURunner : public Runner {
     if (handoff || !params->defer_join) LMI_MUST(lmi_batch_wait((lmi_server *)params->env, pipe_, stream_));
     if (handoff) {
       LMI_MUST(lmi_stream_sync(stream_));  // the batch is complete before the trainer is told
+      // a batch a kernel flagged (bad seed id, scan that gave up) is never handed over: stop here,
+      // as the reference stops on any device error (engine/memorypool.cuh:9-17)
+      LMI_MUST(lmi_server_status((lmi_server *)params->env, 0));
       ipc->IPCPost(device_, pipe_);
     }
   }
@@ -350,9 +353,11 @@ class GPUServer : public Server {
         sink_(&v, 0, runner_->CurrentPipe(), runner_->Stream(), sink_user_);
       }
       ++batches;
+      LMI_MUST(lmi_server_status(h_, 0));  // a host-memory read: conditions of finished batches
     }
     for (int pipe = 0; pipe < LEGION_INTERBATCH_CON; ++pipe) LMI_MUST(lmi_batch_wait(h_, pipe, runner_->Stream()));
     LMI_MUST(lmi_stream_sync(runner_->Stream()));
+    LMI_MUST(lmi_server_status(h_, 0));  // and those of the last ones
     const double sec = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
     std::printf("batches: %lld  time per sample: %.1f us  (%.1f batches/s)\n", (long long)batches,
                 batches ? sec * 1e6 / batches : 0.0, sec > 0 ? batches / sec : 0.0);

@@ -307,6 +307,44 @@ def test_bad_seed_is_reported(lmi):
         feats.free()
 
 
+def test_a_bad_seed_stays_on_record_until_cleared(lmi, oracle):
+    """The per-batch flag is wiped by the pipe's next batch; the server's own record is not: a
+    caller that never reads a batch's counters (the runner loop, a benchmark) still learns of it,
+    without touching the device."""
+    rng = np.random.default_rng(16)
+    indptr, indices = random_graph(rng, 400, 6)
+    feats = make_features(lmi, rng, 400, 8)
+    srv = lmi.Server(8, [3, 2], 8, pipes=2)
+    stream = lmi.stream_create()
+    try:
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        srv.run_once(np.array([1, 2, 3], np.int32), rng_seed=1, stream=stream)
+        srv.fetch(stream=stream)
+        srv.status()                                         # nothing on record
+        srv.batch_wait(stream=stream)
+        srv.run_once(np.array([5, 400, -7, 9], np.int32), rng_seed=2, stream=stream)   # two ids outside [0, 400)
+        lmi.check(lmi.lib().lmi_stream_sync(stream))
+        good = np.array([7, 8, 9, 10], np.int32)
+        srv.run_once(good, rng_seed=3, stream=stream)        # same pipe: wipes the per-batch flag
+        g = srv.fetch(stream=stream)                         # ... so the counters no longer complain
+        o = oracle.sample_batch(indptr, indices, good, [3, 2], 3)
+        assert np.array_equal(g.ids, o.ids)
+        with pytest.raises(lmi.LegionError) as ei:
+            srv.status()
+        assert ei.value.code == -5 and "seed id outside" in str(ei.value)
+        with pytest.raises(lmi.LegionError) as ei:
+            srv.batch_wait(stream=stream)                    # the same code where the runner joins a batch
+        assert ei.value.code == -5
+        with pytest.raises(lmi.LegionError):
+            srv.status(clear=True)                           # reports once more, then forgets
+        srv.status()
+        srv.batch_wait(stream=stream)
+    finally:
+        srv.close()
+        feats.free()
+
+
 @pytest.mark.parametrize("table", [0, 1, 2])
 @pytest.mark.parametrize("dim,dtype", [(128, np.float32), (100, np.float32), (1433, np.float32), (768, np.float16),
                                         (6, np.float16)])

@@ -94,3 +94,23 @@ def test_sampling_server_rejects_two_gpus(tmp_path):
     (tmp_path / "meta_config").write_text("/nonexistent/ 10 10 10 4 1 0 0 100 1")
     out = subprocess.run([BIN, "2", "0", "0"], cwd=str(tmp_path), timeout=60, capture_output=True, text=True)
     assert out.returncode != 0 and "one GPU" in out.stderr
+
+
+def test_sampling_server_stops_on_a_seed_outside_the_graph(tmp_path):
+    """A training set that names a node the graph does not have: the reference would abort on the
+    resulting device error (engine/memorypool.cuh:9-17); the shim exits non-zero and says why
+    instead of reporting a served epoch."""
+    rng = np.random.default_rng(77)
+    n_nodes, dim, batch, n_train = 3000, 16, 50, 160
+    data = tmp_path / "data"
+    data.mkdir()
+    indptr, indices, feats, train = write_dataset(str(data), rng, n_nodes, dim, n_train)
+    train = train.copy()
+    train[60] = n_nodes + 5          # second batch
+    train.tofile(str(data / "trainingset"))
+    (tmp_path / "meta_config").write_text("%s/ %d %d %d %d %d %d %d %d %d" % (
+        data, batch, n_nodes, len(indices), dim, n_train, 50, 40, 500 * dim * 4, 1))
+    out = subprocess.run([BIN, "1", "0", "0", "25,10"], cwd=str(tmp_path), timeout=100, capture_output=True, text=True)
+    assert out.returncode != 0, out.stdout + out.stderr
+    assert "seed id outside" in out.stderr, out.stdout + out.stderr
+    assert "batches:" not in out.stdout       # the run did not report a throughput
