@@ -442,6 +442,60 @@ def test_id_set_sliced_at_its_own_batch_size(lmi, oracle):
         feats.free()
 
 
+@pytest.mark.parametrize("cache", ["static", "int8", "lru"])
+@pytest.mark.parametrize("dim,dtype", [(128, np.float32), (100, np.float32), (768, np.float16)])
+def test_hits_come_from_hbm_and_misses_from_the_host(lmi, oracle, cache, dim, dtype):
+    """A cached fp32 row equals its host row byte for byte, so equality with the host table cannot
+    tell which copy a hit was served from.  Here every host row is overwritten AFTER the cache was
+    filled: hits must still return what was cached, misses must return the new host bytes."""
+    rng = np.random.default_rng(dim + len(cache))
+    n_nodes, batch, fanout = 6000, 200, [10, 5]
+    indptr, indices = random_graph(rng, n_nodes, 9, hubs=5, hub_deg=700)
+    feats = make_features(lmi, rng, n_nodes, dim, dtype)
+    orig = feats.array.copy()
+    srv = lmi.Server(batch, fanout, dim, feat_dtype=lmi.F16 if dtype == np.float16 else lmi.F32)
+    try:
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        seeds = rng.choice(n_nodes, batch, replace=False).astype(np.int32)
+        if cache == "lru":
+            srv.build_lru_cache(1024, 8)              # room for every row of the batches below
+            srv.run_once(seeds[:batch // 2], rng_seed=5)   # cold: every row misses and is inserted
+            first = srv.fetch()
+            assert (first.cache_index < 0).all() and first.features.tobytes() == orig[first.ids].tobytes()
+        elif cache == "static":
+            srv.build_static_cache(2000, lmi.TABLE_RANK)
+        else:
+            srv.build_int8_cache(2000, lmi.TABLE_RANK)
+        # poison: no host row keeps a single one of its bytes
+        feats.array[...] = (orig.astype(np.float32) + 100.0).astype(dtype)
+        poisoned = feats.array.copy()
+        assert not (poisoned == orig).any()
+        srv.run_once(seeds, rng_seed=5)
+        g = srv.fetch()
+        hit = g.cache_index >= 0
+        assert hit.any() and (~hit).any()
+        assert g.features[~hit].tobytes() == poisoned[g.ids[~hit]].tobytes()      # over the host link
+        if cache == "int8":
+            q, sc = oracle.quantize_rows(orig[g.ids[hit]])
+            want = oracle.dequant_rows(q, sc, dtype)
+        else:
+            want = orig[g.ids[hit]]
+        assert g.features[hit].tobytes() == want.tobytes()                          # from the copy in HBM
+        if cache == "lru":
+            # what the second batch inserted was gathered from the poisoned host rows
+            srv.run_once(seeds, rng_seed=5)
+            g3 = srv.fetch()
+            was_miss = ~hit
+            now_hit = g3.cache_index >= 0
+            assert (now_hit & was_miss).any()
+            assert g3.features[now_hit & was_miss].tobytes() == poisoned[g3.ids[now_hit & was_miss]].tobytes()
+            assert g3.features[now_hit & hit].tobytes() == orig[g3.ids[now_hit & hit]].tobytes()
+    finally:
+        srv.close()
+        feats.free()
+
+
 @pytest.mark.parametrize("n_sets,ways", [(64, 8), (16, 4), (1, 32), (500, 2)])
 def test_lru_cache_parity(lmi, oracle, n_sets, ways):
     """Reference-shaped toy workload (comp_cache/tests/test_cache.cu:4-9,48-53):

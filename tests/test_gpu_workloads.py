@@ -137,32 +137,47 @@ def test_int8_workload(lmi, oracle):
         info["feats"].free()
 
 
-def _mem_available_gb():
-    try:
-        for line in open("/proc/meminfo"):
-            if line.startswith("MemAvailable:"):
-                return int(line.split()[1]) / 1e6
-    except OSError:
-        pass
-    return 0.0
-
-
-def test_paper100m_at_full_size_in_groups_of_four(lmi, oracle):
-    """The benchmark's own configuration at its real size (111 M nodes, 1.6 B edges, 57 GB of rows in
-    pinned host memory, 38 GB cache), four batches per launch as bench.py issues them: bit-exact
-    against the oracle, plus the properties that hold at any size."""
-    if _mem_available_gb() < 90:
+@pytest.fixture(scope="module")
+def paper100m_inputs(lmi):
+    """The paper100m-shaped graph and feature table at their real size (111 M nodes, 1.6 B edges in
+    HBM, 57 GB of rows in pinned host memory), built once for the tests below, with a host copy of
+    the graph for the oracle."""
+    import bench
+    if bench.mem_available_gb() < 90:
         pytest.skip("needs about 75 GB of host memory for the feature table and a host copy of the graph")
+    w = dict(bench.WORKLOADS["paper100m"])
+    inputs = bench.build_inputs(lmi, w, 20260101, 0.0)
+    if inputs["scale"] != 1.0:
+        bench.free_inputs(lmi, inputs)
+        pytest.skip("this box does not grant the full 57 GB feature table in pinned memory")
+    inputs["indptr"] = lmi.to_host(inputs["d_indptr"], inputs["n_nodes"] + 1, np.int64)
+    inputs["indices"] = lmi.to_host(inputs["d_indices"], inputs["n_edges"], np.int32)
+    yield inputs
+    bench.free_inputs(lmi, inputs)
+
+
+def test_paper100m_at_full_size_in_groups_of_four(lmi, oracle, paper100m_inputs):
+    """The benchmark's own configuration at its real size (38 GB cache), four batches per launch as
+    bench.py issues them: bit-exact against the oracle, plus the properties that hold at any size."""
     import bench
     w = dict(bench.WORKLOADS["paper100m"])
-    srv, info = bench.build_workload(lmi, w, 20260101, 8, 64.0)
+    srv, info = bench.build_server(lmi, w, paper100m_inputs, 20260101, 8)
     stream = lmi.stream_create()
     feats = info["feats"].array
+    indptr, indices = info["indptr"], info["indices"]
     try:
-        indptr = lmi.to_host(info["d_indptr"], info["n_nodes"] + 1, np.int64)
-        indices = lmi.to_host(info["d_indices"], info["n_edges"], np.int32)
         deg = np.diff(indptr)
         B, fanout = w["batch"], w["fanout"]
+        # the hot set, ties at the threshold degree included: the lowest ids among them
+        slot = srv.cache_dump(info["n_nodes"])
+        cached = slot >= 0
+        thr = int(deg[cached].min())
+        assert int(cached.sum()) == info["cache_rows"] and (deg[~cached] <= thr).all()
+        ties = np.flatnonzero(deg == thr)
+        n_ties_in = int(cached[ties].sum())
+        assert cached[ties[:n_ties_in]].all() and not cached[ties[n_ties_in:]].any()
+        assert np.array_equal(slot[cached], np.arange(info["cache_rows"], dtype=np.int32))   # slot = rank among cached ids
+        del slot, cached, ties
         counters = [3, 4, 5, 6]
         srv.run_group([0, 1, 2, 3], counters, stream=stream)
         got = [srv.fetch(pipe=k, stream=stream) for k in range(4)]
@@ -202,4 +217,49 @@ def test_paper100m_at_full_size_in_groups_of_four(lmi, oracle):
             assert deg[g.ids][hit].min() >= deg[g.ids][~hit].max()
     finally:
         srv.close()
-        info["feats"].free()
+
+
+def test_paper100m_lru_at_full_size(lmi, oracle, paper100m_inputs):
+    """The LRU configuration at its real shape: the full 111 M-node graph, batches of 4096 seeds,
+    fan-out [15,10,5], a 20 GB 8-way LRU cache (39 M rows, 4.9 M sets), 80 % of a batch's seeds drawn
+    from the frontiers of the previous 10 batches.  Every batch bit for bit against the oracle's
+    sampler and its LRU model (policy only: the model keeps no 20 GB of rows); gathered rows against
+    the host table; the final cache state slot by slot."""
+    import bench
+    w = dict(bench.WORKLOADS["paper100m-lru"])
+    srv, info = bench.build_server(lmi, w, paper100m_inputs, 20260101, 2)
+    stream = lmi.stream_create()
+    feats = info["feats"].array
+    indptr, indices = info["indptr"], info["indices"]
+    ci = srv.cache_info()
+    assert int(ci.ways) == 8 and int(ci.capacity_rows) == 20_000_000_000 // 512 // 8 * 8
+    lru = oracle.Lru(int(ci.n_sets), int(ci.ways), 512)
+    frac, depth = w["locality"]
+    rng = np.random.default_rng(12)
+    B, train, recent = w["batch"], info["train"], []
+    hits = inserted = 0
+    try:
+        for it in range(12):
+            n_loc = int(frac * B) if recent else 0
+            parts = [train[rng.integers(0, len(train), B - n_loc)]]
+            if n_loc:
+                pool = np.concatenate(recent[-depth:])
+                parts.insert(0, pool[rng.integers(0, len(pool), n_loc)])
+            seeds = np.array(list(dict.fromkeys(np.concatenate(parts).tolist())), np.int32)   # distinct, order kept
+            srv.run_once(seeds, rng_seed=500 + it, pipe=it % 2, stream=stream)
+            g = srv.fetch(pipe=it % 2, stream=stream)
+            o = oracle.sample_batch(indptr, indices, seeds, w["fanout"], 500 + it)
+            check_batch(g, o)
+            hit, fill, _ = lru.access(o.ids)
+            assert np.array_equal(g.cache_index, hit), "hit/miss set of batch %d" % it
+            assert g.features.tobytes() == feats[o.ids].tobytes()
+            recent.append(o.ids)
+            hits += int((hit >= 0).sum())
+            inserted += int((fill >= 0).sum())
+        keys, use = srv.cache_dump(int(ci.capacity_rows), with_aux=True)
+        okeys, ouse = lru.state()
+        assert np.array_equal(keys, okeys) and np.array_equal(use, ouse)
+        assert hits > 100_000                               # the locality of the seed plan shows
+        assert inserted > int((okeys >= 0).sum())           # some insertions evicted an earlier row
+    finally:
+        srv.close()
