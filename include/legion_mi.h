@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define LMI_ABI_VERSION 1
+#define LMI_ABI_VERSION 2
 #define LMI_MAX_HOPS    3   /* the 16-int headers hold 3 hops (INTRABATCH_CON, include/system_config.cuh:47-57) */
 #define LMI_MAX_FANOUT  64  /* one wavefront lane per slot; the reference asserts <= 32 (operator_impl.cu:504) */
 #define LMI_MAX_PIPES   16  /* output buffer sets; the reference uses INTERBATCH_CON = 2 */
@@ -90,6 +90,7 @@ typedef struct lmi_batch_view {
   int32_t *blk_indptr[LMI_MAX_HOPS];  /* hop k: [n_{k-1}+1] row pointers into hop k's edge segment */
   int32_t *cache_index;               /* [max_nodes] cache slot per row, -1 = miss */
   int64_t  max_nodes, max_edges;
+  int64_t  row_bytes;                 /* bytes of one row of `features` (filled by lmi_batch_view_get) */
 } lmi_batch_view;
 
 typedef struct lmi_cache_info {
@@ -125,6 +126,20 @@ int lmi_device_alloc(size_t bytes, void **dev_ptr);            /* d_alloc_space 
 int lmi_device_free(void *dev_ptr);                            /* d_free_space */
 int lmi_copy_to_host(void *host_dst, const void *dev_src, size_t bytes);   /* d_copy_2_h (synchronous) */
 int lmi_copy_to_device(void *dev_dst, const void *host_src, size_t bytes); /* synchronous */
+/* Asynchronous device-to-device copy on `stream`. */
+int lmi_copy_device(void *dev_dst, const void *dev_src, size_t bytes, void *stream);
+/* Memory shared with another process: what the reference does with cudaIpcGetMemHandle on the
+ * sampler side (engine/ipc_service.cu:163-192) and cudaIpcOpenMemHandle on the trainer side
+ * (training_backend/ipc_cuda_kernel.cu:35-173).  lmi_ipc_export fills the 64-byte handle of the
+ * allocation that holds dev_ptr and says where in it dev_ptr lies and how large it is; an
+ * allocation of LMI_IPC_MAX_BYTES or more is refused (LMI_ERR_CAPACITY): split it.  The
+ * importing process calls lmi_ipc_open once per distinct handle, adds the offset, and closes
+ * the mapping with lmi_ipc_close before it exits. */
+#define LMI_IPC_HANDLE_BYTES 64
+#define LMI_IPC_MAX_BYTES    ((int64_t)1 << 31)
+int lmi_ipc_export(const void *dev_ptr, void *handle, int64_t *offset, int64_t *alloc_bytes);
+int lmi_ipc_open(const void *handle, void **dev_base);
+int lmi_ipc_close(void *dev_base);
 int lmi_stream_create(void **stream);
 int lmi_stream_destroy(void *stream);
 int lmi_stream_sync(void *stream);

@@ -26,7 +26,8 @@ POLICY_DEGREE, POLICY_PRESAMPLED = 0, 1
 ABI_SYMBOLS = [
     "lmi_abi_version", "lmi_last_error", "lmi_server_create", "lmi_server_destroy",
     "lmi_host_alloc", "lmi_host_free", "lmi_device_alloc", "lmi_device_free",
-    "lmi_copy_to_host", "lmi_copy_to_device", "lmi_stream_create", "lmi_stream_destroy",
+    "lmi_copy_to_host", "lmi_copy_to_device", "lmi_copy_device", "lmi_ipc_export", "lmi_ipc_open", "lmi_ipc_close",
+    "lmi_stream_create", "lmi_stream_destroy",
     "lmi_stream_sync", "lmi_device_sync", "lmi_graph_load", "lmi_features_attach",
     "lmi_idset_load", "lmi_idset_batch", "lmi_presample", "lmi_op_hotness", "lmi_presample_reset", "lmi_hotness_dump",
     "lmi_cache_policy", "lmi_cache_build_static", "lmi_cache_build_lru", "lmi_cache_build_int8",
@@ -49,7 +50,7 @@ class BatchView(C.Structure):
                 ("agg_src_ids", C.c_void_p), ("agg_src_off", C.c_void_p), ("agg_dst_off", C.c_void_p),
                 ("node_counter", C.c_void_p), ("edge_counter", C.c_void_p),
                 ("blk_indptr", C.c_void_p * MAX_HOPS), ("cache_index", C.c_void_p),
-                ("max_nodes", C.c_int64), ("max_edges", C.c_int64)]
+                ("max_nodes", C.c_int64), ("max_edges", C.c_int64), ("row_bytes", C.c_int64)]
 
 
 class CacheInfo(C.Structure):
@@ -90,6 +91,10 @@ def lib():
         L.lmi_device_free.argtypes = [C.c_void_p]
         L.lmi_copy_to_host.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
         L.lmi_copy_to_device.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t]
+        L.lmi_copy_device.argtypes = [C.c_void_p, C.c_void_p, C.c_size_t, C.c_void_p]
+        L.lmi_ipc_export.argtypes = [C.c_void_p, C.c_void_p, C.POINTER(C.c_int64), C.POINTER(C.c_int64)]
+        L.lmi_ipc_open.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+        L.lmi_ipc_close.argtypes = [C.c_void_p]
         L.lmi_stream_create.argtypes = [C.POINTER(C.c_void_p)]
         L.lmi_stream_destroy.argtypes = [C.c_void_p]
         L.lmi_stream_sync.argtypes = [C.c_void_p]

@@ -365,6 +365,37 @@ int lmi_copy_to_device(void *dev_dst, const void *host_src, size_t bytes) {
   LMI_HIP(hipMemcpy(dev_dst, host_src, bytes, hipMemcpyHostToDevice));
   return LMI_OK;
 }
+int lmi_copy_device(void *dev_dst, const void *dev_src, size_t bytes, void *stream) {
+  if (bytes) LMI_HIP(hipMemcpyAsync(dev_dst, dev_src, bytes, hipMemcpyDeviceToDevice, (hipStream_t)stream));
+  return LMI_OK;
+}
+int lmi_ipc_export(const void *dev_ptr, void *handle, int64_t *offset, int64_t *alloc_bytes) {
+  static_assert(sizeof(hipIpcMemHandle_t) == LMI_IPC_HANDLE_BYTES, "the handle slot is sized for hipIpcMemHandle_t");
+  if (!dev_ptr || !handle) LMI_FAIL(LMI_ERR_ARG, "null argument");
+  hipDeviceptr_t base = nullptr;
+  size_t size = 0;
+  LMI_HIP(hipMemGetAddressRange(&base, &size, (hipDeviceptr_t)const_cast<void *>(dev_ptr)));
+  if ((int64_t)size >= LMI_IPC_MAX_BYTES)
+    LMI_FAIL(LMI_ERR_CAPACITY, "an allocation of %zu bytes cannot be shared with another process (limit %lld): split it",
+             size, (long long)LMI_IPC_MAX_BYTES);
+  hipIpcMemHandle_t h;
+  LMI_HIP(hipIpcGetMemHandle(&h, (void *)base));
+  memcpy(handle, &h, sizeof(h));
+  if (offset) *offset = (int64_t)((const char *)dev_ptr - (const char *)base);
+  if (alloc_bytes) *alloc_bytes = (int64_t)size;
+  return LMI_OK;
+}
+int lmi_ipc_open(const void *handle, void **dev_base) {
+  if (!handle || !dev_base) LMI_FAIL(LMI_ERR_ARG, "null argument");
+  hipIpcMemHandle_t h;
+  memcpy(&h, handle, sizeof(h));
+  LMI_HIP(hipIpcOpenMemHandle(dev_base, h, hipIpcMemLazyEnablePeerAccess));
+  return LMI_OK;
+}
+int lmi_ipc_close(void *dev_base) {
+  if (dev_base) LMI_HIP(hipIpcCloseMemHandle(dev_base));
+  return LMI_OK;
+}
 int lmi_stream_create(void **stream) {
   if (!stream) LMI_FAIL(LMI_ERR_ARG, "null argument");
   hipStream_t st;
@@ -884,6 +915,7 @@ int lmi_batch_view_get(lmi_server *h, int pipe, lmi_batch_view *out) {
   out->cache_index = p.cache_index;
   out->max_nodes = s->max_nodes;
   out->max_edges = s->max_edges;
+  out->row_bytes = s->row_bytes;
   return LMI_OK;
 }
 

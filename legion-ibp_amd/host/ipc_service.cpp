@@ -15,6 +15,7 @@
 #include <unistd.h>
 
 #include <algorithm>
+#include <array>
 #include <cerrno>
 #include <cstdio>
 #include <cstdlib>
@@ -87,6 +88,7 @@ class HostIPCEnv : public IPCEnv {
     views_.assign((size_t)device_count, std::vector<lmi_batch_view>());
     semr_.assign((size_t)device_count, std::vector<sem_t *>());
     semw_.assign((size_t)device_count, std::vector<sem_t *>());
+    parts_.resize((size_t)device_count);
   }
 
   void EnableHandoff(bool on) override { handoff_ = on; }
@@ -165,11 +167,63 @@ class HostIPCEnv : public IPCEnv {
                                 int32_t pipeline_depth) override {
     (void)batch_size;
     (void)num_ids;
+    (void)feature_dim;  // the server knows the size of its rows (fp32 or fp16)
     if (!handoff_) return;
     const auto &views = views_.at((size_t)device_id);
-    for (int32_t i = 0; i < pipeline_depth && i < (int32_t)views.size(); ++i)
-      publish(device_id, i, LEGION_BUF_FEATURES, views[(size_t)i].features,
-              (uint64_t)views[(size_t)i].max_nodes * (uint64_t)feature_dim * 4);
+    // largest allocation another process can open; smaller on request, to rehearse the split on a small buffer
+    uint64_t part_limit = (uint64_t)LMI_IPC_MAX_BYTES - (1u << 24);
+    if (const char *e = std::getenv("LEGION_MI_IPC_PART_BYTES")) part_limit = std::strtoull(e, nullptr, 10);
+    for (int32_t i = 0; i < pipeline_depth && i < (int32_t)views.size(); ++i) {
+      const lmi_batch_view &v = views[(size_t)i];
+      const uint64_t row_bytes = (uint64_t)v.row_bytes, total = (uint64_t)v.max_nodes * row_bytes;
+      if (total <= part_limit) {
+        publish(device_id, i, LEGION_BUF_FEATURES, v.features, total);
+        continue;
+      }
+      // too large to share as one allocation: pieces of their own, filled by StageFeatures
+      const uint64_t rows_per_part = part_limit / row_bytes;
+      if (rows_per_part < 1) fail("LEGION_MI_IPC_PART_BYTES is smaller than one feature row");
+      const uint64_t n_parts = ((uint64_t)v.max_nodes + rows_per_part - 1) / rows_per_part;
+      if (n_parts > LEGION_MAX_FEATURE_PARTS)
+        fail("a feature buffer of " + std::to_string(total) + " bytes needs more than " +
+             std::to_string(LEGION_MAX_FEATURE_PARTS) + " shared pieces");
+      LegionBufferHandle &h = shm_->memHandle[device_id][i][LEGION_BUF_FEATURES];
+      std::memset(&h, 0, sizeof(h));
+      h.pid = (int64_t)getpid();
+      h.address = (uint64_t)(uintptr_t)v.features;
+      h.bytes = total;
+      h.n_parts = (uint32_t)n_parts;
+      h.rows_per_part = rows_per_part;
+      h.row_bytes = row_bytes;
+      for (uint64_t k = 0; k < n_parts; ++k) {
+        const uint64_t rows = std::min<uint64_t>(rows_per_part, (uint64_t)v.max_nodes - k * rows_per_part);
+        void *piece = nullptr;
+        if (lmi_device_alloc((size_t)(rows * row_bytes), &piece) != LMI_OK) fail(std::string("lmi_device_alloc: ") + lmi_last_error());
+        parts_[(size_t)device_id][(size_t)i].push_back(piece);
+        export_to(&shm_->featPart[device_id][i][k], piece, rows * row_bytes);
+      }
+      __atomic_store_n(&h.magic, LEGION_HANDLE_MAGIC, __ATOMIC_RELEASE);
+    }
+  }
+
+  bool FeaturesInParts(int32_t dev_id) const override {
+    return handoff_ && !parts_.at((size_t)dev_id)[0].empty();
+  }
+
+  void StageFeatures(int32_t dev_id, int32_t current_pipe, int64_t n_rows, void *stream) override {
+    if (!handoff_) return;
+    const int set = current_pipe % pipeline_depth_;
+    const auto &pieces = parts_.at((size_t)dev_id)[(size_t)set];
+    if (pieces.empty()) return;
+    const LegionBufferHandle &h = shm_->memHandle[dev_id][set][LEGION_BUF_FEATURES];
+    const char *src = (const char *)view(dev_id, set).features;
+    for (size_t k = 0; k < pieces.size(); ++k) {
+      const int64_t lo = (int64_t)(k * h.rows_per_part);
+      if (lo >= n_rows) break;
+      const int64_t rows = std::min<int64_t>((int64_t)h.rows_per_part, n_rows - lo);
+      if (lmi_copy_device(pieces[k], src + lo * (int64_t)h.row_bytes, (size_t)(rows * (int64_t)h.row_bytes), stream) != LMI_OK)
+        fail(std::string("lmi_copy_device: ") + lmi_last_error());
+    }
   }
 
   int32_t GetRawBatchsize() override { return raw_batch_size_; }
@@ -227,6 +281,11 @@ class HostIPCEnv : public IPCEnv {
       semr_[(size_t)d].clear();
       semw_[(size_t)d].clear();
     }
+    for (auto &dev : parts_)
+      for (auto &set : dev) {
+        for (void *piece : set) lmi_device_free(piece);
+        set.clear();
+      }
     if (shm_) {
       LegionShmClose(shm_);
       shm_unlink(LEGION_SHM_NAME);
@@ -254,11 +313,22 @@ class HostIPCEnv : public IPCEnv {
   }
 
   void publish(int32_t d, int32_t set, int which, const void *ptr, uint64_t bytes) {
-    LegionBufferHandle &h = shm_->memHandle[d][set][which];
+    export_to(&shm_->memHandle[d][set][which], ptr, bytes);
+  }
+
+  // Fills a slot with the buffer's inter-process handle (of the allocation that holds it), where
+  // the buffer lies in that allocation, and -- for a consumer inside this process -- its address.
+  void export_to(LegionBufferHandle *slot, const void *ptr, uint64_t bytes) {
+    LegionBufferHandle h;
+    std::memset(&h, 0, sizeof(h));
     h.pid = (int64_t)getpid();
     h.address = (uint64_t)(uintptr_t)ptr;
     h.bytes = bytes;
-    h.magic = LEGION_HANDLE_MAGIC;
+    int64_t offset = 0, alloc_bytes = 0;
+    if (lmi_ipc_export(ptr, h.ipc, &offset, &alloc_bytes) != LMI_OK) fail(std::string("lmi_ipc_export: ") + lmi_last_error());
+    h.offset = (uint64_t)offset;
+    *slot = h;
+    __atomic_store_n(&slot->magic, LEGION_HANDLE_MAGIC, __ATOMIC_RELEASE);  // last: the slot is complete
   }
 
   int32_t device_count_;
@@ -268,6 +338,8 @@ class HostIPCEnv : public IPCEnv {
   std::vector<lmi_server *> servers_;
   std::vector<std::vector<lmi_batch_view>> views_;
   std::vector<std::vector<sem_t *>> semr_, semw_;
+  // [device][buffer set]: separately allocated pieces of a feature buffer too large to share whole
+  std::vector<std::array<std::vector<void *>, LEGION_INTERBATCH_CON>> parts_;
   int32_t raw_batch_size_ = 0;
   std::vector<int32_t> train_batch_size_, valid_batch_size_, test_batch_size_;
   int32_t train_step_ = 0, valid_step_ = 0, test_step_ = 0;

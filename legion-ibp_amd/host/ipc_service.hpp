@@ -9,11 +9,16 @@
 // (device, buffer set, buffer), and the named semaphores sem_r_<dev>_<set> /
 // sem_w_<dev>_<set>.
 //
-// What differs: the output buffers belong to the lmi_server's pipes (BindServer), and a
-// handle slot carries {magic, process id, device address, bytes} instead of a CUDA IPC
-// memory handle, so the buffers can be opened by a consumer in the SAME process only
-// (another thread: the trainer-side class in trainer_ipc.hpp).  An empty validation or
-// test set has 0 steps (the reference computes 1 step of 0 ids).
+// What differs: the output buffers belong to the lmi_server's pipes (BindServer).  A handle
+// slot carries the 64-byte inter-process memory handle of the buffer's allocation
+// (lmi_ipc_export; the reference stores a cudaIpcMemHandle_t, engine/ipc_service.cu:163-192)
+// plus the exporting process id, the device address there, the buffer's offset inside the
+// allocation and its size: a trainer in another process opens the handle, one in the same
+// process (another thread) uses the address.  An allocation shared between processes must
+// stay under 2 GiB here, so a feature buffer of that size or more is handed over in pieces:
+// the sampler copies a finished batch's rows into up to LEGION_MAX_FEATURE_PARTS separately
+// allocated pieces (StageFeatures) and the trainer puts them together again.  An empty
+// validation or test set has 0 steps (the reference computes 1 step of 0 ids).
 #pragma once
 
 #include <semaphore.h>
@@ -35,18 +40,27 @@ enum LegionBufferIndex {  // order of the handles of one buffer set (engine/ipc_
   LEGION_BUF_AGG_DST = 4, LEGION_BUF_NODE_COUNTER = 5, LEGION_BUF_EDGE_COUNTER = 6
 };
 
-struct LegionBufferHandle {  // 64 bytes, the size of an IPC memory handle
+#define LEGION_MAX_FEATURE_PARTS 8  // pieces a feature buffer too large for one shared allocation is handed over in
+
+struct LegionBufferHandle {  // 128 bytes
   uint64_t magic;            // LEGION_HANDLE_MAGIC once exported
   int64_t pid;               // exporting process
-  uint64_t address;          // device address, valid in that process
-  uint64_t bytes;
-  uint64_t reserved[4];
+  uint64_t address;          // device address of the buffer, valid in that process
+  uint64_t bytes;            // size of the buffer
+  uint64_t offset;           // of the buffer inside the allocation the handle names
+  uint32_t n_parts;          // features only: > 0 = the rows arrive in that many pieces (featPart), not here
+  uint32_t reserved;
+  uint64_t rows_per_part;    // rows every piece but the last holds
+  uint64_t row_bytes;        // features only
+  uint8_t ipc[64];           // inter-process memory handle of the allocation (LMI_IPC_HANDLE_BYTES)
 };
-#define LEGION_HANDLE_MAGIC 0x4c4d49424e444c45ull
+#define LEGION_HANDLE_MAGIC 0x4c4d49424e444c46ull
 
 struct LegionShm {  // shmStruct (engine/ipc_service.cu:28-31)
   int32_t steps[3];
+  int32_t pad;
   LegionBufferHandle memHandle[LEGION_MAX_DEVICE][LEGION_INTERBATCH_CON][LEGION_MEMORY_USAGE];
+  LegionBufferHandle featPart[LEGION_MAX_DEVICE][LEGION_INTERBATCH_CON][LEGION_MAX_FEATURE_PARTS];
 };
 
 // The fields of the reference's BuildInfo the hand-off reads (include/buildinfo.h:6-80).
@@ -99,6 +113,11 @@ class IPCEnv {
   virtual bool HandoffEnabled() const = 0;
   // Longest IPCWait before the process gives up (the reference waits for ever).
   virtual void SetWaitSeconds(double seconds) = 0;
+  // When the feature buffer of the buffer set is handed over in pieces: copies the first n_rows
+  // rows of the set's feature buffer into them, asynchronously on `stream`; otherwise does nothing.
+  // Between the end of the batch and IPCPost.
+  virtual void StageFeatures(int32_t dev_id, int32_t current_pipe, int64_t n_rows, void *stream) = 0;
+  virtual bool FeaturesInParts(int32_t dev_id) const = 0;
 };
 
 IPCEnv *NewIPCEnv(int32_t device_count);

@@ -181,6 +181,12 @@ class GPURunner : public Runner {
       // a batch a kernel flagged (bad seed id, scan that gave up) is never handed over: stop here,
       // as the reference stops on any device error (engine/memorypool.cuh:9-17)
       LMI_MUST(lmi_server_status((lmi_server *)params->env, 0));
+      if (ipc->FeaturesInParts(device_)) {  // a feature buffer too large to share whole goes over in pieces
+        int32_t nc[16], ec[16];
+        LMI_MUST(lmi_batch_counters((lmi_server *)params->env, pipe_, stream_, nc, ec));
+        ipc->StageFeatures(device_, pipe_, nc[9 + hops_], stream_);
+        LMI_MUST(lmi_stream_sync(stream_));
+      }
       ipc->IPCPost(device_, pipe_);
     }
   }
@@ -275,6 +281,7 @@ class GPUServer : public Server {
     // schedule and hand-off (storage_management.cu builds the IPCEnv and calls Coordinate)
     ipc_ = NewIPCEnv(1);
     ipc_->EnableHandoff(handoff_ || std::getenv("LEGION_MI_HANDOFF") != nullptr);
+    if (const char *ws = std::getenv("LEGION_MI_WAIT_SECONDS")) wait_seconds_ = std::atof(ws);
     ipc_->SetWaitSeconds(wait_seconds_);
     BuildInfo info;
     info.partition_count = 1;
@@ -334,7 +341,7 @@ class GPUServer : public Server {
     lmi_cache_info ci;
     LMI_MUST(lmi_cache_info_get(h_, &ci));
     std::cout << "Cache rows: " << ci.capacity_rows << " (" << ci.capacity_rows * ci.row_bytes << " bytes)\n";
-    std::cout << "System is ready for serving\n";  // the line the reference's scripts wait for
+    std::cout << "System is ready for serving" << std::endl;  // the line the reference's scripts wait for
   }
 
   void Run() override {  // engine/server.cu:124-135

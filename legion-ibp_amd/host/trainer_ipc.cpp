@@ -1,5 +1,7 @@
-// Trainer-side end of the hand-off (see trainer_ipc.hpp).  Plain C++17 + POSIX; the only
-// device interaction is copying the two 16-int headers to the host through the C ABI.
+// Trainer-side end of the hand-off (see trainer_ipc.hpp).  Plain C++17 + POSIX; device
+// interaction goes through the C ABI: opening the sampler's buffers (lmi_ipc_open), copying
+// the two 16-int headers to the host, and putting a feature buffer that arrives in pieces
+// together again.
 #include "trainer_ipc.hpp"
 
 #include <fcntl.h>
@@ -7,6 +9,7 @@
 
 #include <cerrno>
 #include <cstring>
+#include <map>
 #include <string>
 #include <vector>
 
@@ -28,11 +31,28 @@ class HostIPCEnv : public IPCEnv {
     for (int i = 0; i < LEGION_INTERBATCH_CON; ++i) {
       for (int b = 0; b < LEGION_MEMORY_USAGE; ++b) {
         const LegionBufferHandle &h = shm_->memHandle[device][i][b];
-        if (h.magic != LEGION_HANDLE_MAGIC) return set_error("buffer set " + std::to_string(i) + " is not exported yet");
-        if (h.pid != (int64_t)getpid())
-          return set_error("the buffers were exported by process " + std::to_string(h.pid) +
-                           ": this build hands batches over inside one process");
-        buf_[i][b] = (void *)(uintptr_t)h.address;
+        if (__atomic_load_n(&h.magic, __ATOMIC_ACQUIRE) != LEGION_HANDLE_MAGIC)
+          return set_error("buffer set " + std::to_string(i) + " is not exported yet");
+        if (b == LEGION_BUF_FEATURES && h.n_parts > 0) {  // handed over in pieces
+          if (h.n_parts > LEGION_MAX_FEATURE_PARTS || h.rows_per_part == 0 || h.row_bytes == 0)
+            return set_error("the feature buffer's piece table is malformed");
+          for (uint32_t k = 0; k < h.n_parts; ++k) {
+            const LegionBufferHandle &ph = shm_->featPart[device][i][k];
+            if (__atomic_load_n(&ph.magic, __ATOMIC_ACQUIRE) != LEGION_HANDLE_MAGIC)
+              return set_error("a piece of the feature buffer is not exported yet");
+            void *piece = map_buffer(ph);
+            if (!piece) return -1;
+            part_[i][k] = piece;
+          }
+          n_parts_ = (int)h.n_parts;
+          rows_per_part_ = (int64_t)h.rows_per_part;
+          row_bytes_ = (int64_t)h.row_bytes;
+          if (!whole_ && lmi_device_alloc((size_t)h.bytes, &whole_) != LMI_OK) return set_error(lmi_last_error());
+          buf_[i][b] = whole_;
+          continue;
+        }
+        buf_[i][b] = map_buffer(h);
+        if (!buf_[i][b]) return -1;
       }
       semr_[i] = sem_open(LegionSemName('r', device, i).c_str(), O_RDWR);
       semw_[i] = sem_open(LegionSemName('w', device, i).c_str(), O_RDWR);
@@ -43,6 +63,20 @@ class HostIPCEnv : public IPCEnv {
     current_pipe_ = 0;
     ready_ = true;
     return device;
+  }
+  // The rows of a batch whose feature buffer arrives in pieces, put together in a buffer of this
+  // process; a no-op otherwise.  After Wait(), before the features are read.
+  int Assemble(int64_t n_rows) override {
+    if (n_parts_ == 0) return 0;
+    for (int k = 0; k < n_parts_; ++k) {
+      const int64_t lo = (int64_t)k * rows_per_part_;
+      if (lo >= n_rows) break;
+      const int64_t rows = std::min<int64_t>(rows_per_part_, n_rows - lo);
+      if (lmi_copy_device((char *)whole_ + lo * row_bytes_, part_[current_pipe_][k], (size_t)(rows * row_bytes_), nullptr) != LMI_OK)
+        return set_error(lmi_last_error());
+    }
+    if (lmi_stream_sync(nullptr) != LMI_OK) return set_error(lmi_last_error());
+    return 0;
   }
   int32_t *GetIds() override { return (int32_t *)buf_[current_pipe_][LEGION_BUF_IDS]; }
   float *GetFloatFeatures() override { return (float *)buf_[current_pipe_][LEGION_BUF_FEATURES]; }
@@ -55,6 +89,11 @@ class HostIPCEnv : public IPCEnv {
   int32_t GetValidStep() override { return valid_step_; }
   int32_t GetTestStep() override { return test_step_; }
   void Finalize() override {
+    for (auto &kv : opened_) lmi_ipc_close(kv.second);  // mappings of another process's allocations
+    opened_.clear();
+    if (whole_) lmi_device_free(whole_);
+    whole_ = nullptr;
+    n_parts_ = 0;
     for (int i = 0; i < LEGION_INTERBATCH_CON; ++i) {
       if (semr_[i] && semr_[i] != SEM_FAILED) sem_close(semr_[i]);
       if (semw_[i] && semw_[i] != SEM_FAILED) sem_close(semw_[i]);
@@ -81,8 +120,30 @@ class HostIPCEnv : public IPCEnv {
     error_ = e;
     return -1;
   }
+  // Address of an exported buffer in this process: the exporter's own address when that is this
+  // process, otherwise base of the opened allocation (each distinct handle is opened once: the
+  // two headers of a buffer set share an allocation) plus the buffer's offset in it.
+  void *map_buffer(const LegionBufferHandle &h) {
+    if (h.pid == (int64_t)getpid()) return (void *)(uintptr_t)h.address;
+    const std::string key((const char *)h.ipc, sizeof(h.ipc));
+    auto it = opened_.find(key);
+    if (it == opened_.end()) {
+      void *base = nullptr;
+      if (lmi_ipc_open(h.ipc, &base) != LMI_OK) {
+        set_error(std::string("cannot open a buffer of process ") + std::to_string(h.pid) + ": " + lmi_last_error());
+        return nullptr;
+      }
+      it = opened_.emplace(key, base).first;
+    }
+    return (char *)it->second + h.offset;
+  }
   LegionShm *shm_ = nullptr;
   void *buf_[LEGION_INTERBATCH_CON][LEGION_MEMORY_USAGE] = {};
+  std::map<std::string, void *> opened_;  // inter-process handle -> base address of its mapping here
+  void *part_[LEGION_INTERBATCH_CON][LEGION_MAX_FEATURE_PARTS] = {};
+  int n_parts_ = 0;
+  int64_t rows_per_part_ = 0, row_bytes_ = 0;
+  void *whole_ = nullptr;  // this process's own buffer for a feature buffer that arrives in pieces
   sem_t *semr_[LEGION_INTERBATCH_CON] = {}, *semw_[LEGION_INTERBATCH_CON] = {};
   int32_t train_step_ = 0, valid_step_ = 0, test_step_ = 0;
   int current_pipe_ = 0;
@@ -147,6 +208,10 @@ extern "C" int legion_ipc_get_next(legion_ipc_batch *out, double wait_seconds) {
   out->hop_num = hops;
   out->ids = g_env->GetIds();
   out->n_ids = g_node_counter[9 + hops];
+  if (g_env->Assemble(out->n_ids) != 0) {
+    g_error = g_env->LastError();
+    return -1;
+  }
   out->features = g_env->GetFloatFeatures();
   out->labels = g_env->GetLabels();
   out->n_labels = g_node_counter[9];

@@ -8,8 +8,9 @@
 // synchronize / finalize).  The class lives in a namespace because the sampler-side
 // class of the same name may be linked into the same process.
 //
-// The buffers must have been exported by THIS process (the sampling server runs in
-// another thread): a handle slot holds a device address, not an IPC memory handle.
+// The sampling server may run in another process (the reference's deployment: its buffers are
+// opened through the inter-process memory handles of the slab, before this process does any
+// other GPU work) or on another thread of this one (the slab's device addresses are used).
 #pragma once
 
 #include <cstdint>
@@ -37,6 +38,10 @@ class IPCEnv {
   // additions
   virtual bool TimedWait(double seconds) = 0;
   virtual const char *LastError() const = 0;
+  // After a wait: when the sampler hands the feature rows over in pieces (a buffer too large to
+  // share whole), copies the batch's n_rows rows into one buffer of this process, which
+  // GetFloatFeatures then returns.  0, or -1 with the reason in LastError().
+  virtual int Assemble(int64_t n_rows) = 0;
 };
 IPCEnv *NewIPCEnv();
 

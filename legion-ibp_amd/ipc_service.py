@@ -1,11 +1,12 @@
-"""Trainer-side consumer of the sampling server's mini-batches, in the same process.
+"""Trainer-side consumer of the sampling server's mini-batches.
 
 Same functions as the reference's `ipc_service` extension module (Legion-IBP
 training_backend/ipc_service.cpp:15-97: initialize, get_next, get_block_size, get_steps,
 synchronize, finalize; used by training_backend/legion_graphsage.py), over
-liblegion_trainer.so.  The sampling server runs on a background thread of this process
-(`start_server`), because the output buffers are handed over by device address, not by an
-inter-process memory handle.
+liblegion_trainer.so.  The sampling server is another process (the `sampling_server`
+binary with LEGION_MI_HANDOFF=1, as the reference deploys it: `initialize` opens its output
+buffers through inter-process memory handles and must come before any other GPU work of
+this process) or a background thread of this one (`start_server`).
 
     start_server(dyn_cache=0, fanout=[25, 10])      # reads ./meta_config, builds the cache
     initialize()

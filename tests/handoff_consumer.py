@@ -2,9 +2,12 @@
 a failure inside the server thread, which ends the process like the reference's error checks
 do, cannot take the test runner with it).
 
-Starts the sampling server on a background thread, consumes every batch of the reference's
-schedule through the `ipc_service` functions and checks each against the CPU oracle.
-usage: handoff_consumer.py <dataset dir> <batch> <dim> <epochs> <dyn_cache> <numpy|torch>
+Starts the sampling server on a background thread -- or, with `attach`, takes the batches of a
+`sampling_server` process that is already up (the reference's two-process deployment: the
+buffers are then opened through inter-process memory handles, before this process does any
+other GPU work) --, consumes every batch of the reference's schedule through the `ipc_service`
+functions and checks each against the CPU oracle.
+usage: handoff_consumer.py <dataset dir> <batch> <dim> <epochs> <dyn_cache> <numpy|torch> [attach]
 """
 import os
 import sys
@@ -29,7 +32,9 @@ def main():
     ipc = load_ipc_service()
     steps_ref, sizes, total = ipc.schedule(len(sets[0]), len(sets[1]), len(sets[2]), batch, epochs)
 
-    ipc.start_server(dyn_cache=dyn_cache, fanout=fanout, wait_seconds=60.0)
+    attach = len(sys.argv) > 7 and sys.argv[7] == "attach"
+    if not attach:
+        ipc.start_server(dyn_cache=dyn_cache, fanout=fanout, wait_seconds=60.0)
     ipc.initialize()
     assert ipc.get_steps() == steps_ref, (ipc.get_steps(), steps_ref)
     for g in range(total):
@@ -55,7 +60,8 @@ def main():
         assert ipc.get_block_size() == sizes_ref, (ipc.get_block_size(), sizes_ref)
         ipc.synchronize()
     ipc.finalize()
-    ipc.join_server()
+    if not attach:
+        ipc.join_server()
     print("HANDOFF_OK %d batches" % total, flush=True)
 
 

@@ -24,13 +24,13 @@ def test_library_exports_every_declared_symbol(lmi):
     missing = [s for s in declared if not hasattr(lib, s)]
     assert not missing, "declared in legion_mi.h but not exported: %s" % missing
     assert sorted(lmi.ABI_SYMBOLS) == declared, "python mirror out of sync with the header"
-    assert lib.lmi_abi_version() == 1
+    assert lib.lmi_abi_version() == 2
 
 
 def test_struct_layouts_match_header(lmi):
     # sizes computed by hand from include/legion_mi.h (LP64)
     assert ctypes.sizeof(lmi.Config) == 48
-    assert ctypes.sizeof(lmi.BatchView) == 8 * 8 + 3 * 8 + 8 + 16
+    assert ctypes.sizeof(lmi.BatchView) == 8 * 8 + 3 * 8 + 8 + 24
     assert ctypes.sizeof(lmi.CacheInfo) == 48
     assert ctypes.sizeof(lmi.Profile) == 12 * 8
 
