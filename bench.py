@@ -456,14 +456,18 @@ def main():
     srv.profile_enable(2)
     t0 = time.perf_counter()
     run_steps(args.warmup, args.steps)   # exactly --steps batches
-    t_issued = time.perf_counter()
-    lmi.check(lmi.lib().lmi_device_sync())
+    for st in streams:
+        lmi.check(lmi.lib().lmi_stream_sync(st))   # the caller's own kernels are done ...
+    t_caller = time.perf_counter()
+    lmi.check(lmi.lib().lmi_device_sync())          # ... and now the server's side stream is too
     t1 = time.perf_counter()
     srv.status()   # a batch a kernel flagged (bad seed id, scan that gave up) voids the measurement
     srv.profile_enable(0)
     prof = srv.profile_read(reset=True)
     ms_per_step = (t1 - t0) * 1e3 / args.steps
-    drain_ms = (t1 - t_issued) * 1e3   # what was still running when the last batch had been issued
+    # the tail nothing overlaps: how long the side stream (host-link gathers, LRU insertion) of the last
+    # batches kept running after the caller's stream had finished
+    drain_ms = (t1 - t_caller) * 1e3
     done = args.warmup + args.steps
     # Short runs are dominated by their tail: the last group's host-link gather has nothing to
     # overlap with.  A longer leg of the same loop gives the rate a serving loop sustains.
@@ -474,6 +478,8 @@ def main():
     else:
         s0 = time.perf_counter()
         run_steps(done, args.steady_steps)
+        for st in streams:
+            lmi.check(lmi.lib().lmi_stream_sync(st))
         s_issued = time.perf_counter()
         lmi.check(lmi.lib().lmi_device_sync())
         s1 = time.perf_counter()
@@ -514,23 +520,40 @@ def main():
         same_ms = lmi.bench_copy(launch_bytes, 20)
         same_copy_gbs = 2 * launch_bytes / (same_ms * 1e-3) / 1e9
     def mover(host_link):
-        # the instantiation the library picks for this row size: widest lane access that divides the
-        # row, smallest power-of-two lane group (8..64) that covers it
+        # the instantiation the library picks for this row size (launch_move_rows): a power-of-two lane
+        # group when the row is 8, 16, 32 or 64 aligned 16-byte chunks, the tiled mover otherwise
+        flat = int(tunes.get("miss_flat" if host_link else "gather_flat", 0))
+        knobs = int(tunes.get("gather_vector_bytes", 0)) != 0 or (not host_link and int(tunes.get("gather_lanes_per_row", 0)) != 0)
+        exact = rb % 16 == 0 and rb // 16 in (8, 16, 32, 64)
+        hl = "true" if host_link else "false"
+        if rb >= 16 and (flat == 1 or (flat == 0 and not exact and not knobs)):
+            unroll = int(tunes.get("miss_unroll", 1)) if host_link else (int(tunes.get("gather_unroll", 0)) or 2)
+            unroll = 4 if unroll >= 4 else 2 if unroll >= 2 else 1
+            return "move_rows_tiled_kernel<%s,%d,%d,true,%s>" % ("u32x4" if rb % 16 == 0 else "u32x4 at 4-byte alignment",
+                                                                 256 if rb < 128 else 64, unroll, hl)
         vec = 16 if rb % 16 == 0 else 8 if rb % 8 == 0 else 4
         narrower = int(tunes.get("gather_vector_bytes", 0))
         if narrower == 4 or (narrower == 8 and vec == 16):
             vec = narrower
-        lanes = int(tunes.get("gather_lanes_per_row", 0))
+        lanes = 0 if host_link else int(tunes.get("gather_lanes_per_row", 0))
         if lanes not in (1, 4, 8, 16, 32, 64):
             lanes = 8
             while lanes < rb // vec and lanes < 64:
                 lanes *= 2
-        unroll = int(tunes.get("miss_unroll", 1) if host_link else tunes.get("gather_unroll", 1))
-        return "move_rows_kernel<%s,%d,%d,true,%s>" % ({16: "u32x4", 8: "u32x2", 4: "u32"}[vec], lanes, unroll,
-                                                     "true" if host_link else "false")
+        unroll = int(tunes.get("miss_unroll", 1)) if host_link else (int(tunes.get("gather_unroll", 0)) or 1)
+        return "move_rows_kernel<%s,%d,%d,true,%s>" % ({16: "u32x4", 8: "u32x2", 4: "u32"}[vec], lanes, unroll, hl)
     if info["cache_kind"] == "int8":
-        hit_kernel = "gather_int8_kernel<%s,%d> (HBM gather of cache hits, dequantisation fused)" % (
-            "__half" if w["dtype"] == "f16" else "float", 32 if w["dim"] // 16 <= 32 else 64)
+        half = w["dtype"] == "f16"
+        if w["dim"] % 16 == 0 and int(tunes.get("gather_flat", 0)) != 2:
+            epl = int(tunes.get("int8_elements_per_lane", 0))
+            if epl not in (4, 8, 16) or (half and epl == 4):
+                epl = 8 if half else 4
+            unroll = int(tunes.get("gather_unroll", 0))
+            hit_kernel = "gather_int8_tiled_kernel<%s,%d,%d>" % ("__half" if half else "float", epl,
+                                                                 4 if unroll >= 4 else 1 if unroll == 1 else 2)
+        else:
+            hit_kernel = "gather_int8_kernel<%s,%d>" % ("__half" if half else "float", 16 if w["dim"] // 16 <= 16 else 32)
+        hit_kernel += " (HBM gather of cache hits, dequantisation fused)"
     else:
         hit_kernel = mover(False) + " (HBM gather of cache hits)"
     # HBM bytes per launch as the counters saw them: not collected by this run (rocprofv3 --pmc needs runs of

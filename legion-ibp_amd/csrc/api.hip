@@ -1001,6 +1001,7 @@ int lmi_tune(lmi_server *h, const char *key, int64_t value) {
   else if (!strcmp(key, "gather_blocks")) s->gather_blocks = (int)value;
   else if (!strcmp(key, "gather_nontemporal")) s->gather_nt = (int)value;
   else if (!strcmp(key, "gather_flat")) s->gather_flat = (int)value;
+  else if (!strcmp(key, "miss_flat")) s->miss_flat = (int)value;
   else if (!strcmp(key, "gather_tile_rows")) s->gather_tile_rows = (int)value;
   else if (!strcmp(key, "int8_elements_per_lane")) s->int8_epl = (int)value;
   else if (!strcmp(key, "lds_dedup")) s->lds_dedup = (int)value;

@@ -372,7 +372,8 @@ static int launch_move_rows(Server *s, hipStream_t st, const MoveArgs &a, bool n
     const int64_t c16 = a.row_bytes / 16;
     const bool exact = vec == 16 && (c16 == 8 || c16 == 16 || c16 == 32 || c16 == 64);
     const bool knobs = s->gather_vec != 0 || (s->gather_lpr != 0 && !a.host_link);  // measurement knobs of the lane-group mover
-    if (a.row_bytes >= 16 && (s->gather_flat == 1 || (s->gather_flat == 0 && !exact && !knobs)))
+    const int flat = a.host_link ? s->miss_flat : s->gather_flat;  // 0: when no lane group fits; 1: always; 2: never
+    if (a.row_bytes >= 16 && (flat == 1 || (flat == 0 && !exact && !knobs)))
       return launch_move_rows_tiled(s, st, a, nt, vec == 16);
   }
   if (s->gather_vec == 4 || (s->gather_vec == 8 && vec == 16)) vec = s->gather_vec;  // narrower on request

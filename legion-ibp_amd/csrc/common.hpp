@@ -191,6 +191,7 @@ struct Server {
   int gather_blocks = 0;  // blocks per pipe; 0 = auto (auto_gather_blocks)
   int gather_nt = 1;      // non-temporal output stores
   int gather_flat = 0;    // 0: rows that a lane group does not fit exactly use the tiled mover; 1: every row; 2: none
+  int miss_flat = 0;      // the same choice for the host-link gather
   int int8_epl = 0;       // tiled int8 gather: elements per lane (0 = one 16-byte store per lane: 8 fp16 or 4 fp32)
   int64_t fuse_small_max = 32768;  // hops of at most this many nodes use the small tile of hop_tile_nodes
   int64_t table_epochs = int64_t(1) << 30;  // batches a dedup table serves between wipes, less one (also
