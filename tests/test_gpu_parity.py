@@ -288,6 +288,67 @@ def test_duplicate_seeds_and_isolated_nodes(lmi, oracle):
         feats.free()
 
 
+@pytest.mark.parametrize("cache", ["static", "int8", "lru", "none"])
+def test_empty_and_one_seed_batches_between_full_ones(lmi, oracle, cache):
+    """Ragged use: an empty batch, a batch of one isolated seed and a batch of one hub, alone and
+    inside a group with full batches; the caches and the pipes carry on as if nothing had happened."""
+    rng = np.random.default_rng(41)
+    n_nodes, dim, fanout = 3000, 32, [6, 5]
+    indptr, indices = random_graph(rng, n_nodes, 8, hubs=3, hub_deg=900, zero_frac=0.2)
+    deg = np.diff(indptr)
+    feats = make_features(lmi, rng, n_nodes, dim)
+    srv = lmi.Server(64, fanout, dim, pipes=4)
+    stream = lmi.stream_create()
+    lru = oracle.Lru(64, 4, dim * 4)
+    host_rows = feats.array.view(np.uint8).reshape(n_nodes, dim * 4)
+    try:
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        if cache == "static":
+            srv.build_static_cache(800, lmi.TABLE_RANK)
+            slot = oracle.static_cache_build(indptr, 800)
+        elif cache == "int8":
+            srv.build_int8_cache(800, lmi.TABLE_HASH)
+            slot = oracle.static_cache_build(indptr, 800)
+            q, sc = oracle.quantize_rows(feats.array[np.flatnonzero(slot >= 0)])
+        elif cache == "lru":
+            srv.build_lru_cache(64, 4)
+        full = lambda: rng.choice(n_nodes, 64, replace=False).astype(np.int32)
+        isolated = np.array([int(np.flatnonzero(deg == 0)[0])], np.int32)
+        hub = np.array([int(np.argmax(deg))], np.int32)
+        batches = [full(), np.zeros(0, np.int32), isolated, full(), hub, np.zeros(0, np.int32), full()]
+
+        def check(g, seeds, rng_seed):
+            o = oracle.sample_batch(indptr, indices, seeds, fanout, rng_seed)
+            assert_batch_equal(g, o)
+            if cache in ("static", "int8"):
+                assert np.array_equal(g.cache_index, slot[o.ids])
+            if cache == "int8":
+                want = oracle.gather_rows_int8(o.ids, slot[o.ids], q, sc, feats.array)
+            elif cache == "lru":
+                hit, _, want = lru.access(o.ids, host_rows)
+                assert np.array_equal(g.cache_index, hit)
+            else:
+                want = feats.array[o.ids]
+            assert g.features.tobytes() == want.tobytes()
+            if len(seeds) == 0:
+                assert g.n_nodes == [0, 0, 0] and g.n_edges == [0, 0] and len(g.ids) == 0
+
+        for t, seeds in enumerate(batches):          # one after the other
+            srv.run_once(seeds, rng_seed=60 + t, pipe=t % 4, stream=stream)
+            check(srv.fetch(pipe=t % 4, stream=stream), seeds, 60 + t)
+        if cache != "lru":                           # and four at a time, the empty ones among them
+            for first in (0, 3):
+                group = batches[first:first + 4]
+                srv.run_group([0, 1, 2, 3], [0] * 4, seeds=group, rng_seeds=[80 + first + k for k in range(4)], stream=stream)
+                for k, seeds in enumerate(group):
+                    check(srv.fetch(pipe=k, stream=stream), seeds, 80 + first + k)
+        srv.status()
+    finally:
+        srv.close()
+        feats.free()
+
+
 def test_bad_seed_is_reported(lmi):
     rng = np.random.default_rng(6)
     indptr, indices = random_graph(rng, 100, 5)
