@@ -515,10 +515,12 @@ def main():
     # the plain copy kernel moving as many bytes as one launch of the hit gather does: what a launch of
     # this size can reach at all (a launch of a few hundred MB is over before the device is warm)
     launch_bytes = int(hit_rows * hit_bytes) // 32 * 16
-    same_copy_gbs = None
+    same_copy_gbs = same_launch_gbs = None
     if launch_bytes >= 1 << 16:
-        same_ms = lmi.bench_copy(launch_bytes, 20)
+        same_ms = lmi.bench_copy(launch_bytes, 20)                 # back to back: launches overlap their ramps
         same_copy_gbs = 2 * launch_bytes / (same_ms * 1e-3) / 1e9
+        same_ms = lmi.bench_copy_launch(launch_bytes, 20)          # launch by launch, timed as the gather is
+        same_launch_gbs = 2 * launch_bytes / (same_ms * 1e-3) / 1e9
     def mover(host_link):
         # the instantiation the library picks for this row size (launch_move_rows): a power-of-two lane
         # group when the row is 8, 16, 32 or 64 aligned 16-byte chunks, the tiled mover otherwise
@@ -569,7 +571,8 @@ def main():
                     rows_per_launch=round(hit_rows, 1), batches_per_launch=hit_batches, bytes_per_row=hit_bytes,
                     avg_launch_ms=round(hit_ms, 4),
                     measured_copy_gbs=round(copy_gbs, 1),
-                    same_bytes_copy_gbs=round(same_copy_gbs, 1) if same_copy_gbs else None)
+                    same_bytes_copy_gbs=round(same_copy_gbs, 1) if same_copy_gbs else None,
+                    same_bytes_copy_single_launch_gbs=round(same_launch_gbs, 1) if same_launch_gbs else None)
     link_bytes = min(1 << 28, info["feats"].nbytes)
     link_ms = lmi.bench_host_read(info["feats"], link_bytes)
     host_link = dict(bound="host-link", kernel=mover(True) + " (host-link gather of misses)",

@@ -289,6 +289,11 @@ int lmi_tune(lmi_server *s, const char *key, int64_t value);
 /* Plain device copy of `bytes` bytes, repeated; returns mean ms per copy
  * (the measured HBM ceiling quoted beside the nominal peak). */
 int lmi_bench_copy(size_t bytes, int repeats, double *ms_per_copy);
+/* The same copy timed launch by launch: every launch starts on an idle device and is timed from
+ * its own first to its own last wavefront (the start / stop events of the launch itself), which
+ * is how the gather kernels are timed.  What a launch of this size can reach at all: a launch of
+ * a few hundred MB spends a visible part of its time filling and draining the device. */
+int lmi_bench_copy_launch(size_t bytes, int repeats, double *ms_per_launch);
 /* Streaming zero-copy read of `bytes` bytes of pinned host memory (from lmi_host_alloc) into
  * HBM, repeated; returns mean ms per pass (the measured host-link ceiling). */
 int lmi_bench_host_read(const void *host_ptr, size_t bytes, int repeats, double *ms_per_pass);

@@ -34,7 +34,7 @@ ABI_SYMBOLS = [
     "lmi_cache_info_get", "lmi_cache_dump", "lmi_op_batch_generate", "lmi_op_random_sample",
     "lmi_op_cache_lookup", "lmi_op_io_submit", "lmi_op_io_complete", "lmi_run_once",
     "lmi_run_group", "lmi_run_once_static", "lmi_batch_wait", "lmi_server_status", "lmi_batch_view_get", "lmi_batch_counters", "lmi_steps_per_epoch", "lmi_profile_enable",
-    "lmi_profile_read", "lmi_tune", "lmi_bench_copy", "lmi_bench_host_read", "lmi_bench_random_read", "lmi_synth_graph", "lmi_synth_trainset",
+    "lmi_profile_read", "lmi_tune", "lmi_bench_copy", "lmi_bench_copy_launch", "lmi_bench_host_read", "lmi_bench_random_read", "lmi_synth_graph", "lmi_synth_trainset",
     "lmi_synth_features",
 ]
 
@@ -135,6 +135,7 @@ def lib():
         L.lmi_profile_read.argtypes = [C.c_void_p, C.POINTER(Profile), C.c_int]
         L.lmi_tune.argtypes = [C.c_void_p, C.c_char_p, C.c_int64]
         L.lmi_bench_copy.argtypes = [C.c_size_t, C.c_int, C.POINTER(C.c_double)]
+        L.lmi_bench_copy_launch.argtypes = [C.c_size_t, C.c_int, C.POINTER(C.c_double)]
         L.lmi_bench_host_read.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.POINTER(C.c_double)]
         L.lmi_bench_random_read.argtypes = [C.c_void_p, C.c_size_t, C.c_int64, C.c_int, C.POINTER(C.c_double)]
         L.lmi_synth_graph.argtypes = [C.c_uint64, C.c_void_p, C.c_int32, C.c_int64, C.c_int32,
@@ -373,6 +374,13 @@ class Server:
 def bench_copy(nbytes, repeats=10):
     ms = C.c_double()
     check(lib().lmi_bench_copy(nbytes, repeats, C.byref(ms)))
+    return ms.value
+
+
+def bench_copy_launch(nbytes, repeats=10):
+    """Mean ms of one copy launch of nbytes, each launch alone on the device and timed by its own events."""
+    ms = C.c_double()
+    check(lib().lmi_bench_copy_launch(nbytes, repeats, C.byref(ms)))
     return ms.value
 
 

@@ -6,6 +6,8 @@
 #include <mutex>
 #include <new>
 
+#include <hip/hip_ext.h>
+
 #include "common.hpp"
 
 namespace lmi {
@@ -1112,6 +1114,30 @@ int lmi_bench_copy(size_t bytes, int repeats, double *ms_per_copy) {
     hipLaunchKernelGGL(copy_kernel<false>, dim3(16384), dim3(256), 0, 0, (const cp_u32x4 *)m.a, (cp_u32x4 *)m.b, n);
   LMI_HIP(hipGetLastError());
   return m.elapsed(repeats, ms_per_copy);
+}
+
+int lmi_bench_copy_launch(size_t bytes, int repeats, double *ms_per_launch) {
+  if (!ms_per_launch || repeats < 1 || bytes < 16) LMI_FAIL(LMI_ERR_ARG, "bad argument");
+  BenchScratch m;
+  LMI_HIP(hipMalloc(&m.a, bytes));
+  LMI_HIP(hipMalloc(&m.b, bytes));
+  LMI_HIP(hipMemset(m.a, 1, bytes));
+  LMI_TRY(m.events());
+  const size_t n = bytes / 16;
+  // a grid in proportion to the bytes, as the gathers size theirs, between one block and 64 per compute unit
+  const int grid = (int)std::max<size_t>(1, std::min<size_t>(n / (256 * 4), 16384));
+  double total = 0.0;
+  for (int r = -1; r < repeats; ++r) {  // the first launch warms up and is not counted
+    hipExtLaunchKernelGGL(copy_kernel<false>, dim3(grid), dim3(256), 0, 0, m.e0, m.e1, 0, (const cp_u32x4 *)m.a,
+                          (cp_u32x4 *)m.b, n);
+    LMI_HIP(hipGetLastError());
+    LMI_HIP(hipDeviceSynchronize());
+    float ms = 0;
+    LMI_HIP(hipEventElapsedTime(&ms, m.e0, m.e1));
+    if (r >= 0) total += ms;
+  }
+  *ms_per_launch = total / repeats;
+  return LMI_OK;
 }
 
 }  // extern "C"
