@@ -7,6 +7,7 @@
 #include <fcntl.h>
 #include <unistd.h>
 
+#include <algorithm>
 #include <cerrno>
 #include <cstring>
 #include <map>
@@ -174,6 +175,7 @@ extern "C" int legion_ipc_initialize(void) {
   std::memset(g_edge_counter, 0, sizeof(g_edge_counter));
   if (g_env->Initialize() < 0) {
     g_error = g_env->LastError();
+    g_env->Finalize();  // whatever it had opened before it failed
     delete g_env;
     g_env = nullptr;
     return -1;
