@@ -248,7 +248,10 @@ int lmi_run_group(lmi_server *s, int n_batches, const int32_t *pipes, void *stre
  * Servers whose worst case exceeds the limits above, and servers with the LRU cache (whose
  * insertion needs per-pipe state), get LMI_ERR_CAPACITY / LMI_ERR_STATE.  Every call on a GPU
  * shares that GPU's array: calls that overlap on one GPU (two streams, two threads, two
- * servers) race; calls that follow each other on one stream do not. */
+ * servers) race; calls that follow each other on one stream do not.  What a call launches
+ * depends on nothing but its arguments and the device memory they name (the dedup table in the
+ * scratch is wiped by every call): captured in a HIP graph, it may be replayed, with new
+ * seeds written into the same `seeds` buffer between replays. */
 int lmi_run_once_static(lmi_server *s, void *stream, const int32_t *seeds, int32_t n,
                         uint64_t rng_seed, const lmi_batch_view *out);
 

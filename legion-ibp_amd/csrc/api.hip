@@ -831,8 +831,10 @@ int lmi_run_once_static(lmi_server *h, void *stream, const int32_t *seeds, int32
   LMI_HIP(hipSetDevice(device));
   unsigned char *ptr = g_static[device].ptr;
   Pipe &p = g_static[device].pipe;
-  // another server (another table size, other tilings) may have used the array last
-  if (p.dedup.log2cap != lg || p.max_tiles != tiles) p.table_dirty = true;
+  // The table is wiped by every call (no epoch kept on the host): another server may have used the
+  // array last, and the launches of a call must depend on nothing but its arguments and the device
+  // memory they name, so that a caller who captured them in a graph can replay it.
+  p.table_dirty = true;
   p.ids = out->ids;
   p.features = out->features;
   p.labels = out->labels;

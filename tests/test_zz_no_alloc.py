@@ -173,3 +173,68 @@ def test_static_entry_point_refuses_what_it_cannot_hold(lmi):
     finally:
         lmi.check(lmi.lib().lmi_device_free(d))
         feats.free()
+
+
+def hip_runtime():
+    """The HIP runtime the library itself is linked against (already loaded with it)."""
+    hip = C.CDLL("libamdhip64.so.7")
+    hip.hipStreamBeginCapture.argtypes = [C.c_void_p, C.c_int]
+    hip.hipStreamEndCapture.argtypes = [C.c_void_p, C.POINTER(C.c_void_p)]
+    hip.hipGraphInstantiate.argtypes = [C.POINTER(C.c_void_p), C.c_void_p, C.c_void_p, C.c_char_p, C.c_size_t]
+    hip.hipGraphLaunch.argtypes = [C.c_void_p, C.c_void_p]
+    hip.hipGraphExecDestroy.argtypes = [C.c_void_p]
+    hip.hipGraphDestroy.argtypes = [C.c_void_p]
+    return hip
+
+
+def test_static_entry_point_replayed_from_a_captured_graph(lmi, oracle):
+    """The callers the entry point is for: its launches captured once in a HIP graph and replayed
+    with other seeds in the same buffer; eager batches and synchronisations between the replays,
+    every replay checked.  Captured in the global mode, in which an allocation by the capturing
+    thread is an error."""
+    hip = hip_runtime()
+    rng = np.random.default_rng(23)
+    n_nodes, dim, batch, fanout = 30_000, 128, 256, [25, 10]
+    indptr, indices = random_graph(rng, n_nodes, 14, hubs=8, hub_deg=3000)
+    feats = lmi.HostBuffer((n_nodes, dim), np.float32)
+    feats.array[...] = rng.standard_normal((n_nodes, dim)).astype(np.float32)
+    srv = lmi.Server(batch, fanout, dim, pipes=1, seed=5)
+    stream, other = lmi.stream_create(), lmi.stream_create()
+    outs = d = None
+    graph, graph_exec = C.c_void_p(), C.c_void_p()
+    try:
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        srv.build_static_cache(9000, lmi.TABLE_RANK)
+        outs = DeviceOutputs(lmi, srv)
+        d = device_seeds(lmi, np.zeros(batch, np.int32))
+        lmi.check(lmi.lib().lmi_device_sync())
+        assert hip.hipStreamBeginCapture(stream, 0) == 0          # hipStreamCaptureModeGlobal
+        try:
+            srv.run_once_static(d, batch, outs.view, rng_seed=77, stream=stream)
+        finally:
+            rc = hip.hipStreamEndCapture(stream, C.byref(graph))
+        assert rc == 0 and graph.value
+        assert hip.hipGraphInstantiate(C.byref(graph_exec), graph, None, None, 0) == 0
+        for rep in range(4):
+            seeds = rng.choice(n_nodes, batch, replace=False).astype(np.int32)
+            lmi.check(lmi.lib().lmi_copy_to_device(d, seeds.ctypes.data, seeds.nbytes))
+            assert hip.hipGraphLaunch(graph_exec, stream) == 0
+            lmi.check(lmi.lib().lmi_stream_sync(stream))
+            got = outs.fetch()
+            srv.run_once(seeds, rng_seed=77, pipe=0, stream=other)   # eager work between the replays
+            assert_same(got, srv.fetch(pipe=0, stream=other))
+            o = oracle.sample_batch(indptr, indices, seeds, fanout, 77)
+            assert np.array_equal(got.ids, o.ids) and np.array_equal(got.agg_src_off, o.agg_src_off)
+        srv.status()
+    finally:
+        if graph_exec.value:
+            hip.hipGraphExecDestroy(graph_exec)
+        if graph.value:
+            hip.hipGraphDestroy(graph)
+        srv.close()
+        if outs:
+            outs.free()
+        if d:
+            lmi.check(lmi.lib().lmi_device_free(d))
+        feats.free()
