@@ -83,7 +83,10 @@ def lib():
         if not os.path.exists(LIB_PATH):
             raise ImportError("liblegion_mi.so is missing: build it with `make -C %s` "
                               "(there is no CPU fallback)" % _HERE)
-        L = C.CDLL(LIB_PATH)
+        # RTLD_GLOBAL: a HIP runtime loaded later by another package (PyTorch brings its own copy)
+        # then resolves to the one this library already initialised; two runtimes in one process
+        # cannot both open the GPU
+        L = C.CDLL(LIB_PATH, mode=C.RTLD_GLOBAL)
         L.lmi_last_error.restype = C.c_char_p
         L.lmi_host_alloc.argtypes = [C.c_size_t, C.POINTER(C.c_void_p)]
         L.lmi_host_free.argtypes = [C.c_void_p]

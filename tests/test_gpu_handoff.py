@@ -44,8 +44,9 @@ def leftovers():
             if os.path.exists("/dev/shm/" + n)]
 
 
-@pytest.mark.parametrize("dyn_cache,part_bytes", [(0, None), (1, None), (0, 65536)])
-def test_trainer_in_a_process_of_its_own(tmp_path, dyn_cache, part_bytes):
+@pytest.mark.parametrize("dyn_cache,part_bytes,flavour", [(0, None, "numpy"), (1, None, "numpy"), (0, 65536, "numpy"),
+                                                          (0, None, "torch"), (0, 65536, "torch")])
+def test_trainer_in_a_process_of_its_own(tmp_path, dyn_cache, part_bytes, flavour):
     """part_bytes: the largest allocation the server shares whole.  The real limit (2 GiB) only
     matters for feature buffers of the largest configurations; a small one makes this test's
     feature buffer (2560 rows of 128 bytes) go over in five pieces, re-assembled by the trainer."""
@@ -74,7 +75,7 @@ def test_trainer_in_a_process_of_its_own(tmp_path, dyn_cache, part_bytes):
             time.sleep(0.2)
         # the trainer: a fresh process whose first GPU work is opening the server's buffers
         out = subprocess.run([sys.executable, os.path.join(ROOT, "tests", "handoff_consumer.py"), str(data), str(batch),
-                              str(dim), str(epochs), str(dyn_cache), "numpy", "attach"], timeout=300,
+                              str(dim), str(epochs), str(dyn_cache), flavour, "attach"], timeout=300,
                              capture_output=True, text=True, cwd=str(tmp_path))
         assert out.returncode == 0, out.stdout[-3000:] + out.stderr[-3000:] + log_path.read_text()[-2000:]
         assert "HANDOFF_OK %d batches" % ((4 + 1) * epochs + 1) in out.stdout
