@@ -246,7 +246,14 @@ class GPUServer : public Server {
     cfg.hops = (int)fanout.size();
     for (int k = 0; k < cfg.hops && k < LMI_MAX_HOPS; ++k) cfg.fanout[k] = fanout[k];
     cfg.feat_dim = meta_.feature_dim;
-    cfg.feat_dtype = LMI_F32;
+    // meta_config has no field for the element type: fp32 as in the reference's files, fp16 on request
+    const char *dt = std::getenv("LEGION_MI_FEAT_DTYPE");
+    if (dt && std::strcmp(dt, "f16") != 0 && std::strcmp(dt, "f32") != 0) {
+      std::fprintf(stderr, "LEGION_MI_FEAT_DTYPE must be f32 or f16, got %s\n", dt);
+      std::exit(EXIT_FAILURE);
+    }
+    elem_bytes_ = (dt && std::strcmp(dt, "f16") == 0) ? 2 : 4;
+    cfg.feat_dtype = elem_bytes_ == 2 ? LMI_F16 : LMI_F32;
     cfg.pipes = 2;
     cfg.seed = 1;
     LMI_MUST(lmi_server_create(&cfg, &h_));
@@ -260,7 +267,7 @@ class GPUServer : public Server {
     must_read(dp + "edge_dst", indices.data(), meta_.edge_num * 4);
     LMI_MUST(lmi_graph_load(h_, indptr.data(), indices.data(), meta_.node_num, meta_.edge_num, LMI_LOC_HOST));
     // features: pinned + mapped host memory, read zero-copy on cache misses
-    const int64_t fbytes = meta_.node_num * (int64_t)meta_.feature_dim * 4;
+    const int64_t fbytes = meta_.node_num * (int64_t)meta_.feature_dim * elem_bytes_;
     LMI_MUST(lmi_host_alloc((size_t)fbytes, &host_features_));
     must_read(fp + "features", host_features_, fbytes);
     LMI_MUST(lmi_features_attach(h_, host_features_, meta_.node_num, LMI_LOC_HOST));
@@ -314,7 +321,7 @@ class GPUServer : public Server {
       std::fprintf(stderr, "cache aggregation across GPUs is not part of this build (mode %d)\n", cache_agg_mode);
       std::exit(EXIT_FAILURE);
     }
-    const int64_t row_bytes = (int64_t)meta_.feature_dim * 4;
+    const int64_t row_bytes = (int64_t)meta_.feature_dim * elem_bytes_;
     if (std::getenv("LEGION_MI_PRESAMPLE")) {
       // the reference's policy: one presampling pass over the training set through the
       // operator table, then rank by how often each node was sampled (engine/server.cu:31-37,94-122)
@@ -401,6 +408,7 @@ class GPUServer : public Server {
   LegionMetaConfig meta_;
   std::vector<int> fanout_;
   int dyn_cache_ = 0;
+  int elem_bytes_ = 4;  // of a feature element: fp32, or fp16 with LEGION_MI_FEAT_DTYPE=f16
   lmi_server *h_ = nullptr;
   void *host_features_ = nullptr;
   Runner *runner_ = nullptr;

@@ -19,7 +19,7 @@
 namespace {
 struct Dump {
   std::string dir;
-  int left = 0, index = 0, feat_dim = 0;
+  int left = 0, index = 0;
 };
 
 void dump_sink(const lmi_batch_view *b, int, int, void *stream, void *user) {
@@ -34,11 +34,11 @@ void dump_sink(const lmi_batch_view *b, int, int, void *stream, void *user) {
   int64_t e = 0;
   for (int k = 1; k <= hops; ++k) e += ec[9 + k];
   std::vector<int32_t> ids((size_t)n), src((size_t)e), dst((size_t)e);
-  std::vector<float> feat((size_t)n * d->feat_dim);
+  std::vector<unsigned char> feat((size_t)n * (size_t)b->row_bytes);  // fp32 or fp16 rows, as served
   if (n) lmi_copy_to_host(ids.data(), b->ids, (size_t)n * 4);
   if (e) lmi_copy_to_host(src.data(), b->agg_src_off, (size_t)e * 4);
   if (e) lmi_copy_to_host(dst.data(), b->agg_dst_off, (size_t)e * 4);
-  if (n) lmi_copy_to_host(feat.data(), b->features, feat.size() * 4);
+  if (n) lmi_copy_to_host(feat.data(), b->features, feat.size());
   const std::string path = d->dir + "/batch_" + std::to_string(d->index) + ".bin";
   FILE *f = std::fopen(path.c_str(), "wb");
   if (f) {
@@ -47,7 +47,7 @@ void dump_sink(const lmi_batch_view *b, int, int, void *stream, void *user) {
     std::fwrite(ids.data(), 4, ids.size(), f);
     std::fwrite(src.data(), 4, src.size(), f);
     std::fwrite(dst.data(), 4, dst.size(), f);
-    std::fwrite(feat.data(), 4, feat.size(), f);
+    std::fwrite(feat.data(), 1, feat.size(), f);
     std::fclose(f);
   }
   --d->left;
@@ -79,11 +79,7 @@ int main(int argc, char **argv) {
   server->Initialize(std::atoi(argv[1]), fanout, 1, std::atoi(argv[3]));
   Dump dump;
   if (const char *dir = std::getenv("LEGION_MI_DUMP")) {
-    LegionMetaConfig meta;
-    std::string err;
-    LegionReadMetaConfig("./meta_config", &meta, &err);
     dump.dir = dir;
-    dump.feat_dim = meta.feature_dim;
     const char *nb = std::getenv("LEGION_MI_DUMP_BATCHES");
     dump.left = nb ? std::atoi(nb) : 2;
     server->SetBatchSink(dump_sink, &dump);

@@ -26,12 +26,19 @@ def main():
     indptr = np.fromfile(os.path.join(data, "edge_src"), np.int64)
     indices = np.fromfile(os.path.join(data, "edge_dst"), np.int32)
     n_nodes = len(indptr) - 1
-    feats = np.fromfile(os.path.join(data, "features"), np.float32).reshape(n_nodes, dim)
+    # element type of the `features` file: the server and this consumer learn it the same way
+    f16 = os.environ.get("LEGION_MI_FEAT_DTYPE") == "f16"
+    np_dtype = np.float16 if f16 else np.float32
+    feats = np.fromfile(os.path.join(data, "features"), np_dtype).reshape(n_nodes, dim)
     labels = np.fromfile(os.path.join(data, "labels"), np.int32)
     sets = [np.fromfile(os.path.join(data, n), np.int32) for n in ("trainingset", "validationset", "testingset")]
     ipc = load_ipc_service()
     steps_ref, sizes, total = ipc.schedule(len(sets[0]), len(sets[1]), len(sets[2]), batch, epochs)
 
+    if dyn_cache == 8:   # int8 cache: hits arrive dequantised; the oracle's codec says what they must be
+        cache_bytes = int(open(os.environ.get("LEGION_MI_META_CONFIG", "meta_config")).read().split()[8])
+        slot = oracle.static_cache_build(indptr, cache_bytes // (dim + 4))
+        q, sc = oracle.quantize_rows(feats[np.flatnonzero(slot >= 0)])
     attach = len(sys.argv) > 7 and sys.argv[7] == "attach"
     if not attach:
         ipc.start_server(dyn_cache=dyn_cache, fanout=fanout, wait_seconds=60.0)
@@ -41,13 +48,14 @@ def main():
         mode, local = ipc.schedule_batch(len(sets[0]), len(sets[1]), len(sets[2]), batch, epochs, g)
         seeds = sets[mode][local * sizes[mode]:(local + 1) * sizes[mode]]
         if flavour == "torch":
-            out = [t.cpu().numpy() for t in ipc.get_next(dim, wait_seconds=60.0)]
+            out = [t.cpu().numpy() for t in ipc.get_next(dim, wait_seconds=60.0, feature_typestr="<f2" if f16 else "<f4")]
         else:
-            out = ipc.get_next_numpy(dim, wait_seconds=60.0)
+            out = ipc.get_next_numpy(dim, wait_seconds=60.0, feature_dtype=np_dtype)
         o = oracle.sample_batch(indptr, indices, seeds, fanout, 1 + local)
         ids, f, lab = out[0], out[1], out[2]
         assert np.array_equal(ids, o.ids), "ids of batch %d" % g
-        assert f.tobytes() == feats[o.ids].tobytes(), "features of batch %d" % g
+        want = oracle.gather_rows_int8(o.ids, slot[o.ids], q, sc, feats) if dyn_cache == 8 else feats[o.ids]
+        assert f.tobytes() == want.tobytes(), "features of batch %d" % g
         assert np.array_equal(lab, labels[seeds]), "labels of batch %d" % g
         hops = len(fanout)
         sizes_ref = []

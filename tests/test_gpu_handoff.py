@@ -44,9 +44,10 @@ def leftovers():
             if os.path.exists("/dev/shm/" + n)]
 
 
-@pytest.mark.parametrize("dyn_cache,part_bytes,flavour", [(0, None, "numpy"), (1, None, "numpy"), (0, 65536, "numpy"),
-                                                          (0, None, "torch"), (0, 65536, "torch")])
-def test_trainer_in_a_process_of_its_own(tmp_path, dyn_cache, part_bytes, flavour):
+@pytest.mark.parametrize("dyn_cache,part_bytes,flavour,dtype", [
+    (0, None, "numpy", "f32"), (1, None, "numpy", "f32"), (0, 65536, "numpy", "f32"), (0, None, "torch", "f32"),
+    (0, 65536, "torch", "f32"), (0, 40000, "numpy", "f16"), (8, None, "torch", "f16")])
+def test_trainer_in_a_process_of_its_own(tmp_path, dyn_cache, part_bytes, flavour, dtype):
     """part_bytes: the largest allocation the server shares whole.  The real limit (2 GiB) only
     matters for feature buffers of the largest configurations; a small one makes this test's
     feature buffer (2560 rows of 128 bytes) go over in five pieces, re-assembled by the trainer."""
@@ -57,10 +58,11 @@ def test_trainer_in_a_process_of_its_own(tmp_path, dyn_cache, part_bytes, flavou
     n_nodes, dim, batch, n_train, epochs = 4000, 32, 64, 300, 2
     data = tmp_path / "data"
     data.mkdir()
-    indptr, indices, feats, train = write_dataset(str(data), rng, n_nodes, dim, n_train)
+    indptr, indices, feats, train = write_dataset(str(data), rng, n_nodes, dim, n_train,
+                                                  np.float16 if dtype == "f16" else np.float32)
     (tmp_path / "meta_config").write_text("%s/ %d %d %d %d %d %d %d %d %d" % (
         data, batch, n_nodes, len(indices), dim, n_train, 50, 40, 600 * dim * 4, epochs))
-    env = dict(os.environ, LEGION_MI_HANDOFF="1", LEGION_MI_WAIT_SECONDS="90")
+    env = dict(os.environ, LEGION_MI_HANDOFF="1", LEGION_MI_WAIT_SECONDS="90", LEGION_MI_FEAT_DTYPE=dtype)
     if part_bytes:
         env["LEGION_MI_IPC_PART_BYTES"] = str(part_bytes)
     log_path = tmp_path / "server.log"
@@ -76,7 +78,7 @@ def test_trainer_in_a_process_of_its_own(tmp_path, dyn_cache, part_bytes, flavou
         # the trainer: a fresh process whose first GPU work is opening the server's buffers
         out = subprocess.run([sys.executable, os.path.join(ROOT, "tests", "handoff_consumer.py"), str(data), str(batch),
                               str(dim), str(epochs), str(dyn_cache), flavour, "attach"], timeout=300,
-                             capture_output=True, text=True, cwd=str(tmp_path))
+                             capture_output=True, text=True, cwd=str(tmp_path), env=env)
         assert out.returncode == 0, out.stdout[-3000:] + out.stderr[-3000:] + log_path.read_text()[-2000:]
         assert "HANDOFF_OK %d batches" % ((4 + 1) * epochs + 1) in out.stdout
         assert server.wait(timeout=120) == 0, log_path.read_text()[-3000:]

@@ -14,9 +14,9 @@ pytestmark = pytest.mark.gpu
 BIN = os.path.join(ROOT, "legion-ibp_amd", "sampling_server")
 
 
-def write_dataset(d, rng, n_nodes, dim, n_train):
+def write_dataset(d, rng, n_nodes, dim, n_train, dtype=np.float32):
     indptr, indices = random_graph(rng, n_nodes, 10, hubs=4, hub_deg=300)
-    feats = rng.standard_normal((n_nodes, dim)).astype(np.float32)
+    feats = rng.standard_normal((n_nodes, dim)).astype(dtype)
     labels = rng.integers(0, 40, n_nodes).astype(np.int32)
     perm = rng.permutation(n_nodes).astype(np.int32)
     train, valid, test = perm[:n_train], perm[n_train:n_train + 50], perm[n_train + 50:n_train + 90]
@@ -34,8 +34,10 @@ def read_sets(d):
     return [np.fromfile(os.path.join(d, n), np.int32) for n in ("trainingset", "validationset", "testingset")]
 
 
-def read_dump(path, dim):
-    raw = np.fromfile(path, np.int32)
+def read_dump(path, dim, dtype=np.float32):
+    raw = np.fromfile(path, np.uint8)
+    words = dim * np.dtype(dtype).itemsize // 4     # 4-byte words of a feature row
+    raw, dim = raw.view(np.int32), words
     nc, ec = raw[:16], raw[16:32]
     hops = int(nc[8])
     n, e = int(nc[9 + hops]), int(sum(ec[10:10 + hops]))
@@ -43,26 +45,31 @@ def read_dump(path, dim):
     ids = raw[o:o + n]; o += n
     src = raw[o:o + e]; o += e
     dst = raw[o:o + e]; o += e
-    feat = raw[o:o + n * dim].view(np.float32).reshape(n, dim)
+    feat = raw[o:o + n * dim].view(dtype).reshape(n, -1)
     assert o + n * dim == len(raw)
     return nc, ec, ids, src, dst, feat
 
 
-@pytest.mark.parametrize("dyn_cache,table_mode,presample", [(0, False, False), (0, True, False), (1, False, False),
-                                                             (1, True, False), (8, False, False), (0, True, True)])
-def test_sampling_server_binary(tmp_path, oracle, dyn_cache, table_mode, presample):
+@pytest.mark.parametrize("dyn_cache,table_mode,presample,dtype", [
+    (0, False, False, "f32"), (0, True, False, "f32"), (1, False, False, "f32"), (1, True, False, "f32"),
+    (8, False, False, "f32"), (0, True, True, "f32"),
+    (0, False, False, "f16"), (1, False, False, "f16"), (8, False, False, "f16")])   # fp16 `features` file
+def test_sampling_server_binary(tmp_path, oracle, dyn_cache, table_mode, presample, dtype):
     assert os.path.exists(BIN), "build the host shim first (make -C legion-ibp_amd)"
     rng = np.random.default_rng(dyn_cache * 2 + table_mode)
     n_nodes, dim, batch, n_train, fanout = 5000, 64, 100, 350, [25, 10]
     data = tmp_path / "data"
     data.mkdir()
-    indptr, indices, feats, train = write_dataset(str(data), rng, n_nodes, dim, n_train)
+    np_dtype = np.float16 if dtype == "f16" else np.float32
+    indptr, indices, feats, train = write_dataset(str(data), rng, n_nodes, dim, n_train, np_dtype)
     cache_bytes = 1500 * dim * 4
     (tmp_path / "meta_config").write_text("%s/ %d %d %d %d %d %d %d %d %d" % (
         data, batch, n_nodes, len(indices), dim, n_train, 50, 40, cache_bytes, 2))
     dump = tmp_path / "dump"
     dump.mkdir()
     env = dict(os.environ, LEGION_MI_DUMP=str(dump), LEGION_MI_DUMP_BATCHES="4")
+    if dtype == "f16":
+        env["LEGION_MI_FEAT_DTYPE"] = "f16"
     if table_mode:
         env["LEGION_MI_OPERATOR_TABLE"] = "1"
     if presample:
@@ -78,7 +85,7 @@ def test_sampling_server_binary(tmp_path, oracle, dyn_cache, table_mode, presamp
         q, sc = oracle.quantize_rows(feats[np.flatnonzero(slot >= 0)])
     valid = read_sets(str(data))[1]
     for i in range(4):   # three training batches of 100, then the validation batch of 50
-        nc, ec, ids, src, dst, feat = read_dump(str(dump / ("batch_%d.bin" % i)), dim)
+        nc, ec, ids, src, dst, feat = read_dump(str(dump / ("batch_%d.bin" % i)), dim, np_dtype)
         seeds, local = (train[i * batch:(i + 1) * batch], i) if i < 3 else (valid, 0)
         o = oracle.sample_batch(indptr, indices, seeds, fanout, 1 + local)
         assert list(nc) == list(o.node_counter) and list(ec) == list(o.edge_counter)
