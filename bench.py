@@ -40,7 +40,8 @@ def load_package():
 WORKLOADS = {
     # name: nodes, mean degree, alpha, d_max, dim, dtype, batch, fanout, train, cache
     "paper100m": dict(nodes=111_059_956, mean_deg=14.548, alpha=2.0, d_max=100_000, dim=128, dtype="f32",
-                      batch=8000, fanout=[25, 10], train=1_200_000, cache=("static", 38e9)),
+                      batch=8000, fanout=[25, 10], train=1_200_000, cache=("static", 38e9),
+                      tune={"miss_blocks": 36}),
     "products": dict(nodes=2_449_029, mean_deg=25.27, alpha=2.1, d_max=17_000, dim=100, dtype="f32",
                      batch=800, fanout=[25, 10], train=196_615, cache=("static_frac", 0.30)),
     "paper100m-lru": dict(nodes=111_059_956, mean_deg=14.548, alpha=2.0, d_max=100_000, dim=128, dtype="f32",
@@ -356,10 +357,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--workload", default="paper100m", choices=sorted(WORKLOADS))
     ap.add_argument("--scale", type=float, default=1.0, help="shrink node/train counts (testing only)")
-    ap.add_argument("--pipes", type=int, default=8, help="output buffer sets in flight")
+    ap.add_argument("--pipes", type=int, default=16, help="output buffer sets in flight")
     ap.add_argument("--streams", type=int, default=1, help="caller streams the pipes are spread over")
-    ap.add_argument("--group", type=int, default=4,
-                    help="mini-batches issued together with lmi_run_group (their sampling kernels share launches)")
+    ap.add_argument("--group", type=int, default=8,
+                    help="at most this many mini-batches are issued together with lmi_run_group (their sampling "
+                         "kernels share launches)")
     ap.add_argument("--seed", type=int, default=20260101)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget (0 = skip)")
     ap.add_argument("--host-gb", type=float, default=0.0,
@@ -406,8 +408,8 @@ def main():
     tunes = {k: str(v) for k, v in w.get("tune", {}).items()}   # the workload's own settings, then --tune
     tunes.update(kv.split("=") for kv in args.tune)
     # host-link gather grid (miss_blocks, library default 32), measured on paper100m-shaped in groups
-    # of 4 on 8 pipes: 24 -> 6.6 k batches/s, 28 -> 7.2 k, 32 -> 7.5 k, 36 -> 7.3 k, 40 -> 7.0 k,
-    # 48 -> 6.5 k; the HBM gather stays at 66-68 % of peak throughout
+    # of 8 on 16 pipes: 32 -> 8.3 k batches/s, 36 -> 8.6 k, 40 -> 8.6 k, 48 -> 8.2 k; the HBM gather
+    # stays at 68-69 % of peak throughout
     for k, v in tunes.items():
         srv.tune(k, int(v))
     steps_per_epoch = -(-info["n_train"] // w["batch"])
@@ -422,8 +424,9 @@ def main():
         log("recorded %d seed batches with temporal locality (%.1f s)" % (len(plan), time.time() - t0))
 
     group = max(1, args.group)
-    if group > 1 and (args.pipes % group or info["cache_kind"] == "lru"):
-        print("bench.py: --group needs a pipe count that is a multiple of it, and no LRU cache", file=sys.stderr)
+    if group > 1 and (args.pipes < group or info["cache_kind"] == "lru"):
+        print("bench.py: --group needs at least as many pipes (twice as many keep two groups in flight), and no "
+              "LRU cache", file=sys.stderr)
         sys.exit(2)
 
     def step(i, n=None):
@@ -441,10 +444,19 @@ def main():
                           seeds=[plan[k] for k in ks] if plan else None, rng_seeds=[args.seed + k for k in ks],
                           stream=streams[(p // group) % len(streams)])
 
+    def group_sizes(count):
+        """`count` batches as the fewest groups of at most `group`, sized evenly (20 in groups of up to
+        8: 7, 7, 6): the side stream's last, exposed, host-link gather is then no longer than the others."""
+        n_groups = -(-count // group)
+        base, extra = divmod(count, n_groups) if n_groups else (0, 0)
+        return [base + 1] * extra + [base] * (n_groups - extra)
+
     def run_steps(first, count):
-        """Batches first .. first+count-1 in groups (the last group may be a partial one)."""
-        for i in range(first, first + count, group):
-            step(i, min(group, first + count - i))
+        """Batches first .. first+count-1, group by group."""
+        i = first
+        for n in group_sizes(count):
+            step(i, n)
+            i += n
 
     run_steps(0, args.warmup)
     lmi.check(lmi.lib().lmi_device_sync())
@@ -503,8 +515,9 @@ def main():
     # a group's hit gathers are one launch (on the caller's stream) and so are its host-link
     # gathers (on the side stream)
     split = int(tunes.get("split_miss", 1)) == 1
-    hit_batches = group if split else 1
-    miss_batches = group if (split and int(tunes.get("group_miss", 1))) else 1
+    timed_group = args.steps / max(len(group_sizes(args.steps)), 1)   # batches per launch of the timed region
+    hit_batches = timed_group if split else 1
+    miss_batches = timed_group if (split and int(tunes.get("group_miss", 1))) else 1
     hit_ms = prof.gather_hit_ms / max(prof.gather_hit_launches, 1)
     hit_rows = prof.gather_hit_rows / max(prof.gather_hit_launches, 1)
     miss_ms = prof.gather_miss_ms / max(prof.gather_miss_launches, 1)
@@ -568,7 +581,7 @@ def main():
     roofline = dict(bound="hbm", kernel=hit_kernel, achieved=round(achieved, 1),
                     peak=HBM_PEAK_GBS, unit="GB/s", frac=round(achieved / HBM_PEAK_GBS, 4),
                     traffic=traffic, traffic_source=traffic_source,
-                    rows_per_launch=round(hit_rows, 1), batches_per_launch=hit_batches, bytes_per_row=hit_bytes,
+                    rows_per_launch=round(hit_rows, 1), batches_per_launch=round(hit_batches, 2), bytes_per_row=hit_bytes,
                     avg_launch_ms=round(hit_ms, 4),
                     measured_copy_gbs=round(copy_gbs, 1),
                     same_bytes_copy_gbs=round(same_copy_gbs, 1) if same_copy_gbs else None,
@@ -579,7 +592,7 @@ def main():
                      measured_stream_read_gbs=round(link_bytes // 16 * 16 / (link_ms * 1e-3) / 1e9, 2),
                      achieved=round(miss_rows * rb / (miss_ms * 1e-3) / 1e9, 2) if miss_ms > 0 else 0.0,
                      peak=HOST_LINK_PEAK_GBS, unit="GB/s", rows_per_launch=round(miss_rows, 1),
-                     batches_per_launch=miss_batches,
+                     batches_per_launch=round(miss_batches, 2),
                      avg_launch_ms=round(miss_ms, 4))
     # the sampling kernels are bound by cold random reads: what the device sustains on the neighbour array
     rr_reads = 1 << 24

@@ -744,7 +744,7 @@ static int capture_batch_graph(Server *s, Pipe &p, hipStream_t st, const BatchPa
 
 // One batch on each of n pipes, served by the same launches.
 static int run_group(Server *s, Pipe *const *pp, const BatchParams *bps, int n, hipStream_t st) {
-  for (int k = 0; k < n; ++k) LMI_TRY(pipe_join(*pp[k], st));  // a pipe's previous batch may still be gathering misses
+  LMI_TRY(pipes_join(pp, n, st));  // a pipe's previous batch may still be gathering misses
   prof_phase(s, st, &s->prof_open, PROF_SAMPLE);
   if (s->use_graph && st != nullptr && n == 1) {  // the legacy default stream cannot be captured
     Pipe &p = *pp[0];
@@ -1013,6 +1013,7 @@ int lmi_tune(lmi_server *h, const char *key, int64_t value) {
   else if (!strcmp(key, "protect_hits")) s->protect_hits = (int)value;
   else if (!strcmp(key, "group_miss")) s->group_miss = (int)value;
   else if (!strcmp(key, "lru_early_miss")) s->lru_early_miss = (int)value;
+  else if (!strcmp(key, "early_fork")) s->early_fork = (int)value;
   else if (!strcmp(key, "table_epochs")) {
     s->table_epochs = std::max<int64_t>(0, value);
     for (auto &p : s->pipes) p.table_dirty = true;

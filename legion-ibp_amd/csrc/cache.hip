@@ -799,12 +799,30 @@ int launch_lookup(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg_fir
 // wait is only queued when the host cannot already see the event as complete.
 int pipe_join(Pipe &p, hipStream_t st) {
   if (p.side_pending) {
-    const hipError_t q = hipEventQuery(p.join);
+    const hipError_t q = hipEventQuery(p.join_of);
     if (q != hipSuccess) {
       (void)hipGetLastError();  // "not ready" is an answer, not a failure
-      LMI_HIP(hipStreamWaitEvent(st, p.join, 0));
+      LMI_HIP(hipStreamWaitEvent(st, p.join_of, 0));
     }
     p.side_pending = false;
+  }
+  return LMI_OK;
+}
+
+int pipes_join(Pipe *const *pp, int n, hipStream_t st) {
+  hipEvent_t seen[LMI_MAX_GROUP];
+  int n_seen = 0;
+  for (int k = 0; k < n; ++k) {
+    Pipe &p = *pp[k];
+    if (!p.side_pending) continue;
+    bool dup = false;
+    for (int j = 0; j < n_seen; ++j) dup = dup || seen[j] == p.join_of;
+    if (dup) {
+      p.side_pending = false;  // `st` already waits for (or has seen) this event
+      continue;
+    }
+    if (n_seen < LMI_MAX_GROUP) seen[n_seen++] = p.join_of;
+    LMI_TRY(pipe_join(p, st));
   }
   return LMI_OK;
 }
@@ -990,7 +1008,7 @@ int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int s
     // LRU batches are host-link-bound (a fifth of their rows miss): their host-link gather starts
     // beside the HBM gather instead of behind it.  The insertion that follows it on the side stream
     // only overwrites ways this batch's lookup did not touch, so the hits never read a row it writes.
-    const bool early = lru_lists > 0 && s->lru_early_miss;
+    const bool early = (lru_lists > 0 && s->lru_early_miss) || (lru_lists == 0 && s->early_fork);
     fork = nullptr;
     if (early) {
       fork = pp[0]->fork;
@@ -1006,12 +1024,20 @@ int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int s
   // the group's host-link gathers as one launch when nothing has to come between them
   const bool misses_together = n > 1 && mode == 1 && lru_lists == 0 && s->group_miss;
   if (misses_together) LMI_TRY(launch_misses(s, pp, n, s->side, seg, seg_last));
-  for (int k = 0; k < n; ++k) {
+  if (misses_together) {  // nothing else of the group goes to the side stream: one event for all its pipes
+    LMI_HIP(hipEventRecord(pp[0]->join, s->side));
+    for (int k = 0; k < n; ++k) {
+      pp[k]->join_of = pp[0]->join;
+      pp[k]->side_pending = true;
+    }
+  }
+  for (int k = 0; k < n && !misses_together; ++k) {
     Pipe &p = *pp[k];
     if (mode == 2) LMI_TRY(launch_hits(s, pp + k, 1, s->side, seg, seg_last));
-    if (!misses_together) LMI_TRY(launch_misses(s, pp + k, 1, s->side, seg, seg_last));
+    LMI_TRY(launch_misses(s, pp + k, 1, s->side, seg, seg_last));
     if (lru_lists > 0) LMI_TRY(launch_lru_insert(s, p, s->side, lru_lists));  // reads the rows just gathered
     LMI_HIP(hipEventRecord(p.join, s->side));
+    p.join_of = p.join;
     p.side_pending = true;
     // an LRU insertion that comes later on the caller's stream copies the gathered rows: join now
     if (s->cache_kind == LMI_CACHE_LRU && lru_lists == 0) LMI_TRY(pipe_join(p, st));

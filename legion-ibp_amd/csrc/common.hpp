@@ -102,7 +102,11 @@ struct Pipe {
   int32_t *lru_fill = nullptr;                        // [max_nodes] slot granted to a miss
   int32_t *lru_next = nullptr;                        // [max_nodes] next row in the list of misses of the same LRU set
   hipEvent_t fork = nullptr, join = nullptr;
-  bool side_pending = false;   // the side stream still owes this pipe's miss rows (join not yet waited on)
+  // The event that marks the end of this pipe's side-stream work: its own `join`, or that of the
+  // first pipe of the group its misses were gathered with (one record and one wait per group: a
+  // wait on another queue's event costs a stream about 10 us, fired or not).
+  hipEvent_t join_of = nullptr;
+  bool side_pending = false;   // the side stream still owes this pipe's miss rows (join_of not yet waited on)
   int32_t *seed_stage = nullptr;  // [batch_size] host seeds land here
   int32_t n_seeds = 0;
   int32_t hops_done = 0;
@@ -169,6 +173,7 @@ struct Server {
   hipEvent_t side_idle = nullptr;  // recorded behind the last host-link gather issued on the side stream
   bool side_busy = false;
   int protect_hits = 0;            // 1: HBM gathers wait until earlier host-link gathers have drained
+  int early_fork = 0;              // 1: the side stream is released before the HBM gather is launched, not behind it
   int lru_early_miss = 1;          // 1: with the LRU cache the host-link gather starts beside the HBM gather
   int group_miss = 1;              // 1: the host-link gathers of a group of batches are one launch
   hipEvent_t lru_ready = nullptr;  // recorded when an LRU insertion has settled keys and ticks: the next lookup waits for it
@@ -269,6 +274,8 @@ int launch_lru_insert(Server *s, Pipe &p, hipStream_t st, int n_lists);
 int lru_wait_ready(Server *s, hipStream_t st);
 int lru_wait_copied(Server *s, hipStream_t st);  // orders `st` behind the last LRU insertion
 int pipe_join(Pipe &p, hipStream_t st);  // make `st` wait for the pipe's side-stream work
+// the same for n pipes, each distinct event waited on once
+int pipes_join(Pipe *const *pp, int n, hipStream_t st);
 int cache_dump(Server *s, int32_t *slot_of, int64_t n, int32_t *aux);
 
 inline int64_t ceil_div(int64_t a, int64_t b) { return (a + b - 1) / b; }

@@ -3,6 +3,7 @@
 #pragma once
 
 #include "common.hpp"
+#include "lookback.hpp"
 
 namespace lmi {
 
@@ -132,13 +133,12 @@ __device__ __forceinline__ void fill_local_ids(const FillArgs &f, int64_t tid, i
   }
 }
 
-// A launch that serves n pipes interleaves them over blockIdx.x: block b works on pipe b % n
-// as that pipe's block b / n of gridDim.x / n.  Every pipe's blocks are then dispatched in
-// step and in ascending order, which the look-back scans rely on.
-#define LMI_GRID_ROW(n_rows)                                     \
-  const int row = (int)(blockIdx.x % (unsigned)(n_rows));        \
-  const int bx = (int)(blockIdx.x / (unsigned)(n_rows));         \
-  const int gx = (int)(gridDim.x / (unsigned)(n_rows));          \
+// A launch that serves n pipes interleaves them over blockIdx.x (grid_row).
+#define LMI_GRID_ROW(n_rows)                                                   \
+  const GridRow lmi_gr_ = grid_row(blockIdx.x, (unsigned)(n_rows));            \
+  const int row = lmi_gr_.row;                                                 \
+  const int bx = lmi_gr_.bx;                                                   \
+  const int gx = (int)(gridDim.x / (unsigned)(n_rows));                        \
   (void)gx
 
 // ------------------------------------------------------------------- scans

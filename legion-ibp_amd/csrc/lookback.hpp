@@ -32,4 +32,21 @@ LMI_HD inline LookbackWindow lookback_window(uint64_t inc, uint64_t inv) {
   return w;
 }
 
+// Which pipe a block of a launch that serves n pipes works on, and which of that pipe's blocks it
+// is.  Each aligned run of n blocks holds one block of every pipe (block b is its pipe's block
+// b / n), so every pipe's blocks are dispatched in step and in ascending order, which the
+// look-back relies on.  The pipe a place in the run serves rotates from run to run: workgroups
+// go to the 8 XCDs round robin (block b to XCD b % 8), so a plain b % n would pin a pipe to 8 / n
+// of them when n divides 8 (one XCD per pipe at n = 8) and the pipes would finish unevenly.
+// Rotating by the octet (n | 8) or by the run (otherwise) takes every pipe over all the XCDs.
+struct GridRow {
+  int row;  // pipe
+  int bx;   // the pipe's own block index
+};
+
+LMI_HD inline GridRow grid_row(unsigned block, unsigned n) {
+  const unsigned rot = (8u % n == 0) ? block / 8u : block / n;
+  return GridRow{(int)((block % n + rot) % n), (int)(block / n)};
+}
+
 }  // namespace lmi

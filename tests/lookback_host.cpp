@@ -28,3 +28,10 @@ extern "C" int lookback_prefix(const uint64_t *status, int tile, int64_t *prefix
   if (windows_out) *windows_out = windows;
   return 1;
 }
+
+// The block -> (pipe, block of that pipe) mapping of launches that serve n pipes.
+extern "C" void grid_row_of(unsigned block, unsigned n, int *row, int *bx) {
+  const lmi::GridRow g = lmi::grid_row(block, n);
+  *row = g.row;
+  *bx = g.bx;
+}

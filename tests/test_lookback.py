@@ -55,3 +55,23 @@ def test_lookback_gives_the_exact_prefix_or_waits(lookback, n_tiles):
             else:
                 assert done == 1 and got.value == want == int(sums[:tile].sum())
                 assert windows.value <= (tile + 63) // 64 + 1
+
+
+@pytest.mark.parametrize("n", range(1, 9))
+def test_blocks_of_a_shared_launch_map_onto_pipes(lookback, n):
+    """What the look-back needs of the mapping: every pipe's blocks are numbered 0, 1, 2, ... in
+    launch order, block k of every pipe lies in the k-th run of n blocks (so the pipes advance in
+    step).  What the hardware wants: with workgroups dealt to 8 XCDs round robin, every pipe's blocks
+    visit all 8."""
+    lookback.grid_row_of.argtypes = [C.c_uint, C.c_uint, C.POINTER(C.c_int), C.POINTER(C.c_int)]
+    row, bx = C.c_int(), C.c_int()
+    seen = {p: [] for p in range(n)}
+    xcds = {p: set() for p in range(n)}
+    for b in range(n * 8 * 50):
+        lookback.grid_row_of(b, n, C.byref(row), C.byref(bx))
+        assert 0 <= row.value < n and bx.value == b // n
+        seen[row.value].append(bx.value)
+        xcds[row.value].add(b % 8)
+    for p in range(n):
+        assert seen[p] == list(range(8 * 50)), "pipe %d of %d" % (p, n)
+        assert len(xcds[p]) == 8
