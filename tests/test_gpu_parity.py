@@ -1058,3 +1058,46 @@ def test_random_groups_sweep(lmi, oracle, case):
     finally:
         srv.close()
         feats.free()
+
+
+@pytest.mark.parametrize("streams", [1, 2])
+def test_groups_that_reuse_pipes_wait_for_the_host_link_gather_before(lmi, oracle, streams):
+    """Groups issued back to back on overlapping sets of pipes, nothing fetched in between: a pipe's
+    next batch may only start once the side stream has finished the host-link gather of the one
+    before (one event per group marks that, whichever pipes of it are reused first).  The host-link
+    gather is slowed to one block and most rows miss, so a batch that started early would be
+    overwritten by the rows of its predecessor."""
+    rng = np.random.default_rng(77 + streams)
+    n_nodes, batch, dim, fanout, pipes = 40_000, 500, 128, [10, 5], 8
+    indptr, indices = random_graph(rng, n_nodes, 12, hubs=4, hub_deg=2000)
+    feats = make_features(lmi, rng, n_nodes, dim)
+    srv = lmi.Server(batch, fanout, dim, pipes=pipes, seed=3)
+    ss = [lmi.stream_create() for _ in range(streams)]
+    try:
+        srv.tune("miss_blocks", 1)
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        srv.build_static_cache(n_nodes // 10, lmi.TABLE_RANK)
+        last, issued = {}, 0
+        for rnd in range(14):
+            n = int(rng.integers(1, pipes + 1))
+            plist = [int(x) for x in rng.choice(pipes, n, replace=False)]
+            seeds = [rng.choice(n_nodes, int(rng.integers(batch // 2, batch + 1)), replace=False).astype(np.int32)
+                     for _ in plist]
+            rs = [900 + issued + k for k in range(n)]
+            issued += n
+            if n == 1 and rnd % 2:
+                srv.run_once(seeds[0], rng_seed=rs[0], pipe=plist[0], stream=ss[rnd % streams])
+            else:
+                srv.run_group(plist, [0] * n, seeds=seeds, rng_seeds=rs, stream=ss[rnd % streams])
+            for k, pipe in enumerate(plist):
+                last[pipe] = (seeds[k], rs[k])
+        for pipe, (seeds, r) in sorted(last.items()):
+            g = srv.fetch(pipe=pipe, stream=ss[0])
+            o = oracle.sample_batch(indptr, indices, seeds, fanout, r)
+            assert_batch_equal(g, o)
+            assert g.features.tobytes() == feats.array[o.ids].tobytes(), "pipe %d" % pipe
+        srv.status()
+    finally:
+        srv.close()
+        feats.free()
