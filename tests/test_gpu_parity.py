@@ -1024,7 +1024,8 @@ def test_random_groups_sweep(lmi, oracle, case):
     slot_ref = q = sc = None
     try:
         for key, vals in (("group_miss", [0, 1]), ("protect_hits", [0, 1]), ("fuse_count", [0, 1]),
-                          ("table_epochs", [0, 2, 1 << 30]), ("miss_blocks", [1, 8, 32]), ("split_miss", [0, 1, 2])):
+                          ("table_epochs", [0, 2, 1 << 30]), ("miss_blocks", [1, 8, 32]), ("split_miss", [0, 1, 2]),
+                          ("early_fork", [0, 1])):
             srv.tune(key, int(rng.choice(vals)))
         srv.load_graph(indptr, indices)
         srv.attach_features(feats)
