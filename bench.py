@@ -516,7 +516,8 @@ def main():
     # a group's hit gathers are one launch (on the caller's stream) and so are its host-link
     # gathers (on the side stream)
     split = int(tunes.get("split_miss", 1)) == 1
-    timed_group = args.steps / max(len(group_sizes(args.steps)), 1)   # batches per launch of the timed region
+    # batches per launch of the profiled groups (the library counts the batches of the calls it profiles)
+    timed_group = prof.batches / max(prof.gather_hit_launches, 1) if group > 1 else 1
     hit_batches = timed_group if split else 1
     miss_batches = timed_group if (split and int(tunes.get("group_miss", 1))) else 1
     hit_ms = prof.gather_hit_ms / max(prof.gather_hit_launches, 1)
@@ -599,7 +600,7 @@ def main():
     rr_reads = 1 << 24
     rr_ms = lmi.bench_random_read(info["d_indices"], info["n_edges"] * 4, rr_reads)
     total_rows = prof.gather_hit_rows + prof.gather_miss_rows
-    profiled_batches = int(max(prof.gather_hit_launches * hit_batches, prof.gather_miss_launches * miss_batches))
+    profiled_batches = int(prof.batches)
     out = {
         "metric": "sampled mini-batches/sec", "value": round(args.steps / (t1 - t0), 2), "unit": "batches/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": round(ms_per_step, 4),

@@ -108,7 +108,7 @@ typedef struct lmi_profile {
   double  gather_miss_ms;  int64_t gather_miss_launches; int64_t gather_miss_rows;
   double  sample_ms;       int64_t sample_launches;      /* all kernels of the sampling hops */
   double  lookup_ms;       int64_t lookup_launches;
-  double  batch_ms;        int64_t batches;              /* reserved (0) */
+  double  batch_ms;        int64_t batches;              /* batch_ms reserved (0); batches = mini-batches the profiled calls served */
 } lmi_profile;
 
 /* ---- lifecycle ------------------------------------------------------- */

@@ -56,9 +56,10 @@ hipEvent_t prof_phase(Server *s, hipStream_t st, int *open, int next_kind) {
   return e;
 }
 
-// Start of a batch: decides whether this one is profiled.
-static void prof_batch(Server *s) {
+// Start of a batch, or of a group of n batches served together: decides whether it is profiled.
+static void prof_batch(Server *s, int n = 1) {
   s->prof_on = s->prof_level != 0 && (s->prof_seq++ % std::max(1, s->prof_every)) == 0;
+  if (s->prof_on) s->prof.batches += n;
 }
 
 void prof_kernel_events(Server *s, int kind, hipEvent_t *start, hipEvent_t *stop) {
@@ -794,7 +795,7 @@ int lmi_run_group(lmi_server *h, int n_batches, const int32_t *pipes, void *stre
       if (pipes[j] == pipes[k]) LMI_FAIL(LMI_ERR_ARG, "pipe %d named twice in one group", pipes[k]);
     pp[k] = &s->pipes[pipes[k]];
   }
-  prof_batch(s);
+  prof_batch(s, n_batches);
   for (int k = 0; k < n_batches; ++k)
     LMI_TRY(batch_params(s, *pp[k], st, seeds ? seeds[k] : nullptr, (seeds && n_seeds) ? n_seeds[k] : 0, seeds_location,
                          batch_counters[k], mode, rng_seeds ? rng_seeds[k] : 0, &bps[k]));
