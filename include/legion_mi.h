@@ -18,6 +18,11 @@
  * `stream` arguments are hipStream_t values passed as void* (NULL = the default
  * stream).  Output buffers are owned by the server and borrowed by the caller
  * until the same pipe is used for another batch (engine/server.cu:337,377).
+ * A pipe may be driven from different streams over time: a call that names a pipe
+ * orders its stream behind whatever the pipe's previous batch still has queued, on
+ * the server's side stream or on the stream that carried that batch -- which must
+ * therefore still exist (destroy a stream only after the pipes it drove have been
+ * waited for, lmi_batch_wait + lmi_stream_sync, or used from another stream).
  */
 #ifndef LEGION_MI_H
 #define LEGION_MI_H
@@ -29,7 +34,7 @@
 extern "C" {
 #endif
 
-#define LMI_ABI_VERSION 2
+#define LMI_ABI_VERSION 3
 #define LMI_MAX_HOPS    3   /* the 16-int headers hold 3 hops (INTRABATCH_CON, include/system_config.cuh:47-57) */
 #define LMI_MAX_FANOUT  64  /* one wavefront lane per slot; the reference asserts <= 32 (operator_impl.cu:504) */
 #define LMI_MAX_PIPES   16  /* output buffer sets; the reference uses INTERBATCH_CON = 2 */
@@ -118,6 +123,11 @@ const char *lmi_last_error(void);                               /* thread-local 
 int lmi_server_create(const lmi_config *cfg, lmi_server **out);
 /* Server::Finalize / Runner::Finalize (engine/server.cu:137-170,402-451) */
 int lmi_server_destroy(lmi_server *s);
+/* Adds output buffer sets until the server has `pipes` of them (1..LMI_MAX_PIPES; never removes
+ * one, so views of the existing sets stay valid).  The reference fixes INTERBATCH_CON = 2 at compile
+ * time (include/system_config.cuh:47-57); a runner that issues groups of batches wants two groups'
+ * worth.  Allocates device memory: not inside a batch loop. */
+int lmi_server_pipes(lmi_server *s, int32_t pipes);
 
 /* ---- memory helpers (engine/server_imp.cuh:2-52) ---------------------- */
 int lmi_host_alloc(size_t bytes, void **host_ptr);             /* host_alloc_space: pinned + mapped */
@@ -268,8 +278,13 @@ int lmi_batch_wait(lmi_server *s, int pipe, void *stream);
  * clear != 0) -- a seed id outside [0, n_nodes) (LMI_ERR_BAD_ID; the id was skipped) or a
  * device scan that gave up waiting (LMI_ERR_HIP; that batch is incomplete).  The kernels
  * record it in pinned host memory, so this call reads no device memory and synchronises
- * nothing; a condition of a batch still running shows once that batch is done.
- * lmi_batch_wait returns the same code. */
+ * nothing; a condition of a batch still running shows once that batch is done.  It keeps
+ * reporting the condition until a call with clear != 0 (which reports it one last time).
+ * lmi_batch_wait returns the same code, but only ONCE per condition (to the first wait that
+ * sees it; again after a clear): one bad batch does not fail the wait of every good batch
+ * after it.  Neither call says WHICH batch: the words are read as the host sees them, so the
+ * wait of the faulty batch itself can still pass and a later one report.  A per-batch verdict
+ * is what lmi_batch_counters gives (it synchronises and reads the batch's own flags). */
 int lmi_server_status(lmi_server *s, int clear);
 int lmi_batch_view_get(lmi_server *s, int pipe, lmi_batch_view *out);
 /* Synchronises `stream`, copies both headers to the host, reports a bad seed id. */
@@ -297,6 +312,15 @@ int lmi_bench_copy(size_t bytes, int repeats, double *ms_per_copy);
  * is how the gather kernels are timed.  What a launch of this size can reach at all: a launch of
  * a few hundred MB spends a visible part of its time filling and draining the device. */
 int lmi_bench_copy_launch(size_t bytes, int repeats, double *ms_per_launch);
+/* The ceiling of a gather's SHAPE: a streaming kernel that reads read_bytes and writes write_bytes
+ * per lane and step -- 4:16 (int8 -> fp32), 8:16 (int8 -> fp16), 8:32, or 16:16 (a row mover; with
+ * misalign = 4 both sides sit 4 bytes off a 16-byte boundary, as rows of 16 k + 12 bytes do) --
+ * over `units` such steps, contiguous, no indirection.  launch_by_launch != 0 times every launch
+ * alone, from its own first to its own last wavefront (lmi_bench_copy_launch); 0 times `repeats`
+ * launches back to back (lmi_bench_copy).  A 1:1 copy says little about a kernel that writes twice
+ * what it reads: HBM takes writes more slowly than reads. */
+int lmi_bench_stream(size_t units, int read_bytes, int write_bytes, int misalign, int repeats, int launch_by_launch,
+                     double *ms_per_launch);
 /* Streaming zero-copy read of `bytes` bytes of pinned host memory (from lmi_host_alloc) into
  * HBM, repeated; returns mean ms per pass (the measured host-link ceiling). */
 int lmi_bench_host_read(const void *host_ptr, size_t bytes, int repeats, double *ms_per_pass);

@@ -24,7 +24,7 @@ POLICY_DEGREE, POLICY_PRESAMPLED = 0, 1
 
 # every symbol include/legion_mi.h declares
 ABI_SYMBOLS = [
-    "lmi_abi_version", "lmi_last_error", "lmi_server_create", "lmi_server_destroy",
+    "lmi_abi_version", "lmi_last_error", "lmi_server_create", "lmi_server_destroy", "lmi_server_pipes",
     "lmi_host_alloc", "lmi_host_free", "lmi_device_alloc", "lmi_device_free",
     "lmi_copy_to_host", "lmi_copy_to_device", "lmi_copy_device", "lmi_ipc_export", "lmi_ipc_open", "lmi_ipc_close",
     "lmi_stream_create", "lmi_stream_destroy",
@@ -34,7 +34,7 @@ ABI_SYMBOLS = [
     "lmi_cache_info_get", "lmi_cache_dump", "lmi_op_batch_generate", "lmi_op_random_sample",
     "lmi_op_cache_lookup", "lmi_op_io_submit", "lmi_op_io_complete", "lmi_run_once",
     "lmi_run_group", "lmi_run_once_static", "lmi_batch_wait", "lmi_server_status", "lmi_batch_view_get", "lmi_batch_counters", "lmi_steps_per_epoch", "lmi_profile_enable",
-    "lmi_profile_read", "lmi_tune", "lmi_bench_copy", "lmi_bench_copy_launch", "lmi_bench_host_read", "lmi_bench_random_read", "lmi_synth_graph", "lmi_synth_trainset",
+    "lmi_profile_read", "lmi_tune", "lmi_bench_copy", "lmi_bench_copy_launch", "lmi_bench_stream", "lmi_bench_host_read", "lmi_bench_random_read", "lmi_synth_graph", "lmi_synth_trainset",
     "lmi_synth_features",
 ]
 
@@ -103,6 +103,7 @@ def lib():
         L.lmi_stream_sync.argtypes = [C.c_void_p]
         L.lmi_server_create.argtypes = [C.POINTER(Config), C.POINTER(C.c_void_p)]
         L.lmi_server_destroy.argtypes = [C.c_void_p]
+        L.lmi_server_pipes.argtypes = [C.c_void_p, C.c_int32]
         L.lmi_graph_load.argtypes = [C.c_void_p, C.c_void_p, C.c_void_p, C.c_int64, C.c_int64, C.c_int]
         L.lmi_features_attach.argtypes = [C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
         L.lmi_idset_load.argtypes = [C.c_void_p, C.c_int, C.c_void_p, C.c_void_p, C.c_int64, C.c_int]
@@ -139,6 +140,7 @@ def lib():
         L.lmi_tune.argtypes = [C.c_void_p, C.c_char_p, C.c_int64]
         L.lmi_bench_copy.argtypes = [C.c_size_t, C.c_int, C.POINTER(C.c_double)]
         L.lmi_bench_copy_launch.argtypes = [C.c_size_t, C.c_int, C.POINTER(C.c_double)]
+        L.lmi_bench_stream.argtypes = [C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double)]
         L.lmi_bench_host_read.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.POINTER(C.c_double)]
         L.lmi_bench_random_read.argtypes = [C.c_void_p, C.c_size_t, C.c_int64, C.c_int, C.POINTER(C.c_double)]
         L.lmi_synth_graph.argtypes = [C.c_uint64, C.c_void_p, C.c_int32, C.c_int64, C.c_int32,
@@ -205,6 +207,11 @@ class Server:
         if self.h:
             check(lib().lmi_server_destroy(self.h))
             self.h = None
+
+    def add_pipes(self, pipes):
+        """Grow the server to `pipes` output buffer sets (lmi_server_pipes)."""
+        check(lib().lmi_server_pipes(self.h, pipes))
+        self.cfg.pipes = max(int(self.cfg.pipes), pipes)
 
     # storage -----------------------------------------------------------------
     def load_graph(self, indptr, indices):
@@ -384,6 +391,13 @@ def bench_copy_launch(nbytes, repeats=10):
     """Mean ms of one copy launch of nbytes, each launch alone on the device and timed by its own events."""
     ms = C.c_double()
     check(lib().lmi_bench_copy_launch(nbytes, repeats, C.byref(ms)))
+    return ms.value
+
+
+def bench_stream(units, read_bytes, write_bytes, misalign=0, repeats=10, launch_by_launch=False):
+    """Mean ms of one launch of the streaming kernel that reads read_bytes and writes write_bytes per unit."""
+    ms = C.c_double()
+    check(lib().lmi_bench_stream(int(units), read_bytes, write_bytes, misalign, repeats, int(launch_by_launch), C.byref(ms)))
     return ms.value
 
 

@@ -5,6 +5,7 @@
 #include <cstring>
 #include <mutex>
 #include <new>
+#include <type_traits>
 
 #include <hip/hip_ext.h>
 
@@ -112,6 +113,7 @@ static void pipe_free(Pipe &p) {
   if (p.graph) (void)hipGraphDestroy(p.graph);
   if (p.fork) (void)hipEventDestroy(p.fork);
   if (p.join) (void)hipEventDestroy(p.join);
+  if (p.handover) (void)hipEventDestroy(p.handover);
   p = Pipe{};
 }
 
@@ -161,6 +163,7 @@ static int pipe_alloc(Server *s, Pipe &p) {
   LMI_TRY(dmalloc(&p.seed_stage, s->cfg.batch_size));
   LMI_HIP(hipEventCreateWithFlags(&p.fork, hipEventDisableTiming));
   LMI_HIP(hipEventCreateWithFlags(&p.join, hipEventDisableTiming));
+  LMI_HIP(hipEventCreateWithFlags(&p.handover, hipEventDisableTiming));
   return LMI_OK;
 }
 
@@ -180,6 +183,56 @@ static __global__ __launch_bounds__(256) void copy_kernel(const cp_u32x4 *__rest
 #pragma unroll
     for (int u = 0; u < 4; ++u)
       if (i + (size_t)u * blockDim.x < n) __builtin_nontemporal_store(v[u], dst + i + (size_t)u * blockDim.x);
+  }
+}
+
+// The copy with a gather's read : write shape but none of its indirection: a lane reads RB bytes and
+// writes WB bytes per step (8 : 16 is the int8 -> fp16 gather, 4 : 16 int8 -> fp32, 16 : 16 a row
+// mover), four steps in flight, each block on contiguous chunks.  A4 offsets both sides by 4 bytes and
+// lets the 16-byte accesses assume no more than 4-byte alignment, as rows of 4 k + 4 bytes force.
+typedef uint32_t cp_u32x2 __attribute__((ext_vector_type(2)));
+typedef cp_u32x4 cp_u32x4_a4 __attribute__((aligned(4)));
+template <int RB> struct StreamIn;
+template <> struct StreamIn<16> { typedef cp_u32x4 type; };
+template <> struct StreamIn<8> { typedef cp_u32x2 type; };
+template <> struct StreamIn<4> { typedef uint32_t type; };
+template <int RB, int WB, bool A4>
+static __global__ __launch_bounds__(256) void stream_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
+                                                            size_t n) {
+  typedef typename StreamIn<RB>::type IN;
+  typedef typename std::conditional<A4, cp_u32x4_a4, cp_u32x4>::type OUT;
+  static_assert(WB % 16 == 0 && (!A4 || RB == 16), "whole 16-byte stores; the unaligned variant is the 16 : 16 one");
+  const size_t stride = (size_t)gridDim.x * blockDim.x * 4;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x * 4 + threadIdx.x; i < n; i += stride) {
+    union {
+      IN v;
+      OUT o;
+      uint32_t w[4];
+    } r[4];
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const size_t j = i + (size_t)u * blockDim.x;
+      if (j < n) {
+        if (A4) r[u].o = __builtin_nontemporal_load(reinterpret_cast<const OUT *>(src + j * RB));
+        else r[u].v = __builtin_nontemporal_load(reinterpret_cast<const IN *>(src + j * RB));
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const size_t j = i + (size_t)u * blockDim.x;
+      if (j < n) {
+        cp_u32x4 o;
+        o.x = r[u].w[0];
+        o.y = RB >= 8 ? r[u].w[1] : r[u].w[0] + 1u;
+        o.z = RB >= 16 ? r[u].w[2] : r[u].w[0] + 2u;
+        o.w = RB >= 16 ? r[u].w[3] : r[u].w[0] + 3u;
+#pragma unroll
+        for (int k = 0; k < WB / 16; ++k) {
+          o.x += (uint32_t)k;
+          __builtin_nontemporal_store((OUT)o, reinterpret_cast<OUT *>(dst + j * WB + 16 * k));
+        }
+      }
+    }
   }
 }
 
@@ -209,7 +262,6 @@ static __device__ __align__(256) unsigned char scratch[LMI_STATIC_SCRATCH_BYTES]
 constexpr int kMaxDevices = 16;
 struct StaticScratch {
   unsigned char *ptr = nullptr;  // device address of `scratch` on this device
-  Pipe pipe;                     // host-side bookkeeping of the one "pipe" that lives in it
 };
 static StaticScratch g_static[kMaxDevices];
 static std::mutex g_static_mu;
@@ -309,6 +361,25 @@ int lmi_server_create(const lmi_config *cfg, lmi_server **out) {
     return rc;
   }
   *out = reinterpret_cast<lmi_server *>(s);
+  return LMI_OK;
+}
+
+int lmi_server_pipes(lmi_server *h, int32_t pipes) {
+  Server *s = reinterpret_cast<Server *>(h);
+  if (!s) LMI_FAIL(LMI_ERR_ARG, "null server");
+  if (pipes < 1 || pipes > LMI_MAX_PIPES) LMI_FAIL(LMI_ERR_ARG, "pipes must be 1..%d", LMI_MAX_PIPES);
+  const size_t have = s->pipes.size();
+  if ((size_t)pipes <= have) return LMI_OK;  // never shrinks: callers may hold views of the existing sets
+  LMI_HIP(hipSetDevice(s->cfg.device_id));
+  s->pipes.resize((size_t)pipes);  // moves the host-side records only; device buffers stay where they are
+  int rc = LMI_OK;
+  for (size_t k = have; k < s->pipes.size() && rc == LMI_OK; ++k) rc = pipe_alloc(s, s->pipes[k]);
+  if (rc != LMI_OK) {
+    for (size_t k = have; k < s->pipes.size(); ++k) pipe_free(s->pipes[k]);
+    s->pipes.resize(have);
+    return rc;
+  }
+  s->cfg.pipes = pipes;
   return LMI_OK;
 }
 
@@ -630,6 +701,7 @@ int lmi_op_batch_generate(lmi_server *h, int pipe, void *stream, const int32_t *
   BatchParams bp{};
   prof_batch(s);
   LMI_TRY(pipe_join(p, st));
+  pipe_begin(p, st);
   LMI_TRY(batch_params(s, p, st, seeds, n, seeds_location, batch_counter, mode, rng_seed, &bp));
   Pipe *pp[1] = {&p};
   return launch_batch_generate(s, pp, &bp, 1, st, true);
@@ -642,6 +714,8 @@ int lmi_op_random_sample(lmi_server *h, int pipe, void *stream, int hop) {
   Pipe &p = s->pipes[pipe];
   if (hop != p.hops_done || hop >= s->cfg.hops) LMI_FAIL(LMI_ERR_ARG, "hop %d out of order (next is %d)", hop, p.hops_done);
   hipStream_t st = (hipStream_t)stream;
+  LMI_TRY(pipe_handover(p, st));  // a stream other than the one of the operator before is ordered behind it
+  pipe_begin(p, st);
   prof_phase(s, st, &s->prof_open, PROF_SAMPLE);
   Pipe *pp[1] = {&p};
   LMI_TRY(launch_hop(s, pp, 1, st, hop, false, false));
@@ -657,6 +731,7 @@ int lmi_op_cache_lookup(lmi_server *h, int pipe, void *stream, int segment) {
   if (segment < 0 || segment > p.hops_done) LMI_FAIL(LMI_ERR_ARG, "segment %d not sampled yet", segment);
   hipStream_t st = (hipStream_t)stream;
   LMI_TRY(pipe_join(p, st));
+  pipe_begin(p, st);
   LMI_TRY(lru_wait_ready(s, st));
   prof_phase(s, st, &s->prof_open, PROF_LOOKUP);
   Pipe *pp[1] = {&p};
@@ -670,6 +745,8 @@ int lmi_op_hotness(lmi_server *h, int pipe, void *stream) {
   Server *s = reinterpret_cast<Server *>(h);
   LMI_TRY(check_pipe(s, pipe));
   LMI_TRY(ready(s));
+  LMI_TRY(pipe_join(s->pipes[pipe], (hipStream_t)stream));
+  pipe_begin(s->pipes[pipe], (hipStream_t)stream);
   return launch_hotness(s, s->pipes[pipe], (hipStream_t)stream);
 }
 
@@ -682,6 +759,7 @@ int lmi_presample(lmi_server *h, int pipe, void *stream, int mode, int32_t first
   for (int32_t b = first_batch; b < first_batch + n_batches; ++b) {
     BatchParams bp{};
     LMI_TRY(pipe_join(p, st));
+    pipe_begin(p, st);
     const int tick = s->lru_tick;
     LMI_TRY(batch_params(s, p, st, nullptr, 0, LMI_LOC_DEVICE, b, mode, 0, &bp));
     s->lru_tick = tick;  // presampling does not age the LRU cache
@@ -705,6 +783,7 @@ int lmi_op_io_complete(lmi_server *h, int pipe, void *stream) {
   Pipe &p = s->pipes[pipe];
   hipStream_t st = (hipStream_t)stream;
   LMI_TRY(pipe_join(p, st));
+  pipe_begin(p, st);
   LMI_TRY(launch_lru_insert(s, p, st, s->cfg.hops + 1));
   return LMI_OK;
 }
@@ -744,8 +823,9 @@ static int capture_batch_graph(Server *s, Pipe &p, hipStream_t st, const BatchPa
 }
 
 // One batch on each of n pipes, served by the same launches.
+// The caller has ordered `st` behind the pipes' previous batches (pipes_join) before it staged the seeds.
 static int run_group(Server *s, Pipe *const *pp, const BatchParams *bps, int n, hipStream_t st) {
-  LMI_TRY(pipes_join(pp, n, st));  // a pipe's previous batch may still be gathering misses
+  for (int k = 0; k < n; ++k) pipe_begin(*pp[k], st);
   prof_phase(s, st, &s->prof_open, PROF_SAMPLE);
   if (s->use_graph && st != nullptr && n == 1) {  // the legacy default stream cannot be captured
     Pipe &p = *pp[0];
@@ -773,6 +853,9 @@ int lmi_run_once(lmi_server *h, int pipe, void *stream, const int32_t *seeds, in
   hipStream_t st = (hipStream_t)stream;
   BatchParams bp{};
   prof_batch(s);
+  // a pipe's previous batch may still be gathering misses, or sit on another stream: only behind it may
+  // this batch's first command, the copy of host seeds into the pipe's staging buffer, be queued
+  LMI_TRY(pipes_join(pp, 1, st));
   LMI_TRY(batch_params(s, *pp[0], st, seeds, n, seeds_location, batch_counter, mode, rng_seed, &bp));
   return run_group(s, pp, &bp, 1, st);
 }
@@ -796,6 +879,7 @@ int lmi_run_group(lmi_server *h, int n_batches, const int32_t *pipes, void *stre
     pp[k] = &s->pipes[pipes[k]];
   }
   prof_batch(s, n_batches);
+  LMI_TRY(pipes_join(pp, n_batches, st));  // before the seeds are staged: see lmi_run_once
   for (int k = 0; k < n_batches; ++k)
     LMI_TRY(batch_params(s, *pp[k], st, seeds ? seeds[k] : nullptr, (seeds && n_seeds) ? n_seeds[k] : 0, seeds_location,
                          batch_counters[k], mode, rng_seeds ? rng_seeds[k] : 0, &bps[k]));
@@ -831,10 +915,12 @@ int lmi_run_once_static(lmi_server *h, void *stream, const int32_t *seeds, int32
     LMI_FAIL(LMI_ERR_STATE, "no static scratch on device %d", device);
   LMI_HIP(hipSetDevice(device));
   unsigned char *ptr = g_static[device].ptr;
-  Pipe &p = g_static[device].pipe;
-  // The table is wiped by every call (no epoch kept on the host): another server may have used the
-  // array last, and the launches of a call must depend on nothing but its arguments and the device
-  // memory they name, so that a caller who captured them in a graph can replay it.
+  // The "pipe" of this call lives on the stack: nothing of it outlasts the call, so two servers on one
+  // GPU share the device array (the documented race) but no host-side state.  Its table is wiped by
+  // every call (no epoch kept on the host): another server may have used the array last, and the
+  // launches of a call must depend on nothing but its arguments and the device memory they name, so
+  // that a caller who captured them in a graph can replay it.
+  Pipe p;
   p.table_dirty = true;
   p.ids = out->ids;
   p.features = out->features;
@@ -872,7 +958,6 @@ int lmi_run_once_static(lmi_server *h, void *stream, const int32_t *seeds, int32
       rc = LMI_ERR_HIP;
     }
   }
-  if (rc != LMI_OK) p.table_dirty = true;  // a batch cut short may have left half an epoch behind
   s->prof_on = prof;
   return rc;
 }
@@ -881,7 +966,10 @@ int lmi_run_once_static(lmi_server *h, void *stream, const int32_t *seeds, int32
 static int fault_status(Server *s, int clear) {
   if (!s->fault_host) return LMI_OK;
   const int32_t bad = s->fault_host[kFaultBadId], scan = s->fault_host[kFaultScan];
-  if (clear) s->fault_host[kFaultBadId] = s->fault_host[kFaultScan] = 0;
+  if (clear) {
+    s->fault_host[kFaultBadId] = s->fault_host[kFaultScan] = 0;
+    s->fault_told[kFaultBadId] = s->fault_told[kFaultScan] = false;
+  }
   if (scan) LMI_FAIL(LMI_ERR_HIP, "a device scan timed out waiting for an earlier tile: that batch is incomplete");
   if (bad)
     LMI_FAIL(LMI_ERR_BAD_ID, "a seed id outside [0, %lld) was seen on the device and skipped", (long long)s->n_nodes);
@@ -894,11 +982,26 @@ int lmi_server_status(lmi_server *h, int clear) {
   return fault_status(s, clear);
 }
 
+// The same words for lmi_batch_wait: a condition is reported by the first call that sees it and
+// not again (lmi_server_status keeps reporting it until it is cleared), so that one bad batch does
+// not fail the wait of every good batch after it.
+static int fault_status_once(Server *s) {
+  if (!s->fault_host) return LMI_OK;
+  const bool scan = s->fault_host[kFaultScan] != 0 && !s->fault_told[kFaultScan];
+  const bool bad = s->fault_host[kFaultBadId] != 0 && !s->fault_told[kFaultBadId];
+  if (scan) s->fault_told[kFaultScan] = true;
+  if (bad) s->fault_told[kFaultBadId] = true;
+  if (scan) LMI_FAIL(LMI_ERR_HIP, "a device scan timed out waiting for an earlier tile: that batch is incomplete");
+  if (bad)
+    LMI_FAIL(LMI_ERR_BAD_ID, "a seed id outside [0, %lld) was seen on the device and skipped", (long long)s->n_nodes);
+  return LMI_OK;
+}
+
 int lmi_batch_wait(lmi_server *h, int pipe, void *stream) {
   Server *s = reinterpret_cast<Server *>(h);
   LMI_TRY(check_pipe(s, pipe));
   LMI_TRY(pipe_join(s->pipes[pipe], (hipStream_t)stream));
-  return fault_status(s, 0);
+  return fault_status_once(s);
 }
 
 // ------------------------------------------------------------------ outputs
@@ -1142,6 +1245,54 @@ int lmi_bench_copy_launch(size_t bytes, int repeats, double *ms_per_launch) {
   }
   *ms_per_launch = total / repeats;
   return LMI_OK;
+}
+
+int lmi_bench_stream(size_t units, int read_bytes, int write_bytes, int misalign, int repeats, int launch_by_launch,
+                     double *ms_per_launch) {
+  if (!ms_per_launch || repeats < 1 || units < 1) LMI_FAIL(LMI_ERR_ARG, "bad argument");
+  const int shape = read_bytes * 100 + write_bytes;
+  if (shape != 416 && shape != 816 && shape != 832 && shape != 1616)
+    LMI_FAIL(LMI_ERR_ARG, "read : write bytes per unit must be 4:16, 8:16, 8:32 or 16:16");
+  if (misalign != 0 && (misalign != 4 || shape != 1616)) LMI_FAIL(LMI_ERR_ARG, "misalign is 0, or 4 with 16:16");
+  BenchScratch m;
+  LMI_HIP(hipMalloc(&m.a, units * read_bytes + 64));
+  LMI_HIP(hipMalloc(&m.b, units * write_bytes + 64));
+  LMI_HIP(hipMemset(m.a, 1, units * read_bytes + 64));
+  LMI_TRY(m.events());
+  const uint8_t *src = (const uint8_t *)m.a + misalign;
+  uint8_t *dst = (uint8_t *)m.b + misalign;
+  const int grid = (int)std::max<size_t>(1, std::min<size_t>(units / (256 * 4), 16384));
+  auto launch = [&](hipEvent_t e0, hipEvent_t e1) {
+#define LMI_STREAM(RB_, WB_, A4_)                                                                                   \
+  if (e0)                                                                                                           \
+    hipExtLaunchKernelGGL((stream_kernel<RB_, WB_, A4_>), dim3(grid), dim3(256), 0, 0, e0, e1, 0, src, dst, units);  \
+  else                                                                                                              \
+    hipLaunchKernelGGL((stream_kernel<RB_, WB_, A4_>), dim3(grid), dim3(256), 0, 0, src, dst, units)
+    if (shape == 416) { LMI_STREAM(4, 16, false); }
+    else if (shape == 816) { LMI_STREAM(8, 16, false); }
+    else if (shape == 832) { LMI_STREAM(8, 32, false); }
+    else if (misalign) { LMI_STREAM(16, 16, true); }
+    else { LMI_STREAM(16, 16, false); }
+#undef LMI_STREAM
+  };
+  if (launch_by_launch) {  // each launch alone on the device, timed from its own first to its own last wavefront
+    double total = 0.0;
+    for (int r = -1; r < repeats; ++r) {
+      launch(m.e0, m.e1);
+      LMI_HIP(hipGetLastError());
+      LMI_HIP(hipDeviceSynchronize());
+      float ms = 0;
+      LMI_HIP(hipEventElapsedTime(&ms, m.e0, m.e1));
+      if (r >= 0) total += ms;
+    }
+    *ms_per_launch = total / repeats;
+    return LMI_OK;
+  }
+  launch(nullptr, nullptr);
+  LMI_HIP(hipEventRecord(m.e0, 0));
+  for (int r = 0; r < repeats; ++r) launch(nullptr, nullptr);
+  LMI_HIP(hipGetLastError());
+  return m.elapsed(repeats, ms_per_launch);
 }
 
 }  // extern "C"

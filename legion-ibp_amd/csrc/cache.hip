@@ -794,35 +794,63 @@ int launch_lookup(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg_fir
   return LMI_OK;
 }
 
-// Orders `st` behind the pipe's work on the side stream.  A wait on another queue's
-// event holds a stream up for about 10 us even when the event fired long ago, so the
-// wait is only queued when the host cannot already see the event as complete.
-int pipe_join(Pipe &p, hipStream_t st) {
-  if (p.side_pending) {
-    const hipError_t q = hipEventQuery(p.join_of);
-    if (q != hipSuccess) {
-      (void)hipGetLastError();  // "not ready" is an answer, not a failure
-      LMI_HIP(hipStreamWaitEvent(st, p.join_of, 0));
-    }
-    p.side_pending = false;
+// Orders `st` behind the pipe's last batch.  Its side-stream work ends with the event `join_of`; a
+// wait on another queue's event holds a stream up for about 10 us even when the event fired long
+// ago, so that wait is only queued when the host cannot already see the event as complete.  Work
+// of the batch that `join_of` does not cover sits on the caller's stream that carried the batch:
+// the same stream orders itself, another one is put behind an event recorded there now (at that
+// stream's present tail, which is at or behind the batch's last kernel).
+int pipe_handover(Pipe &p, hipStream_t st) {
+  if (p.tail_unjoined && p.last_stream != st && p.handover) {
+    LMI_HIP(hipEventRecord(p.handover, p.last_stream));
+    LMI_HIP(hipStreamWaitEvent(st, p.handover, 0));
+    p.last_stream = st;  // `st` now carries the order
   }
   return LMI_OK;
 }
 
+int pipe_join(Pipe &p, hipStream_t st) {
+  LMI_TRY(pipe_handover(p, st));
+  if (!p.side_pending || (p.join_waited && p.join_waiter == st)) return LMI_OK;
+  if (hipEventQuery(p.join_of) == hipSuccess) {
+    p.side_pending = false;  // complete: no stream has to wait any more
+    return LMI_OK;
+  }
+  (void)hipGetLastError();  // "not ready" is an answer, not a failure
+  LMI_HIP(hipStreamWaitEvent(st, p.join_of, 0));
+  p.join_waited = true;  // this stream is in order; another one that names the pipe later still has to wait
+  p.join_waiter = st;
+  return LMI_OK;
+}
+
+// A join event was just recorded for the pipe on the side stream.
+static void pipe_side_owes(Pipe &p, hipEvent_t join_of) {
+  p.join_of = join_of;
+  p.side_pending = true;
+  p.join_waited = false;
+}
+
 int pipes_join(Pipe *const *pp, int n, hipStream_t st) {
   hipEvent_t seen[LMI_MAX_GROUP];
+  bool done[LMI_MAX_GROUP];
   int n_seen = 0;
   for (int k = 0; k < n; ++k) {
     Pipe &p = *pp[k];
+    LMI_TRY(pipe_handover(p, st));
     if (!p.side_pending) continue;
-    bool dup = false;
-    for (int j = 0; j < n_seen; ++j) dup = dup || seen[j] == p.join_of;
-    if (dup) {
-      p.side_pending = false;  // `st` already waits for (or has seen) this event
+    int dup = -1;
+    for (int j = 0; j < n_seen; ++j)
+      if (seen[j] == p.join_of) dup = j;
+    if (dup >= 0) {  // `st` already waits for this event, or has seen it complete
+      if (done[dup]) p.side_pending = false;
+      else p.join_waited = true, p.join_waiter = st;
       continue;
     }
-    if (n_seen < LMI_MAX_GROUP) seen[n_seen++] = p.join_of;
     LMI_TRY(pipe_join(p, st));
+    if (n_seen < LMI_MAX_GROUP) {
+      seen[n_seen] = p.join_of;
+      done[n_seen++] = !p.side_pending;
+    }
   }
   return LMI_OK;
 }
@@ -987,6 +1015,7 @@ int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int s
   hipEvent_t closing = prof_phase(s, st, &s->prof_open, -1);
   if (mode == 0) {
     for (int k = 0; k < n; ++k) {
+      pp[k]->tail_unjoined = true;  // everything is on the caller's stream
       if (have_cache) LMI_TRY(launch_hits(s, pp + k, 1, st, seg, seg_last));
       LMI_TRY(launch_misses(s, pp + k, 1, st, seg, seg_last));
       if (lru_lists > 0) LMI_TRY(launch_lru_insert(s, *pp[k], st, lru_lists));
@@ -994,6 +1023,8 @@ int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int s
     return LMI_OK;
   }
   hipEvent_t fork = closing;  // when mode 2 forks right here, the closing event doubles as the fork
+  if (mode == 2)
+    for (int k = 0; k < n; ++k) pp[k]->tail_unjoined = false;  // both gathers run behind the fork
   if (mode == 1) {
     // Host-link reads in flight halve the HBM gather's bandwidth: optionally hold the hits back
     // until the side stream has drained the host-link gathers issued before (other pipes').
@@ -1008,7 +1039,11 @@ int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int s
     // LRU batches are host-link-bound (a fifth of their rows miss): their host-link gather starts
     // beside the HBM gather instead of behind it.  The insertion that follows it on the side stream
     // only overwrites ways this batch's lookup did not touch, so the hits never read a row it writes.
-    const bool early = (lru_lists > 0 && s->lru_early_miss) || (lru_lists == 0 && s->early_fork);
+    const bool early = (lru_lists > 0 && s->lru_early_miss) ||
+                       (lru_lists == 0 && (s->early_fork == 1 || (s->early_fork == 2 && n > 1)));
+    // behind a late fork the join event covers the whole batch; ahead of an early one the HBM gather stays
+    // on the caller's stream alone
+    for (int k = 0; k < n; ++k) pp[k]->tail_unjoined = early;
     fork = nullptr;
     if (early) {
       fork = pp[0]->fork;
@@ -1026,10 +1061,7 @@ int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int s
   if (misses_together) LMI_TRY(launch_misses(s, pp, n, s->side, seg, seg_last));
   if (misses_together) {  // nothing else of the group goes to the side stream: one event for all its pipes
     LMI_HIP(hipEventRecord(pp[0]->join, s->side));
-    for (int k = 0; k < n; ++k) {
-      pp[k]->join_of = pp[0]->join;
-      pp[k]->side_pending = true;
-    }
+    for (int k = 0; k < n; ++k) pipe_side_owes(*pp[k], pp[0]->join);
   }
   for (int k = 0; k < n && !misses_together; ++k) {
     Pipe &p = *pp[k];
@@ -1037,8 +1069,7 @@ int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int s
     LMI_TRY(launch_misses(s, pp + k, 1, s->side, seg, seg_last));
     if (lru_lists > 0) LMI_TRY(launch_lru_insert(s, p, s->side, lru_lists));  // reads the rows just gathered
     LMI_HIP(hipEventRecord(p.join, s->side));
-    p.join_of = p.join;
-    p.side_pending = true;
+    pipe_side_owes(p, p.join);
     // an LRU insertion that comes later on the caller's stream copies the gathered rows: join now
     if (s->cache_kind == LMI_CACHE_LRU && lru_lists == 0) LMI_TRY(pipe_join(p, st));
   }

@@ -106,7 +106,16 @@ struct Pipe {
   // first pipe of the group its misses were gathered with (one record and one wait per group: a
   // wait on another queue's event costs a stream about 10 us, fired or not).
   hipEvent_t join_of = nullptr;
-  bool side_pending = false;   // the side stream still owes this pipe's miss rows (join_of not yet waited on)
+  bool side_pending = false;   // the side stream may still owe this pipe's miss rows (join_of not yet seen complete)
+  bool join_waited = false;    // a wait for join_of has been queued on join_waiter: that stream needs no second one,
+  hipStream_t join_waiter = nullptr;  // any other stream still does
+  // The caller's stream that carried the pipe's last batch, and whether that stream still holds work
+  // of the batch that `join_of` does not cover (everything when no side stream is used; the HBM
+  // gather when the side stream was released ahead of it).  A later call that uses the pipe from
+  // ANOTHER stream is then ordered behind `last_stream` through `handover` (pipe_join).
+  hipStream_t last_stream = nullptr;
+  bool tail_unjoined = false;
+  hipEvent_t handover = nullptr;
   int32_t *seed_stage = nullptr;  // [batch_size] host seeds land here
   int32_t n_seeds = 0;
   int32_t hops_done = 0;
@@ -173,7 +182,9 @@ struct Server {
   hipEvent_t side_idle = nullptr;  // recorded behind the last host-link gather issued on the side stream
   bool side_busy = false;
   int protect_hits = 0;            // 1: HBM gathers wait until earlier host-link gathers have drained
-  int early_fork = 0;              // 1: the side stream is released before the HBM gather is launched, not behind it
+  int early_fork = 2;              // when the side stream is released ahead of the HBM gather instead of behind it:
+                                   // 0 never, 1 always, 2 for groups of batches (their host-link gather then starts a
+                                   // whole HBM gather earlier, which is what a short run or a first batch waits for)
   int lru_early_miss = 1;          // 1: with the LRU cache the host-link gather starts beside the HBM gather
   int group_miss = 1;              // 1: the host-link gathers of a group of batches are one launch
   hipEvent_t lru_ready = nullptr;  // recorded when an LRU insertion has settled keys and ticks: the next lookup waits for it
@@ -184,6 +195,7 @@ struct Server {
   // [0] a seed id outside [0, n_nodes), [1] a look-back scan gave up
   volatile int32_t *fault_host = nullptr;
   int32_t *fault_dev = nullptr;  // the same words as the device addresses them
+  bool fault_told[2] = {false, false};  // lmi_batch_wait has reported the condition once already
   // pipes
   std::vector<Pipe> pipes;
   hipStream_t side = nullptr;  // server-owned second stream for gathers that must not hold up the caller's stream
@@ -192,7 +204,8 @@ struct Server {
   int gather_vec = 0;     // bytes per lane access (0 = widest that fits: 16)
   int gather_unroll = 0;  // rows (units) in flight per lane; 0 = the mover's own best: 1 for the lane-group mover
                           // (a few percent ahead of 4), 2 for the tiled movers
-  int gather_tile_rows = 0;  // tiled movers: rows per tile (0 = about 32 KB worth, 4..64)
+  int gather_tile_rows = 0;  // tiled movers: rows per tile; 0 = the mover's own rule: about 8 KB worth of rows,
+                             // 2..64 (256 for rows under 128 bytes); the tiled int8 gather takes 32
   int gather_blocks = 0;  // blocks per pipe; 0 = auto (auto_gather_blocks)
   int gather_nt = 1;      // non-temporal output stores
   int gather_flat = 0;    // 0: rows that a lane group does not fit exactly use the tiled mover; 1: every row; 2: none
@@ -273,7 +286,13 @@ int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int s
 int launch_lru_insert(Server *s, Pipe &p, hipStream_t st, int n_lists);
 int lru_wait_ready(Server *s, hipStream_t st);
 int lru_wait_copied(Server *s, hipStream_t st);  // orders `st` behind the last LRU insertion
-int pipe_join(Pipe &p, hipStream_t st);  // make `st` wait for the pipe's side-stream work
+int pipe_join(Pipe &p, hipStream_t st);  // make `st` wait for the pipe's last batch, wherever it ran
+int pipe_handover(Pipe &p, hipStream_t st);  // only for what another caller's stream still holds of it
+// `st` is about to carry work of the pipe's next batch (after pipe_join)
+inline void pipe_begin(Pipe &p, hipStream_t st) {
+  p.last_stream = st;
+  p.tail_unjoined = true;
+}
 // the same for n pipes, each distinct event waited on once
 int pipes_join(Pipe *const *pp, int n, hipStream_t st);
 int cache_dump(Server *s, int32_t *slot_of, int64_t n, int32_t *aux);

@@ -122,6 +122,7 @@ class GPURunner : public Runner {
     hops_ = (int)params->fanout.size();
     device_ = params->device_id;
     LMI_MUST(lmi_stream_create(&stream_));
+    LMI_MUST(lmi_stream_create(&post_stream_));
     if (IPCEnv *ipc = (IPCEnv *)params->ipc) {  // engine/server.cu:256
       lmi_batch_view v;
       LMI_MUST(lmi_batch_view_get((lmi_server *)params->env, 0, &v));
@@ -175,29 +176,56 @@ class GPURunner : public Runner {
       run_table(params, local, mode, false);
     }
     const bool handoff = ipc && ipc->HandoffEnabled();
-    if (handoff || !params->defer_join) LMI_MUST(lmi_batch_wait((lmi_server *)params->env, pipe_, stream_));
     if (handoff) {
-      LMI_MUST(lmi_stream_sync(stream_));  // the batch is complete before the trainer is told
-      // a batch a kernel flagged (bad seed id, scan that gave up) is never handed over: stop here,
-      // as the reference stops on any device error (engine/memorypool.cuh:9-17)
-      LMI_MUST(lmi_server_status((lmi_server *)params->env, 0));
-      if (ipc->FeaturesInParts(device_)) {  // a feature buffer too large to share whole goes over in pieces
-        int32_t nc[16], ec[16];
-        LMI_MUST(lmi_batch_counters((lmi_server *)params->env, pipe_, stream_, nc, ec));
-        ipc->StageFeatures(device_, pipe_, nc[9 + hops_], stream_);
-        LMI_MUST(lmi_stream_sync(stream_));
+      // The batch is posted once it is complete.  With defer_post the one before it is posted now and
+      // this one by the next call (or Flush): the device then always has the next batch queued while
+      // the host waits for one to finish, and that batch's host-link gather overlaps this one's sampling.
+      if (params->defer_post) {
+        if (unposted_ >= 0) post(params, unposted_);
+        unposted_ = pipe_;
+      } else {
+        post(params, pipe_);
       }
-      ipc->IPCPost(device_, pipe_);
+    } else if (!params->defer_join) {
+      LMI_MUST(lmi_batch_wait((lmi_server *)params->env, pipe_, stream_));
     }
   }
+  // `count` consecutive batches of the schedule, first = params->global_batch_id, all of one mode,
+  // issued together on `count` output buffer sets taken in turn (params->pipes of them exist).
+  void RunGroup(RunnerParams *params, int count, int *pipes_out) override {
+    IPCEnv *ipc = (IPCEnv *)params->ipc;
+    if (count < 1 || count > LMI_MAX_GROUP || count > params->pipes) {
+      std::fprintf(stderr, "a group holds 1..%d batches and no more than there are buffer sets\n", LMI_MAX_GROUP);
+      std::exit(EXIT_FAILURE);
+    }
+    int32_t pipes[LMI_MAX_GROUP], counters[LMI_MAX_GROUP];
+    int mode = params->mode;
+    if (ipc) mode = ipc->GetCurrentMode(params->global_batch_id);
+    for (int k = 0; k < count; ++k) {
+      pipes[k] = next_pipe_;
+      next_pipe_ = (next_pipe_ + 1) % params->pipes;
+      counters[k] = ipc ? ipc->GetLocalBatchId(params->global_batch_id + k) : params->global_batch_id + k;
+      if (pipes_out) pipes_out[k] = pipes[k];
+    }
+    pipe_ = pipes[count - 1];
+    LMI_MUST(lmi_run_group((lmi_server *)params->env, count, pipes, stream_, nullptr, nullptr, LMI_LOC_DEVICE, counters,
+                           mode, nullptr));
+  }
+  void Flush(RunnerParams *params) override {
+    if (unposted_ >= 0) post(params, unposted_);
+    unposted_ = -1;
+  }
   void Finalize(RunnerParams *params) override {
+    Flush(params);
     // the trainer must have released the last batch before its buffers go away
     if (IPCEnv *ipc = (IPCEnv *)params->ipc)
       if (ran_) ipc->IPCWait(device_, pipe_);
     if (stream_) {
       LMI_MUST(lmi_stream_sync(stream_));
+      LMI_MUST(lmi_stream_sync(post_stream_));
+      LMI_MUST(lmi_stream_destroy(post_stream_));
       LMI_MUST(lmi_stream_destroy(stream_));
-      stream_ = nullptr;
+      stream_ = post_stream_ = nullptr;
     }
     for (Operator *o : ops_) delete o;
     ops_.clear();
@@ -206,6 +234,25 @@ class GPURunner : public Runner {
   void *Stream() const override { return stream_; }
 
  private:
+  // Hands the batch in buffer set `pipe` to the trainer once all of it is there.  The wait is for that
+  // batch alone -- a stream of its own is put behind the batch's last event and the host waits for that
+  // stream -- so a batch queued after it on the runner's stream keeps running meanwhile.
+  void post(RunnerParams *params, int pipe) {
+    IPCEnv *ipc = (IPCEnv *)params->ipc;
+    lmi_server *h = (lmi_server *)params->env;
+    LMI_MUST(lmi_batch_wait(h, pipe, post_stream_));
+    LMI_MUST(lmi_stream_sync(post_stream_));
+    // a batch a kernel flagged (bad seed id, scan that gave up) is never handed over: stop here,
+    // as the reference stops on any device error (engine/memorypool.cuh:9-17)
+    LMI_MUST(lmi_server_status(h, 0));
+    if (ipc->FeaturesInParts(device_)) {  // a feature buffer too large to share whole goes over in pieces
+      int32_t nc[16], ec[16];
+      LMI_MUST(lmi_batch_counters(h, pipe, post_stream_, nc, ec));
+      ipc->StageFeatures(device_, pipe, nc[9 + hops_], post_stream_);
+      LMI_MUST(lmi_stream_sync(post_stream_));
+    }
+    ipc->IPCPost(device_, pipe);
+  }
   void run_table(RunnerParams *, int local_batch_id, int mode, bool presc) {
     for (size_t i = 0; i < ops_.size(); ++i) {
       OpParams &o = op_params_[i];
@@ -217,8 +264,10 @@ class GPURunner : public Runner {
     }
   }
   int hops_ = 0, pipe_ = 1, device_ = 0;
+  int next_pipe_ = 0;   // RunGroup: the buffer set the next batch goes into
+  int unposted_ = -1;   // hand-off with defer_post: the buffer set whose batch is issued but not yet posted
   bool ran_ = false;
-  void *stream_ = nullptr;
+  void *stream_ = nullptr, *post_stream_ = nullptr;
   std::vector<Operator *> ops_;
   std::vector<OpParams> op_params_;
 };
@@ -353,23 +402,39 @@ class GPUServer : public Server {
 
   void Run() override {  // engine/server.cu:124-135
     const int32_t max_step = ipc_->GetMaxStep();
+    const bool handoff = ipc_->HandoffEnabled();
+    // Batches go out in groups (every launch of a group serves all its batches, lmi_run_group) unless
+    // something takes them one by one: the trainer's two buffer sets and their semaphores, the LRU
+    // cache (its state advances batch by batch), the operator table.  LEGION_MI_GROUP=1 restores the
+    // reference's one batch per RunOnce; LEGION_MI_PIPES sets the number of buffer sets (default: two
+    // groups' worth, so that one group's host-link gather overlaps the next group's sampling).
+    int group = LMI_MAX_GROUP;
+    if (const char *g = std::getenv("LEGION_MI_GROUP")) group = std::max(1, std::min(LMI_MAX_GROUP, std::atoi(g)));
+    const bool lru = (dyn_cache_ & LEGION_DYN_ENABLE) && !(dyn_cache_ & LEGION_DYN_COMP);
+    if (handoff || lru || !params_.fused) group = 1;
     const auto t0 = std::chrono::steady_clock::now();
     int64_t batches = 0;
-    // with nobody reading the batches as they come (no sink, no trainer), a batch's host-link
-    // gather may run on beside the next batch's sampling
-    params_.defer_join = !sink_ && !ipc_->HandoffEnabled();
-    for (int32_t batch_id = 0; batch_id < max_step; ++batch_id) {
-      params_.global_batch_id = batch_id;
-      runner_->RunOnce(&params_);
-      if (sink_) {
-        lmi_batch_view v;
-        LMI_MUST(lmi_batch_view_get(h_, runner_->CurrentPipe(), &v));
-        sink_(&v, 0, runner_->CurrentPipe(), runner_->Stream(), sink_user_);
+    if (group > 1) {
+      int pipes = 2 * group;
+      if (const char *p = std::getenv("LEGION_MI_PIPES")) pipes = std::max(group, std::min(LMI_MAX_PIPES, std::atoi(p)));
+      LMI_MUST(lmi_server_pipes(h_, pipes));
+      params_.pipes = pipes;
+      batches = run_groups(max_step, group);
+    } else {
+      // with nobody reading the batches as they come (no sink, no trainer), a batch's host-link
+      // gather may run on beside the next batch's sampling; a trainer gets batch i while i + 1 runs
+      params_.defer_join = !sink_ && !handoff;
+      params_.defer_post = handoff;
+      for (int32_t batch_id = 0; batch_id < max_step; ++batch_id) {
+        params_.global_batch_id = batch_id;
+        runner_->RunOnce(&params_);
+        if (sink_) deliver(runner_->CurrentPipe());
+        ++batches;
+        LMI_MUST(lmi_server_status(h_, 0));  // a host-memory read: conditions of finished batches
       }
-      ++batches;
-      LMI_MUST(lmi_server_status(h_, 0));  // a host-memory read: conditions of finished batches
+      runner_->Flush(&params_);
+      for (int pipe = 0; pipe < LEGION_INTERBATCH_CON; ++pipe) LMI_MUST(lmi_batch_wait(h_, pipe, runner_->Stream()));
     }
-    for (int pipe = 0; pipe < LEGION_INTERBATCH_CON; ++pipe) LMI_MUST(lmi_batch_wait(h_, pipe, runner_->Stream()));
     LMI_MUST(lmi_stream_sync(runner_->Stream()));
     LMI_MUST(lmi_server_status(h_, 0));  // and those of the last ones
     const double sec = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
@@ -405,6 +470,46 @@ class GPUServer : public Server {
   lmi_server *Handle(int) override { return h_; }
 
  private:
+  // The sink's turn for the batch in buffer set `pipe`: the stream is put behind all of the batch first.
+  void deliver(int pipe) {
+    lmi_batch_view v;
+    LMI_MUST(lmi_batch_wait(h_, pipe, runner_->Stream()));
+    LMI_MUST(lmi_batch_view_get(h_, pipe, &v));
+    sink_(&v, 0, pipe, runner_->Stream(), sink_user_);
+  }
+
+  // The schedule in groups of at most `group` batches of one mode (a run of r such batches goes out as
+  // the fewest groups, sized evenly).  A sink sees the batches of a group, in order, after the NEXT
+  // group has been issued: the device keeps working while the host handles them, and the buffer sets
+  // of a group are not written again before the group after the next.
+  int64_t run_groups(int32_t max_step, int group) {
+    std::vector<int> before, now;
+    int64_t batches = 0;
+    int32_t b = 0;
+    while (b < max_step) {
+      const int mode = ipc_->GetCurrentMode(b);
+      int32_t run = 1;
+      while (b + run < max_step && ipc_->GetCurrentMode(b + run) == mode) ++run;
+      const int32_t n_groups = (run + group - 1) / group;
+      for (int32_t g = 0; g < n_groups; ++g) {
+        const int count = run / n_groups + (g < run % n_groups ? 1 : 0);
+        now.assign((size_t)count, 0);
+        params_.global_batch_id = b;
+        runner_->RunGroup(&params_, count, now.data());
+        if (sink_)
+          for (int pipe : before) deliver(pipe);
+        before = now;
+        b += count;
+        batches += count;
+        LMI_MUST(lmi_server_status(h_, 0));  // a host-memory read: conditions of finished batches
+      }
+    }
+    if (sink_)
+      for (int pipe : before) deliver(pipe);
+    for (int pipe = 0; pipe < params_.pipes; ++pipe) LMI_MUST(lmi_batch_wait(h_, pipe, runner_->Stream()));
+    return batches;
+  }
+
   LegionMetaConfig meta_;
   std::vector<int> fanout_;
   int dyn_cache_ = 0;

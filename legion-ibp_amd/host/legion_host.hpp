@@ -23,8 +23,12 @@
 //     engine/ipc_service.cu:60-128,212-260);
 //   * the hand-off to a trainer is a callback (SetBatchSink) and, once EnableHandoff(true)
 //     was called, the reference's shared-memory slab + two named semaphores per output
-//     buffer set (ipc_service.hpp) towards a consumer in the same process; the buffers
-//     either receives are the reference's output contract.
+//     buffer set (ipc_service.hpp) towards a trainer in another process, or on another thread
+//     of this one; the buffers either receives are the reference's output contract;
+//   * Run() issues the schedule in groups of up to LMI_MAX_GROUP batches of one mode, on twice
+//     as many output buffer sets, unless the batches are taken one by one (the trainer's two
+//     buffer sets, the LRU cache, the operator table, LEGION_MI_GROUP=1); a sink then sees a
+//     group's batches, in order, once the next group has been issued.
 #pragma once
 
 #include <cstdint>
@@ -57,6 +61,10 @@ struct RunnerParams {
   bool defer_join = false;  // true: RunOnce does not order the stream behind the batch's host-link
                             // gather (nobody reads the batch yet); the pipe's next batch does, so the
                             // gather overlaps the sampling of the batch in between
+  bool defer_post = false;  // hand-off only.  false: RunOnce returns with its batch posted to the trainer,
+                            // as the reference's does.  true: it returns with the batch BEFORE posted and
+                            // its own still running; the next RunOnce, Flush or Finalize posts that one
+  int pipes = 2;            // output buffer sets RunGroup takes in turn (lmi_server_pipes made them)
 };
 
 // Called once per finished batch with the pipe's device buffers; the stream has
@@ -91,7 +99,13 @@ class Runner {
   virtual void RunPreSc(RunnerParams *params) = 0;                  // sampling only, no gather
   virtual void RunOnce(RunnerParams *params) = 0;
   virtual void Finalize(RunnerParams *params) = 0;
-  virtual int CurrentPipe() const = 0;  // pipe holding the batch RunOnce produced last
+  // additions
+  // `count` <= LMI_MAX_GROUP consecutive batches of one mode, the first params->global_batch_id,
+  // every launch shared by all of them (lmi_run_group), into `count` of the params->pipes buffer
+  // sets taken in turn; pipes_out (may be null) receives the set of each batch.  No hand-off.
+  virtual void RunGroup(RunnerParams *params, int count, int *pipes_out) = 0;
+  virtual void Flush(RunnerParams *params) = 0;  // posts the batch a RunOnce with defer_post left behind
+  virtual int CurrentPipe() const = 0;  // pipe holding the batch issued last
   virtual void *Stream() const = 0;
 };
 Runner *NewGPURunner();

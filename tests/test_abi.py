@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol(lmi):
     missing = [s for s in declared if not hasattr(lib, s)]
     assert not missing, "declared in legion_mi.h but not exported: %s" % missing
     assert sorted(lmi.ABI_SYMBOLS) == declared, "python mirror out of sync with the header"
-    assert lib.lmi_abi_version() == 2
+    assert lib.lmi_abi_version() == 3
 
 
 def test_struct_layouts_match_header(lmi):

@@ -395,12 +395,22 @@ def test_a_bad_seed_stays_on_record_until_cleared(lmi, oracle):
             srv.status()
         assert ei.value.code == -5 and "seed id outside" in str(ei.value)
         with pytest.raises(lmi.LegionError) as ei:
-            srv.batch_wait(stream=stream)                    # the same code where the runner joins a batch
+            srv.batch_wait(stream=stream)                    # the same code where the runner joins a batch ...
         assert ei.value.code == -5
+        srv.batch_wait(stream=stream)                        # ... once: the good batches after it wait in peace
+        with pytest.raises(lmi.LegionError):
+            srv.status()                                     # while the server's own record stays
         with pytest.raises(lmi.LegionError):
             srv.status(clear=True)                           # reports once more, then forgets
         srv.status()
         srv.batch_wait(stream=stream)
+        srv.run_once(np.array([5, 401], np.int32), rng_seed=4, stream=stream)   # a new condition after the clear
+        lmi.check(lmi.lib().lmi_stream_sync(stream))
+        with pytest.raises(lmi.LegionError):
+            srv.batch_wait(stream=stream)                    # is reported again, once
+        srv.batch_wait(stream=stream)
+        with pytest.raises(lmi.LegionError):
+            srv.status(clear=True)
     finally:
         srv.close()
         feats.free()
@@ -1061,13 +1071,16 @@ def test_random_groups_sweep(lmi, oracle, case):
         feats.free()
 
 
+@pytest.mark.parametrize("early_fork", [0, 1, 2])
 @pytest.mark.parametrize("streams", [1, 2])
-def test_groups_that_reuse_pipes_wait_for_the_host_link_gather_before(lmi, oracle, streams):
+def test_groups_that_reuse_pipes_wait_for_the_host_link_gather_before(lmi, oracle, streams, early_fork):
     """Groups issued back to back on overlapping sets of pipes, nothing fetched in between: a pipe's
     next batch may only start once the side stream has finished the host-link gather of the one
     before (one event per group marks that, whichever pipes of it are reused first).  The host-link
     gather is slowed to one block and most rows miss, so a batch that started early would be
-    overwritten by the rows of its predecessor."""
+    overwritten by the rows of its predecessor.  With the side stream released ahead of the HBM gather
+    (early_fork) that event does not cover the HBM gather: a pipe taken over by the other caller's
+    stream is ordered behind the stream that carried its batch."""
     rng = np.random.default_rng(77 + streams)
     n_nodes, batch, dim, fanout, pipes = 40_000, 500, 128, [10, 5], 8
     indptr, indices = random_graph(rng, n_nodes, 12, hubs=4, hub_deg=2000)
@@ -1076,6 +1089,7 @@ def test_groups_that_reuse_pipes_wait_for_the_host_link_gather_before(lmi, oracl
     ss = [lmi.stream_create() for _ in range(streams)]
     try:
         srv.tune("miss_blocks", 1)
+        srv.tune("early_fork", early_fork)
         srv.load_graph(indptr, indices)
         srv.attach_features(feats)
         srv.build_static_cache(n_nodes // 10, lmi.TABLE_RANK)
@@ -1098,6 +1112,68 @@ def test_groups_that_reuse_pipes_wait_for_the_host_link_gather_before(lmi, oracl
             o = oracle.sample_batch(indptr, indices, seeds, fanout, r)
             assert_batch_equal(g, o)
             assert g.features.tobytes() == feats.array[o.ids].tobytes(), "pipe %d" % pipe
+        srv.status()
+    finally:
+        srv.close()
+        feats.free()
+
+
+@pytest.mark.parametrize("cache", ["none", "static-early", "static-late"])
+def test_a_pipe_read_from_another_stream_sees_the_whole_batch(lmi, oracle, cache):
+    """A batch issued on one stream and waited for (lmi_batch_wait, and the read-back that follows)
+    on another: without a cache the whole batch sits on the issuing stream, with the side stream
+    released early its HBM gather does -- the waiting stream must be ordered behind that too."""
+    rng = np.random.default_rng(5150)
+    n_nodes, batch, dim, fanout = 60_000, 1500, 128, [15, 8]
+    indptr, indices = random_graph(rng, n_nodes, 14, hubs=3, hub_deg=3000)
+    feats = make_features(lmi, rng, n_nodes, dim)
+    srv = lmi.Server(batch, fanout, dim, pipes=2, seed=9)
+    a, b = lmi.stream_create(), lmi.stream_create()
+    try:
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        if cache != "none":
+            srv.build_static_cache(n_nodes * 9 // 10, lmi.TABLE_RANK)   # nearly everything is an HBM hit
+            srv.tune("early_fork", 1 if cache == "static-early" else 0)
+        for it in range(6):
+            seeds = rng.choice(n_nodes, batch, replace=False).astype(np.int32)
+            srv.run_once(seeds, rng_seed=40 + it, pipe=it % 2, stream=a if it % 2 == 0 else b)
+            srv.batch_wait(it % 2, b if it % 2 == 0 else a)              # the OTHER stream waits ...
+            g = srv.fetch(pipe=it % 2, stream=b if it % 2 == 0 else a)   # ... and reads
+            o = oracle.sample_batch(indptr, indices, seeds, fanout, 40 + it)
+            assert_batch_equal(g, o)
+            assert g.features.tobytes() == feats.array[o.ids].tobytes(), "batch %d" % it
+    finally:
+        srv.close()
+        feats.free()
+
+
+def test_a_wait_on_one_stream_does_not_release_another(lmi, oracle):
+    """The host-link gather of a batch is slowed to one block; a second stream waits for the batch
+    (lmi_batch_wait), then the pipe's NEXT batch is issued on the first stream at once.  That stream
+    has not waited yet: it must still be held until the first batch's rows are in, or they would land
+    among the second batch's."""
+    rng = np.random.default_rng(616)
+    n_nodes, batch, dim, fanout = 50_000, 800, 128, [10, 6]
+    indptr, indices = random_graph(rng, n_nodes, 12, hubs=3, hub_deg=2500)
+    feats = make_features(lmi, rng, n_nodes, dim)
+    srv = lmi.Server(batch, fanout, dim, pipes=1, seed=2)
+    a, b = lmi.stream_create(), lmi.stream_create()
+    try:
+        srv.tune("miss_blocks", 1)
+        srv.load_graph(indptr, indices)
+        srv.attach_features(feats)
+        srv.build_static_cache(n_nodes // 20, lmi.TABLE_RANK)            # most rows cross the host link
+        for it in range(4):
+            s1 = rng.choice(n_nodes, batch, replace=False).astype(np.int32)
+            s2 = rng.choice(n_nodes, batch // 2, replace=False).astype(np.int32)
+            srv.run_once(s1, rng_seed=70 + it, pipe=0, stream=a)
+            srv.batch_wait(0, b)                                         # stream b is now behind the batch
+            srv.run_once(s2, rng_seed=170 + it, pipe=0, stream=a)        # stream a is not, unless the call sees to it
+            g = srv.fetch(pipe=0, stream=a)
+            o = oracle.sample_batch(indptr, indices, s2, fanout, 170 + it)
+            assert_batch_equal(g, o)
+            assert g.features.tobytes() == feats.array[o.ids].tobytes(), "round %d" % it
         srv.status()
     finally:
         srv.close()

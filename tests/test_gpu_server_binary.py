@@ -50,11 +50,15 @@ def read_dump(path, dim, dtype=np.float32):
     return nc, ec, ids, src, dst, feat
 
 
-@pytest.mark.parametrize("dyn_cache,table_mode,presample,dtype", [
-    (0, False, False, "f32"), (0, True, False, "f32"), (1, False, False, "f32"), (1, True, False, "f32"),
-    (8, False, False, "f32"), (0, True, True, "f32"),
-    (0, False, False, "f16"), (1, False, False, "f16"), (8, False, False, "f16")])   # fp16 `features` file
-def test_sampling_server_binary(tmp_path, oracle, dyn_cache, table_mode, presample, dtype):
+# group: None = the server's own choice (groups of up to 8 batches of one mode when nothing takes the batches
+# one by one -- here the static and int8 caches without the operator table), 1 = one batch per RunOnce as in
+# the reference, 2 = small groups, so that the three training steps of an epoch go out as 2 + 1
+@pytest.mark.parametrize("dyn_cache,table_mode,presample,dtype,group", [
+    (0, False, False, "f32", None), (0, False, False, "f32", 1), (0, False, False, "f32", 2),
+    (0, True, False, "f32", None), (1, False, False, "f32", None), (1, True, False, "f32", None),
+    (8, False, False, "f32", None), (0, True, True, "f32", None), (0, False, True, "f32", None),
+    (0, False, False, "f16", None), (1, False, False, "f16", None), (8, False, False, "f16", None)])   # fp16 `features` file
+def test_sampling_server_binary(tmp_path, oracle, dyn_cache, table_mode, presample, dtype, group):
     assert os.path.exists(BIN), "build the host shim first (make -C legion-ibp_amd)"
     rng = np.random.default_rng(dyn_cache * 2 + table_mode)
     n_nodes, dim, batch, n_train, fanout = 5000, 64, 100, 350, [25, 10]
@@ -67,7 +71,9 @@ def test_sampling_server_binary(tmp_path, oracle, dyn_cache, table_mode, presamp
         data, batch, n_nodes, len(indices), dim, n_train, 50, 40, cache_bytes, 2))
     dump = tmp_path / "dump"
     dump.mkdir()
-    env = dict(os.environ, LEGION_MI_DUMP=str(dump), LEGION_MI_DUMP_BATCHES="4")
+    env = dict(os.environ, LEGION_MI_DUMP=str(dump), LEGION_MI_DUMP_BATCHES="9")
+    if group:
+        env["LEGION_MI_GROUP"] = str(group)
     if dtype == "f16":
         env["LEGION_MI_FEAT_DTYPE"] = "f16"
     if table_mode:
@@ -83,10 +89,12 @@ def test_sampling_server_binary(tmp_path, oracle, dyn_cache, table_mode, presamp
     if dyn_cache == 8:
         slot = oracle.static_cache_build(indptr, cache_bytes // (dim + 4))
         q, sc = oracle.quantize_rows(feats[np.flatnonzero(slot >= 0)])
-    valid = read_sets(str(data))[1]
-    for i in range(4):   # three training batches of 100, then the validation batch of 50
+    _, valid, test = read_sets(str(data))
+    # every batch of the schedule, in order: per epoch three training batches of 100 and the validation
+    # batch of 50, the test batch of 40 at the end
+    schedule = ([(train[k * batch:(k + 1) * batch], k) for k in range(3)] + [(valid, 0)]) * 2 + [(test, 0)]
+    for i, (seeds, local) in enumerate(schedule):
         nc, ec, ids, src, dst, feat = read_dump(str(dump / ("batch_%d.bin" % i)), dim, np_dtype)
-        seeds, local = (train[i * batch:(i + 1) * batch], i) if i < 3 else (valid, 0)
         o = oracle.sample_batch(indptr, indices, seeds, fanout, 1 + local)
         assert list(nc) == list(o.node_counter) and list(ec) == list(o.edge_counter)
         assert np.array_equal(ids, o.ids) and np.array_equal(src, o.agg_src_off) and np.array_equal(dst, o.agg_dst_off)
@@ -121,3 +129,53 @@ def test_sampling_server_stops_on_a_seed_outside_the_graph(tmp_path):
     assert out.returncode != 0, out.stdout + out.stderr
     assert "seed id outside" in out.stderr, out.stdout + out.stderr
     assert "batches:" not in out.stdout       # the run did not report a throughput
+
+
+def test_server_run_reaches_the_rate_of_the_grouped_path(tmp_path, lmi):
+    """A products-sized dataset on disk (2.45 M nodes, 61.9 M edges, 100-d fp32 rows, batch 800, fan-out
+    [25,10], cache = 30 % of the rows) served by the `sampling_server` binary through Server::Run, which
+    issues groups of eight batches on sixteen buffer sets when nothing takes the batches one by one: its
+    own batches/s line against bench.py's products figure (the same graph, the same issue pattern through
+    the Python binding)."""
+    import json
+    import re
+    import sys
+    sys.path.insert(0, ROOT)
+    import bench
+    if bench.mem_available_gb() < 16:
+        pytest.skip("needs a few GB of host memory and of /tmp")
+    w = dict(bench.WORKLOADS["products"])
+    inputs = bench.build_inputs(lmi, w, 20260101, 8.0)
+    data = tmp_path / "data"
+    data.mkdir()
+    try:
+        n_nodes, n_edges, n_train = inputs["n_nodes"], inputs["n_edges"], inputs["n_train"]
+        lmi.to_host(inputs["d_indptr"], n_nodes + 1, np.int64).tofile(str(data / "edge_src"))
+        lmi.to_host(inputs["d_indices"], n_edges, np.int32).tofile(str(data / "edge_dst"))
+        inputs["feats"].array.tofile(str(data / "features"))
+        inputs["train"].astype(np.int32).tofile(str(data / "trainingset"))
+    finally:
+        bench.free_inputs(lmi, inputs)
+    epochs = 8
+    cache_bytes = int(n_nodes * 0.30) * w["dim"] * 4
+    (tmp_path / "meta_config").write_text("%s/ %d %d %d %d %d %d %d %d %d" % (
+        data, w["batch"], n_nodes, n_edges, w["dim"], n_train, 0, 0, cache_bytes, epochs))
+    out = subprocess.run([BIN, "1", "0", "0", "25,10"], cwd=str(tmp_path), timeout=300, capture_output=True, text=True)
+    assert out.returncode == 0, out.stdout[-2000:] + out.stderr[-2000:]
+    steps = (n_train - 1) // w["batch"] * epochs
+    m = re.search(r"batches: (\d+) .*\(([0-9.]+) batches/s\)", out.stdout)
+    assert m and int(m.group(1)) == steps, out.stdout[-2000:]
+    served = float(m.group(2))
+    one = subprocess.run([BIN, "1", "0", "0", "25,10"], cwd=str(tmp_path), timeout=300, capture_output=True, text=True,
+                         env=dict(os.environ, LEGION_MI_GROUP="1"))
+    assert one.returncode == 0, one.stdout[-2000:] + one.stderr[-2000:]
+    one_by_one = float(re.search(r"\(([0-9.]+) batches/s\)", one.stdout).group(1))
+    ref = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--workload", "products", "--steps", str(steps),
+                          "--warmup", "16", "--cpu-seconds", "0", "--runner-steps", "0", "--companion-steps", "0"],
+                         timeout=600, capture_output=True, text=True)
+    assert ref.returncode == 0, ref.stderr[-3000:]
+    line = json.loads(ref.stdout.strip().splitlines()[-1])
+    print("Server::Run %.0f batches/s (one batch per RunOnce: %.0f); bench.py --workload products %.0f batches/s" % (
+        served, one_by_one, line["value"]))
+    assert served >= 0.85 * line["value"], (served, line["value"])
+    assert served > one_by_one

@@ -1,7 +1,7 @@
 """The five target configurations (Cora-, products-, paper100m-, paper100m-LRU- and
 MAG240M-shaped) as parity cases: the synthetic workload
 builder of bench.py (graph generated on the GPU) at full size (cora, products,
-paper100m in groups of four) or at a stated fraction of the node count,
+paper100m in the groups bench.py issues) or at a stated fraction of the node count,
 compared with the CPU oracle batch by batch."""
 import os
 import sys
@@ -156,19 +156,15 @@ def paper100m_inputs(lmi):
     bench.free_inputs(lmi, inputs)
 
 
-def test_paper100m_at_full_size_in_groups_of_four(lmi, oracle, paper100m_inputs):
-    """The benchmark's own configuration at its real size (38 GB cache), four batches per launch as
-    bench.py issues them: bit-exact against the oracle, plus the properties that hold at any size."""
+def test_paper100m_hot_set_at_full_size(lmi, oracle, paper100m_inputs):
+    """The 38 GB degree-ordered cache of the benchmark's own configuration, read back whole: the hot
+    set is everything above the threshold degree plus the lowest ids among the ties, and a node's
+    slot is its rank among the cached ids."""
     import bench
     w = dict(bench.WORKLOADS["paper100m"])
-    srv, info = bench.build_server(lmi, w, paper100m_inputs, 20260101, 8)
-    stream = lmi.stream_create()
-    feats = info["feats"].array
-    indptr, indices = info["indptr"], info["indices"]
+    srv, info = bench.build_server(lmi, w, paper100m_inputs, 20260101, 1)
     try:
-        deg = np.diff(indptr)
-        B, fanout = w["batch"], w["fanout"]
-        # the hot set, ties at the threshold degree included: the lowest ids among them
+        deg = np.diff(info["indptr"])
         slot = srv.cache_dump(info["n_nodes"])
         cached = slot >= 0
         thr = int(deg[cached].min())
@@ -177,21 +173,60 @@ def test_paper100m_at_full_size_in_groups_of_four(lmi, oracle, paper100m_inputs)
         n_ties_in = int(cached[ties].sum())
         assert cached[ties[:n_ties_in]].all() and not cached[ties[n_ties_in:]].any()
         assert np.array_equal(slot[cached], np.arange(info["cache_rows"], dtype=np.int32))   # slot = rank among cached ids
-        del slot, cached, ties
-        counters = [3, 4, 5, 6]
-        srv.run_group([0, 1, 2, 3], counters, stream=stream)
-        got = [srv.fetch(pipe=k, stream=stream) for k in range(4)]
+    finally:
+        srv.close()
+
+
+# (pipes, tuning, sizes of the groups issued back to back with nothing read in between): the last is what
+# bench.py issues for the driver's `--steps 20` -- 7, 7, 6 on 16 pipes, batch i in pipe i % 16, so the
+# third group takes over pipes of the first while the first group's host-link gather may still run
+GROUPED = [(8, {}, [4]), (16, {"miss_blocks": 40}, [8, 8]), (16, {"miss_blocks": 40}, [7, 7, 6]),
+           (16, {"miss_blocks": 40, "early_fork": 0}, [8, 8, 8])]
+
+
+@pytest.mark.parametrize("pipes,tune,sizes", GROUPED, ids=["4on8", "8+8on16", "7+7+6on16", "8+8+8on16-latefork"])
+def test_paper100m_at_full_size_in_groups(lmi, oracle, paper100m_inputs, pipes, tune, sizes):
+    """The benchmark's own configuration at its real size (111 M nodes, 38 GB cache), issued exactly as
+    bench.py's timed region issues it -- lmi_run_group, the same group sizes, pipes and tuning, every
+    group queued before anything is read back: each batch still in a pipe afterwards bit for bit against
+    the oracle, plus the properties that hold at any size."""
+    import bench
+    w = dict(bench.WORKLOADS["paper100m"])
+    srv, info = bench.build_server(lmi, w, paper100m_inputs, 20260101, pipes)
+    stream = lmi.stream_create()
+    feats = info["feats"].array
+    indptr, indices = info["indptr"], info["indices"]
+    try:
+        for k, v in tune.items():
+            srv.tune(k, v)
+        deg = np.diff(indptr)
+        B, fanout = w["batch"], w["fanout"]
+        first, holder = 3, {}                         # pipe -> batch counter of the batch it holds at the end
+        i = first
+        for n in sizes:
+            ks = list(range(i, i + n))
+            srv.run_group([(k - first) % pipes for k in ks], ks, stream=stream)
+            holder.update({(k - first) % pipes: k for k in ks})
+            i += n
+        assert len(holder) == min(pipes, sum(sizes))
+        got = {c: srv.fetch(pipe=p, stream=stream) for p, c in sorted(holder.items())}
+        srv.status()
         # the same batch issued alone, later, on another pipe: a batch depends on nothing but its seeds and RNG seed
-        srv.run_once(None, batch_counter=counters[1], pipe=5, stream=stream)
-        alone = srv.fetch(pipe=5, stream=stream)
-        check_batch(alone, got[1])
-        assert alone.features.tobytes() == got[1].features.tobytes()
-        for k, g in enumerate(got):
-            seeds = info["train"][counters[k] * B:(counters[k] + 1) * B]
-            o = oracle.sample_batch(indptr, indices, seeds, fanout, 20260101 + counters[k])
+        c1 = sorted(got)[1]
+        spare = (max(holder) + 1) % pipes             # every batch above is on the host by now
+        srv.run_once(None, batch_counter=c1, pipe=spare, stream=stream)
+        alone = srv.fetch(pipe=spare, stream=stream)
+        check_batch(alone, got[c1])
+        assert alone.features.tobytes() == got[c1].features.tobytes()
+        for n_checked, (c, g) in enumerate(sorted(got.items())):
+            seeds = info["train"][c * B:(c + 1) * B]
+            o = oracle.sample_batch(indptr, indices, seeds, fanout, 20260101 + c)
             check_batch(g, o)
             assert g.features.tobytes() == feats[g.ids].tobytes()
-            # closed forms and invariants
+            hit = g.cache_index >= 0
+            assert deg[g.ids][hit].min() >= deg[g.ids][~hit].max()
+            if n_checked >= 2:
+                continue                              # the closed forms below on the first two batches
             assert np.array_equal(g.ids[:len(seeds)], seeds) and len(np.unique(g.ids)) == len(g.ids)
             n_prev = len(seeds)
             for h in range(g.hops):
@@ -201,8 +236,8 @@ def test_paper100m_at_full_size_in_groups_of_four(lmi, oracle, paper100m_inputs)
                 assert np.array_equal(g.ids[g.agg_src_off[e0:e1]], src) and dst.max() < n_prev
                 # new nodes are numbered by first appearance in edge order
                 new = src[~np.isin(src, g.ids[:n_prev])]
-                _, first = np.unique(new, return_index=True)
-                assert np.array_equal(g.ids[n_prev:g.n_nodes[h + 1]], new[np.sort(first)])
+                _, first_at = np.unique(new, return_index=True)
+                assert np.array_equal(g.ids[n_prev:g.n_nodes[h + 1]], new[np.sort(first_at)])
                 # a node of at most `fanout` neighbours contributes its whole row, in CSR order
                 small = np.flatnonzero(deg[g.ids[:n_prev]] <= fanout[h])[:2000]
                 rows = g.blk_indptr[h]
@@ -213,8 +248,6 @@ def test_paper100m_at_full_size_in_groups_of_four(lmi, oracle, paper100m_inputs)
                     d = g.ids[dst[e]]
                     assert src[e] in indices[indptr[d]:indptr[d + 1]]
                 n_prev = g.n_nodes[h + 1]
-            hit = g.cache_index >= 0
-            assert deg[g.ids][hit].min() >= deg[g.ids][~hit].max()
     finally:
         srv.close()
 

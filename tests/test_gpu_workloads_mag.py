@@ -22,7 +22,9 @@ def test_mag240m_int8_at_the_largest_size_the_box_serves(lmi, oracle):
     srv = None
     try:
         assert inputs["feats"].nbytes > 40e9, "expected a table of tens of GB, got %.1f GB" % (inputs["feats"].nbytes / 1e9)
-        srv, info = bench.build_server(lmi, w, inputs, 777, 4)
+        srv, info = bench.build_server(lmi, w, inputs, 777, 16)
+        for k, v in w.get("tune", {}).items():
+            srv.tune(k, int(v))                      # the workload's own settings, as bench.py applies them
         stream = lmi.stream_create()
         feats = info["feats"].array
         indptr = lmi.to_host(info["d_indptr"], info["n_nodes"] + 1, np.int64)
@@ -33,12 +35,15 @@ def test_mag240m_int8_at_the_largest_size_the_box_serves(lmi, oracle):
         thr = int(deg[slot >= 0].min())
         assert (deg[slot < 0] <= thr).all()
         B = w["batch"]
-        counters = [0, 1, 2, 3]
-        srv.run_group([0, 1, 2, 3], counters, stream=stream)     # as bench.py issues them
-        got = [srv.fetch(pipe=k, stream=stream) for k in range(4)]
-        srv.run_once(None, batch_counter=7, pipe=0, stream=stream)
+        # as bench.py issues them: groups of eight on sixteen pipes, the second queued behind the first
+        # with nothing read in between
+        counters = list(range(16))
+        srv.run_group(list(range(8)), counters[:8], stream=stream)
+        srv.run_group(list(range(8, 16)), counters[8:], stream=stream)
+        got = [srv.fetch(pipe=k, stream=stream) for k in range(16)]
+        srv.run_once(None, batch_counter=19, pipe=0, stream=stream)
         got.append(srv.fetch(pipe=0, stream=stream))
-        counters.append(7)
+        counters.append(19)
         for c, g in zip(counters, got):
             o = oracle.sample_batch(indptr, indices, info["train"][c * B:(c + 1) * B], w["fanout"], 777 + c)
             assert list(g.node_counter) == list(o.node_counter) and list(g.edge_counter) == list(o.edge_counter)

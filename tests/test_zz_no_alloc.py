@@ -131,6 +131,57 @@ def test_static_entry_point_matches_run_once_twice_in_a_row(lmi, oracle, cache, 
         feats.free()
 
 
+def test_static_entry_point_at_the_largest_server_it_takes(lmi, oracle):
+    """Batch 800 with fan-out [25, 10]: 228 800 rows and 208 000 edges of a hop in the worst case, just
+    inside the limits (2^18 each), on a graph dense enough that a batch comes close to them; a second
+    server on the same GPU uses the entry point in between (the scratch array is shared, nothing on the
+    host is)."""
+    rng = np.random.default_rng(41)
+    n_nodes, dim, batch, fanout = 400_000, 100, 800, [25, 10]
+    indptr, indices = random_graph(rng, n_nodes, 30, hubs=4, hub_deg=5000, zero_frac=0.02)
+    feats = lmi.HostBuffer((n_nodes, dim), np.float32)
+    feats.array[...] = rng.standard_normal((n_nodes, dim)).astype(np.float32)
+    srv = lmi.Server(batch, fanout, dim, pipes=1, seed=5)
+    other = lmi.Server(64, [5, 4], dim, pipes=1, seed=6)
+    stream = lmi.stream_create()
+    outs = outs2 = None
+    dseeds = []
+    try:
+        assert int(srv.view(0).max_nodes) == 228_800 <= lmi.STATIC_MAX_NODES
+        for sv in (srv, other):
+            sv.load_graph(indptr, indices)
+            sv.attach_features(feats)
+            sv.build_static_cache(120_000, lmi.TABLE_RANK)
+        outs, outs2 = DeviceOutputs(lmi, srv), DeviceOutputs(lmi, other)
+        for call, n in enumerate([batch, 37, batch]):
+            seeds = rng.choice(n_nodes, n, replace=False).astype(np.int32)
+            d = device_seeds(lmi, seeds)
+            dseeds.append(d)
+            srv.run_once_static(d, n, outs.view, rng_seed=300 + call, stream=stream)
+            # the other server takes the same scratch right behind it, on the same stream (no overlap)
+            small = seeds[:min(n, 64)]
+            other.run_once_static(d, len(small), outs2.view, rng_seed=900 + call, stream=stream)
+            lmi.check(lmi.lib().lmi_stream_sync(stream))
+            got, got2 = outs.fetch(), outs2.fetch()
+            srv.run_once(seeds, rng_seed=300 + call, pipe=0, stream=stream)
+            assert_same(got, srv.fetch(pipe=0, stream=stream))
+            other.run_once(small, rng_seed=900 + call, pipe=0, stream=stream)
+            assert_same(got2, other.fetch(pipe=0, stream=stream))
+            o = oracle.sample_batch(indptr, indices, seeds, fanout, 300 + call)
+            assert np.array_equal(got.ids, o.ids) and np.array_equal(got.agg_src_off, o.agg_src_off)
+            if n == batch:
+                assert len(got.ids) > 150_000      # the batch comes close to the worst case
+    finally:
+        srv.close()
+        other.close()
+        for o_ in (outs, outs2):
+            if o_:
+                o_.free()
+        for d in dseeds:
+            lmi.check(lmi.lib().lmi_device_free(d))
+        feats.free()
+
+
 def test_static_entry_point_refuses_what_it_cannot_hold(lmi):
     rng = np.random.default_rng(3)
     n_nodes, dim = 5000, 32
