@@ -609,7 +609,7 @@ def main():
     # the streaming kernel of the gather's own read : write shape (no indirection): an int8 -> fp16 gather
     # writes twice what it reads and HBM takes writes more slowly than reads, rows of 16 k + 12 bytes put
     # every 16-byte access 4 bytes off its natural boundary -- a 1 : 1 aligned copy is the wrong yardstick for both
-    shape_gbs = shape_launch_gbs = shape = None
+    shape_gbs = shape_launch_gbs = shape = rows_gbs = rows_launch_gbs = None
     if hit_rows * rb >= 1 << 16:
         if info["cache_kind"] == "int8":
             rd = 8 if w["dtype"] == "f16" else 4                 # int8 bytes a lane reads per 16-byte store
@@ -622,6 +622,15 @@ def main():
         shape_gbs = units * (rd + wr) / (ms * 1e-3) / 1e9
         ms = lmi.bench_stream(units, rd, wr, mis, 20, True)
         shape_launch_gbs = units * (rd + wr) / (ms * 1e-3) / 1e9
+        # ... and with the rows taken from all over a table as large as the cache (computed places: no index
+        # to wait for): what HBM gives a gather of this shape before the gather's own costs
+        src_pitch = w["dim"] if info["cache_kind"] == "int8" else rb
+        upr = src_pitch // rd
+        moved = int(hit_rows) * upr * (rd + wr)
+        ms = lmi.bench_row_stream(int(hit_rows), src_pitch, rd, wr, max(2, info["cache_rows"]), 20, False)
+        rows_gbs = moved / (ms * 1e-3) / 1e9
+        ms = lmi.bench_row_stream(int(hit_rows), src_pitch, rd, wr, max(2, info["cache_rows"]), 20, True)
+        rows_launch_gbs = moved / (ms * 1e-3) / 1e9
 
     def mover(host_link):
         # the instantiation the library picks for this row size (launch_move_rows): a power-of-two lane
@@ -630,6 +639,10 @@ def main():
         knobs = int(tunes.get("gather_vector_bytes", 0)) != 0 or (not host_link and int(tunes.get("gather_lanes_per_row", 0)) != 0)
         exact = rb % 16 == 0 and rb // 16 in (8, 16, 32, 64)
         hl = "true" if host_link else "false"
+        if not host_link and rb >= 16 and not knobs and flat in (0, 3):   # the hits: the flat gather
+            unroll = int(tunes.get("gather_unroll", 0)) or 2
+            return "gather_rows_flat_kernel<%s,%d,true>" % ("u32x4" if rb % 16 == 0 else "u32x4 at 4-byte alignment",
+                                                            4 if unroll >= 4 else 2 if unroll >= 2 else 1)
         if rb >= 16 and (flat == 1 or (flat == 0 and not exact and not knobs)):
             unroll = int(tunes.get("miss_unroll", 1)) if host_link else (int(tunes.get("gather_unroll", 0)) or 2)
             unroll = 4 if unroll >= 4 else 2 if unroll >= 2 else 1
@@ -689,7 +702,9 @@ def main():
                     same_bytes_copy_single_launch_gbs=round(same_launch_gbs, 1) if same_launch_gbs else None,
                     same_shape_stream=shape,
                     same_shape_stream_gbs=round(shape_gbs, 1) if shape_gbs else None,
-                    same_shape_stream_single_launch_gbs=round(shape_launch_gbs, 1) if shape_launch_gbs else None)
+                    same_shape_stream_single_launch_gbs=round(shape_launch_gbs, 1) if shape_launch_gbs else None,
+                    same_shape_scattered_rows_gbs=round(rows_gbs, 1) if rows_gbs else None,
+                    same_shape_scattered_rows_single_launch_gbs=round(rows_launch_gbs, 1) if rows_launch_gbs else None)
     link_bytes = min(1 << 28, info["feats"].nbytes)
     link_ms = lmi.bench_host_read(info["feats"], link_bytes)
     host_link = dict(bound="host-link", kernel=mover(True) + " (host-link gather of misses)",

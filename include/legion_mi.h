@@ -321,6 +321,16 @@ int lmi_bench_copy_launch(size_t bytes, int repeats, double *ms_per_launch);
  * what it reads: HBM takes writes more slowly than reads. */
 int lmi_bench_stream(size_t units, int read_bytes, int write_bytes, int misalign, int repeats, int launch_by_launch,
                      double *ms_per_launch);
+/* The same with the one property of a gather that lmi_bench_stream leaves out: the rows come from all
+ * over a large table.  Output row r (rows contiguous) is row hash(r) of a table of the largest power
+ * of two <= table_rows rows, src_pitch bytes each, moved as units of read_bytes in and write_bytes
+ * out (4:16, 8:16, 16:16; a pitch that is no multiple of 16 goes with 16:16 and 16-byte accesses at
+ * 4-byte alignment).  The source row is computed, not loaded: no index to wait for, no table
+ * lookup, no LDS, no barrier.  What is left between a gather and this figure is the gather's own
+ * doing; what is left between this figure and lmi_bench_stream is what HBM charges for rows that
+ * do not follow each other. */
+int lmi_bench_row_stream(int64_t rows, int64_t src_pitch, int read_bytes, int write_bytes, int64_t table_rows,
+                         int repeats, int launch_by_launch, double *ms_per_launch);
 /* Streaming zero-copy read of `bytes` bytes of pinned host memory (from lmi_host_alloc) into
  * HBM, repeated; returns mean ms per pass (the measured host-link ceiling). */
 int lmi_bench_host_read(const void *host_ptr, size_t bytes, int repeats, double *ms_per_pass);

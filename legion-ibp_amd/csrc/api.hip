@@ -236,6 +236,71 @@ static __global__ __launch_bounds__(256) void stream_kernel(const uint8_t *__res
   }
 }
 
+// The same without the one thing stream_kernel leaves out that no gather can avoid: the rows come from
+// places all over a large table.  Row r of the output (contiguous, dst_pitch bytes apart) is row
+// hash(r) of a table of 2^log2_src_rows rows src_pitch bytes apart, `upr` units of RB bytes each; the
+// source row is computed, not loaded, so nothing waits for an index.  A block takes rows_per_block
+// consecutive output rows at a time and its 256 threads walk their units in flat order, four in
+// flight per lane -- the access pattern of the tiled gathers, minus table lookups, LDS and barriers.
+template <int RB, int WB, bool A4>
+static __global__ __launch_bounds__(256) void row_stream_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
+                                                                int64_t n_rows, int upr, int64_t src_pitch,
+                                                                int64_t dst_pitch, int log2_src_rows, int rows_per_block) {
+  typedef typename StreamIn<RB>::type IN;
+  typedef typename std::conditional<A4, cp_u32x4_a4, cp_u32x4>::type OUT;
+  const int dq = 256 / upr, dr = 256 % upr;
+  const int64_t n_tiles = (n_rows + rows_per_block - 1) / rows_per_block;
+  for (int64_t tile = blockIdx.x; tile < n_tiles; tile += gridDim.x) {
+    const int64_t row0 = tile * rows_per_block;
+    const int nr = (int)(n_rows - row0 < rows_per_block ? n_rows - row0 : rows_per_block);
+    const int lim = nr * upr;
+    int rr = (int)threadIdx.x / upr, uu = (int)threadIdx.x % upr;
+    for (int f0 = threadIdx.x; f0 < lim; f0 += 256 * 4) {
+      union {
+        IN v;
+        OUT o;
+        uint32_t w[4];
+      } r[4];
+      int64_t da[4];
+      bool on[4];
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        on[u] = f0 + u * 256 < lim;
+        const uint32_t out_row = (uint32_t)(row0 + rr);
+        uint32_t h = out_row;  // a 32-bit mixer: places as irregular as the ids of a sampled batch, not evenly spread
+        h ^= h >> 16; h *= 0x7feb352du; h ^= h >> 15; h *= 0x846ca68bu; h ^= h >> 16;
+        const uint32_t src_row = h >> (32 - log2_src_rows);
+        const int64_t sa = (int64_t)src_row * src_pitch + (int64_t)uu * RB;
+        da[u] = (int64_t)out_row * dst_pitch + (int64_t)uu * WB;
+        if (on[u]) {
+          if (A4) r[u].o = __builtin_nontemporal_load(reinterpret_cast<const OUT *>(src + sa));
+          else r[u].v = __builtin_nontemporal_load(reinterpret_cast<const IN *>(src + sa));
+        }
+        uu += dr;
+        rr += dq;
+        if (uu >= upr) {
+          uu -= upr;
+          ++rr;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < 4; ++u)
+        if (on[u]) {
+          cp_u32x4 o;
+          o.x = r[u].w[0];
+          o.y = RB >= 8 ? r[u].w[1] : r[u].w[0] + 1u;
+          o.z = RB >= 16 ? r[u].w[2] : r[u].w[0] + 2u;
+          o.w = RB >= 16 ? r[u].w[3] : r[u].w[0] + 3u;
+#pragma unroll
+          for (int k = 0; k < WB / 16; ++k) {
+            o.x += (uint32_t)k;
+            __builtin_nontemporal_store((OUT)o, reinterpret_cast<OUT *>(dst + da[u] + 16 * k));
+          }
+        }
+    }
+  }
+}
+
 // ------------------------------------------- scratch of lmi_run_once_static
 // One array per GPU: every device that loads this code object holds its own copy at its own
 // address, from load until the process ends.  It stands in for the scratch a Pipe allocates at
@@ -354,6 +419,8 @@ int lmi_server_create(const lmi_config *cfg, lmi_server **out) {
       s->fault_host = (volatile int32_t *)fh;
       if (hipHostGetDevicePointer(&fd, fh, 0) != hipSuccess) rc = LMI_ERR_HIP;
       s->fault_dev = (int32_t *)fd;
+      s->rows_seen_host = s->fault_host + 8;  // the second half of the 64 bytes
+      s->rows_seen_dev = s->fault_dev ? s->fault_dev + 8 : nullptr;
     }
   }
   if (rc != LMI_OK) {
@@ -1108,6 +1175,7 @@ int lmi_tune(lmi_server *h, const char *key, int64_t value) {
   else if (!strcmp(key, "gather_vector_bytes")) s->gather_vec = (int)value;
   else if (!strcmp(key, "gather_blocks")) s->gather_blocks = (int)value;
   else if (!strcmp(key, "gather_nontemporal")) s->gather_nt = (int)value;
+  else if (!strcmp(key, "gather_adaptive")) s->gather_adaptive = (int)value;
   else if (!strcmp(key, "gather_flat")) s->gather_flat = (int)value;
   else if (!strcmp(key, "miss_flat")) s->miss_flat = (int)value;
   else if (!strcmp(key, "gather_tile_rows")) s->gather_tile_rows = (int)value;
@@ -1158,6 +1226,15 @@ struct BenchScratch {
   }
 };
 }  // namespace
+
+// Repeats of a measurement kernel go round this many separate copies of its buffers, so that what is
+// timed comes from and goes to HBM: a launch repeated on one buffer of a few hundred MB would be
+// served in part by the 256 MB memory-side cache in front of HBM, which no gather of a serving loop
+// (sixteen output buffer sets, a table of tens of GB) ever is.
+static int bench_copies(size_t bytes_per_launch) {
+  const size_t want = size_t(3) << 29;  // 1.5 GB of footprint
+  return (int)std::max<size_t>(1, std::min<size_t>(64, (want + bytes_per_launch - 1) / std::max<size_t>(bytes_per_launch, 1)));
+}
 
 int lmi_bench_host_read(const void *host_ptr, size_t bytes, int repeats, double *ms_per_pass) {
   if (!host_ptr || !ms_per_pass || repeats < 1 || bytes < 16) LMI_FAIL(LMI_ERR_ARG, "bad argument");
@@ -1210,15 +1287,21 @@ int lmi_bench_random_read(const void *device_ptr, size_t bytes, int64_t n_reads,
 int lmi_bench_copy(size_t bytes, int repeats, double *ms_per_copy) {
   if (!ms_per_copy || repeats < 1 || bytes < 16) LMI_FAIL(LMI_ERR_ARG, "bad argument");
   BenchScratch m;
-  LMI_HIP(hipMalloc(&m.a, bytes));
-  LMI_HIP(hipMalloc(&m.b, bytes));
-  LMI_HIP(hipMemset(m.a, 1, bytes));
+  const int copies = bench_copies(2 * bytes);
+  const size_t pitch = (bytes + 255) / 256 * 256;
+  LMI_HIP(hipMalloc(&m.a, pitch * copies));
+  LMI_HIP(hipMalloc(&m.b, pitch * copies));
+  LMI_HIP(hipMemset(m.a, 1, pitch * copies));
   LMI_TRY(m.events());
   const size_t n = bytes / 16;
-  hipLaunchKernelGGL(copy_kernel<false>, dim3(16384), dim3(256), 0, 0, (const cp_u32x4 *)m.a, (cp_u32x4 *)m.b, n);
+  auto launch = [&](int r) {
+    const size_t at = pitch * (size_t)(r % copies);
+    hipLaunchKernelGGL(copy_kernel<false>, dim3(16384), dim3(256), 0, 0, (const cp_u32x4 *)((const char *)m.a + at),
+                       (cp_u32x4 *)((char *)m.b + at), n);
+  };
+  launch(0);
   LMI_HIP(hipEventRecord(m.e0, 0));
-  for (int r = 0; r < repeats; ++r)
-    hipLaunchKernelGGL(copy_kernel<false>, dim3(16384), dim3(256), 0, 0, (const cp_u32x4 *)m.a, (cp_u32x4 *)m.b, n);
+  for (int r = 0; r < repeats; ++r) launch(r + 1);
   LMI_HIP(hipGetLastError());
   return m.elapsed(repeats, ms_per_copy);
 }
@@ -1226,17 +1309,20 @@ int lmi_bench_copy(size_t bytes, int repeats, double *ms_per_copy) {
 int lmi_bench_copy_launch(size_t bytes, int repeats, double *ms_per_launch) {
   if (!ms_per_launch || repeats < 1 || bytes < 16) LMI_FAIL(LMI_ERR_ARG, "bad argument");
   BenchScratch m;
-  LMI_HIP(hipMalloc(&m.a, bytes));
-  LMI_HIP(hipMalloc(&m.b, bytes));
-  LMI_HIP(hipMemset(m.a, 1, bytes));
+  const int copies = bench_copies(2 * bytes);
+  const size_t pitch = (bytes + 255) / 256 * 256;
+  LMI_HIP(hipMalloc(&m.a, pitch * copies));
+  LMI_HIP(hipMalloc(&m.b, pitch * copies));
+  LMI_HIP(hipMemset(m.a, 1, pitch * copies));
   LMI_TRY(m.events());
   const size_t n = bytes / 16;
   // a grid in proportion to the bytes, as the gathers size theirs, between one block and 64 per compute unit
   const int grid = (int)std::max<size_t>(1, std::min<size_t>(n / (256 * 4), 16384));
   double total = 0.0;
   for (int r = -1; r < repeats; ++r) {  // the first launch warms up and is not counted
-    hipExtLaunchKernelGGL(copy_kernel<false>, dim3(grid), dim3(256), 0, 0, m.e0, m.e1, 0, (const cp_u32x4 *)m.a,
-                          (cp_u32x4 *)m.b, n);
+    const size_t at = pitch * (size_t)((r + 1) % copies);
+    hipExtLaunchKernelGGL(copy_kernel<false>, dim3(grid), dim3(256), 0, 0, m.e0, m.e1, 0,
+                          (const cp_u32x4 *)((const char *)m.a + at), (cp_u32x4 *)((char *)m.b + at), n);
     LMI_HIP(hipGetLastError());
     LMI_HIP(hipDeviceSynchronize());
     float ms = 0;
@@ -1255,14 +1341,18 @@ int lmi_bench_stream(size_t units, int read_bytes, int write_bytes, int misalign
     LMI_FAIL(LMI_ERR_ARG, "read : write bytes per unit must be 4:16, 8:16, 8:32 or 16:16");
   if (misalign != 0 && (misalign != 4 || shape != 1616)) LMI_FAIL(LMI_ERR_ARG, "misalign is 0, or 4 with 16:16");
   BenchScratch m;
-  LMI_HIP(hipMalloc(&m.a, units * read_bytes + 64));
-  LMI_HIP(hipMalloc(&m.b, units * write_bytes + 64));
-  LMI_HIP(hipMemset(m.a, 1, units * read_bytes + 64));
+  const int copies = bench_copies(units * (size_t)(read_bytes + write_bytes));
+  const size_t src_pitch = (units * read_bytes + 64 + 255) / 256 * 256, dst_pitch = (units * write_bytes + 64 + 255) / 256 * 256;
+  LMI_HIP(hipMalloc(&m.a, src_pitch * copies));
+  LMI_HIP(hipMalloc(&m.b, dst_pitch * copies));
+  LMI_HIP(hipMemset(m.a, 1, src_pitch * copies));
   LMI_TRY(m.events());
-  const uint8_t *src = (const uint8_t *)m.a + misalign;
-  uint8_t *dst = (uint8_t *)m.b + misalign;
+  int turn = 0;
   const int grid = (int)std::max<size_t>(1, std::min<size_t>(units / (256 * 4), 16384));
   auto launch = [&](hipEvent_t e0, hipEvent_t e1) {
+    const uint8_t *src = (const uint8_t *)m.a + src_pitch * (size_t)(turn % copies) + misalign;
+    uint8_t *dst = (uint8_t *)m.b + dst_pitch * (size_t)(turn % copies) + misalign;
+    ++turn;
 #define LMI_STREAM(RB_, WB_, A4_)                                                                                   \
   if (e0)                                                                                                           \
     hipExtLaunchKernelGGL((stream_kernel<RB_, WB_, A4_>), dim3(grid), dim3(256), 0, 0, e0, e1, 0, src, dst, units);  \
@@ -1276,6 +1366,67 @@ int lmi_bench_stream(size_t units, int read_bytes, int write_bytes, int misalign
 #undef LMI_STREAM
   };
   if (launch_by_launch) {  // each launch alone on the device, timed from its own first to its own last wavefront
+    double total = 0.0;
+    for (int r = -1; r < repeats; ++r) {
+      launch(m.e0, m.e1);
+      LMI_HIP(hipGetLastError());
+      LMI_HIP(hipDeviceSynchronize());
+      float ms = 0;
+      LMI_HIP(hipEventElapsedTime(&ms, m.e0, m.e1));
+      if (r >= 0) total += ms;
+    }
+    *ms_per_launch = total / repeats;
+    return LMI_OK;
+  }
+  launch(nullptr, nullptr);
+  LMI_HIP(hipEventRecord(m.e0, 0));
+  for (int r = 0; r < repeats; ++r) launch(nullptr, nullptr);
+  LMI_HIP(hipGetLastError());
+  return m.elapsed(repeats, ms_per_launch);
+}
+
+int lmi_bench_row_stream(int64_t rows, int64_t src_pitch, int read_bytes, int write_bytes, int64_t table_rows,
+                         int repeats, int launch_by_launch, double *ms_per_launch) {
+  if (!ms_per_launch || repeats < 1 || rows < 1 || table_rows < 2) LMI_FAIL(LMI_ERR_ARG, "bad argument");
+  const int shape = read_bytes * 100 + write_bytes;
+  if (shape != 416 && shape != 816 && shape != 1616) LMI_FAIL(LMI_ERR_ARG, "read : write bytes per unit must be 4:16, 8:16 or 16:16");
+  if (src_pitch < read_bytes || src_pitch % 4 != 0) LMI_FAIL(LMI_ERR_ARG, "rows are a multiple of 4 bytes and hold a unit");
+  const bool a4 = src_pitch % 16 != 0;  // 16-byte accesses that may only assume 4-byte alignment
+  if (a4 && shape != 1616) LMI_FAIL(LMI_ERR_ARG, "rows that are no multiple of 16 bytes go with 16:16");
+  const int upr = (int)(src_pitch / read_bytes);  // whole units; a row's last few bytes are left out
+  if (upr < 1 || upr > (1 << 20)) LMI_FAIL(LMI_ERR_ARG, "row length out of range");
+  int lg = 1;
+  while ((int64_t(2) << lg) <= table_rows && lg < 31) ++lg;  // the table holds 2^lg rows, at most table_rows
+  const int64_t dst_pitch = a4 ? src_pitch : (int64_t)upr * write_bytes;
+  BenchScratch m;
+  const size_t src_bytes = (size_t)(int64_t(1) << lg) * src_pitch + 64;
+  const size_t dst_bytes = ((size_t)rows * dst_pitch + 64 + 255) / 256 * 256;
+  const int copies = bench_copies(dst_bytes);  // of the output; the table is as large as the caller says
+  LMI_HIP(hipMalloc(&m.a, src_bytes));
+  LMI_HIP(hipMalloc(&m.b, dst_bytes * copies));
+  LMI_HIP(hipMemset(m.a, 1, src_bytes));
+  LMI_TRY(m.events());
+  const uint8_t *src = (const uint8_t *)m.a;
+  int turn = 0;
+  // about 32 KB of output per block visit, at least one row
+  const int rpb = (int)std::max<int64_t>(1, std::min<int64_t>(64, 32768 / std::max<int64_t>(1, dst_pitch)));
+  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>((rows + rpb - 1) / rpb, 16384));
+  auto launch = [&](hipEvent_t e0, hipEvent_t e1) {
+    uint8_t *dst = (uint8_t *)m.b + dst_bytes * (size_t)(turn++ % copies);
+#define LMI_ROWS(RB_, WB_, A4_)                                                                                      \
+  if (e0)                                                                                                            \
+    hipExtLaunchKernelGGL((row_stream_kernel<RB_, WB_, A4_>), dim3(grid), dim3(256), 0, 0, e0, e1, 0, src, dst,       \
+                          rows, upr, src_pitch, dst_pitch, lg, rpb);                                                 \
+  else                                                                                                               \
+    hipLaunchKernelGGL((row_stream_kernel<RB_, WB_, A4_>), dim3(grid), dim3(256), 0, 0, src, dst, rows, upr,          \
+                       src_pitch, dst_pitch, lg, rpb)
+    if (shape == 416) { LMI_ROWS(4, 16, false); }
+    else if (shape == 816) { LMI_ROWS(8, 16, false); }
+    else if (a4) { LMI_ROWS(16, 16, true); }
+    else { LMI_ROWS(16, 16, false); }
+#undef LMI_ROWS
+  };
+  if (launch_by_launch) {
     double total = 0.0;
     for (int r = -1; r < repeats; ++r) {
       launch(m.e0, m.e1);

@@ -236,6 +236,93 @@ static __global__ __launch_bounds__(256) void move_rows_tiled_kernel(
   }
 }
 
+// The HBM gather of cache hits for rows that no power-of-two lane group fits.  Output rows [first, n)
+// directly, source row = src_index[row] (a cache slot; negative = a miss, skipped).  A block takes a
+// tile of consecutive rows and its 256 threads walk the tile's 16-byte units in flat order -- unit f is
+// piece f % upr of row f / upr -- U units per lane and pass: the U slots (lanes of one row read the
+// same word: one cache line per wavefront), then the U row pieces, then the U stores, each step
+// issued whole before the next waits.  Lanes without a unit, or whose row is a miss, issue nothing
+// (every access they would make costs the memory pipeline a cycle whether or not HBM sees it).
+// Nothing else stands between a block and its bytes: no LDS, no barrier.  Measured against the same
+// loop with computed source rows on one output buffer, this shape keeps 90 % of its rate; staging a
+// tile's rows through LDS first kept 70 %.  A row that is no multiple of 16 bytes ends with a unit
+// that overlaps the one before it (both write the same bytes), so every access is 16 bytes wide, at
+// 4-byte alignment when the row length demands it (V16 says which).
+// rows_seen (pinned host memory, or null): the launch leaves each pipe's row count there for the host
+// to size later grids by (see launch_gather_flat).
+template <typename V16, int U, bool NT>
+static __global__ __launch_bounds__(256) void gather_rows_flat_kernel(MoveGroup g, const uint8_t *__restrict__ src,
+                                                                      int upr, int last_off, int rows_per_tile,
+                                                                      int64_t src_pitch, int64_t dst_pitch,
+                                                                      unsigned long long *row_counter,
+                                                                      int32_t *rows_seen) {
+  LMI_GRID_ROW(g.n);
+  const MoveRow &r = g.p[row];
+  const int32_t *__restrict__ src_index = r.src_index;
+  uint8_t *__restrict__ dst = r.dst;
+  const int n = *r.n_ptr;
+  const int first = r.first_ptr ? *r.first_ptr : 0;
+  if (bx == 0 && threadIdx.x == 0) {
+    if (row_counter && n > first) atomicAdd(row_counter, (unsigned long long)(n - first));  // profiling
+    if (rows_seen) rows_seen[row] = n - first;
+  }
+  const int dq = (256 * 1) / upr, dr = 256 % upr;  // what 256 units further means in (row, piece)
+  const int r0 = (int)threadIdx.x / upr, u0 = (int)threadIdx.x % upr;
+  const int n_tiles = (n - first + rows_per_tile - 1) / rows_per_tile;
+  for (int tile = bx; tile < n_tiles; tile += gx) {
+    const int row0 = first + tile * rows_per_tile;
+    const int nr = n - row0 < rows_per_tile ? n - row0 : rows_per_tile;
+    const int lim = nr * upr;
+    int rr = r0, uu = u0;
+    for (int f0 = threadIdx.x; f0 < lim; f0 += 256 * U) {
+      int slot[U], off[U];
+      int64_t da[U];
+      V16 v[U];
+#pragma unroll
+      for (int k = 0; k < U; ++k) {
+        const int i = row0 + rr;
+        slot[k] = f0 + 256 * k < lim ? src_index[i] : -1;
+        off[k] = (uu == upr - 1) ? last_off : 16 * uu;
+        da[k] = (int64_t)i * dst_pitch + off[k];
+        uu += dr;
+        rr += dq;
+        if (uu >= upr) {
+          uu -= upr;
+          ++rr;
+        }
+      }
+#pragma unroll
+      for (int k = 0; k < U; ++k)
+        if (slot[k] >= 0)
+          v[k] = __builtin_nontemporal_load(reinterpret_cast<const V16 *>(src + (int64_t)slot[k] * src_pitch + off[k]));
+#pragma unroll
+      for (int k = 0; k < U; ++k)
+        if (slot[k] >= 0) {
+          V16 *d = reinterpret_cast<V16 *>(dst + da[k]);
+          if (NT) __builtin_nontemporal_store(v[k], d);
+          else *d = v[k];
+        }
+    }
+  }
+}
+
+// Grid of a gather whose real row count only the device knows.  The worst case of a batch is about
+// ten times what a batch holds, and a block that finds no tile is not free: the device starts about one
+// workgroup per clock, so the 8 000 idle blocks of a worst-case grid cost a 40 us launch a seventh of
+// its time.  The gather kernels leave the row count of every launch in pinned host memory
+// (rows_seen); the largest of the last launch, with an eighth on top, sizes the next grid.  The
+// kernels stride over their tiles by the grid, so a grid that turns out small is slower, not wrong.
+static int64_t hinted_rows(Server *s, int64_t n_max) {
+  if (!s->rows_seen_host || !s->gather_adaptive) return n_max;
+  int32_t seen = 0;
+  for (int k = 0; k < LMI_MAX_GROUP; ++k) {
+    const int32_t v = s->rows_seen_host[k];
+    seen = v > seen ? v : seen;
+  }
+  if (seen <= 0) return n_max;  // nothing seen yet
+  return std::min<int64_t>(n_max, (int64_t)seen + seen / 8 + 64);
+}
+
 struct MoveArgs {
   MoveGroup g;     // per pipe: work list, bounds, index arrays, destination
   int src_from_list;
@@ -340,6 +427,39 @@ static int tiled_tile_rows(Server *s, int64_t row_bytes) {
   return t;
 }
 
+// Rows per tile of the flat gather: about 8 KB worth of rows, two at least.
+static int launch_gather_flat(Server *s, hipStream_t st, const MoveArgs &a, bool nt, bool aligned16) {
+  const int upr = (int)((a.row_bytes + 15) / 16);
+  const int last_off = (int)a.row_bytes - 16;
+  const int u_want = s->gather_unroll > 0 ? s->gather_unroll : 2;
+  const int U = u_want >= 4 ? 4 : u_want >= 2 ? 2 : 1;
+  int rpt = (int)std::max<int64_t>(2, std::min<int64_t>(64, 8192 / a.row_bytes));
+  if (s->gather_tile_rows > 0) rpt = std::min(s->gather_tile_rows, 256);
+  const int64_t want = ceil_div(hinted_rows(s, a.n_max), rpt);
+  const int64_t cap = a.max_blocks > 0 ? a.max_blocks : s->gather_blocks > 0 ? s->gather_blocks : (int64_t)s->n_cu * 64;
+  const int grid = (int)std::max<int64_t>(1, std::min(want, cap));
+#define LMI_FLAT(V_, U_, NT_)                                                                                          \
+  if (a.ev_start)                                                                                                      \
+    hipExtLaunchKernelGGL((gather_rows_flat_kernel<V_, U_, NT_>), dim3(grid * a.g.n), dim3(256), 0, st, a.ev_start,     \
+                          a.ev_stop, 0, a.g, a.src, upr, last_off, rpt, a.src_row_bytes, a.dst_row_bytes,              \
+                          a.row_counter, s->rows_seen_dev);                                                            \
+  else                                                                                                                 \
+    hipLaunchKernelGGL((gather_rows_flat_kernel<V_, U_, NT_>), dim3(grid * a.g.n), dim3(256), 0, st, a.g, a.src, upr,   \
+                       last_off, rpt, a.src_row_bytes, a.dst_row_bytes, a.row_counter, s->rows_seen_dev)
+#define LMI_FLAT_U(V_, NT_)                 \
+  if (U == 4) { LMI_FLAT(V_, 4, NT_); }     \
+  else if (U == 2) { LMI_FLAT(V_, 2, NT_); } \
+  else { LMI_FLAT(V_, 1, NT_); }
+  if (aligned16 && nt) { LMI_FLAT_U(u32x4, true) }
+  else if (aligned16) { LMI_FLAT_U(u32x4, false) }
+  else if (nt) { LMI_FLAT_U(u32x4_a4, true) }
+  else { LMI_FLAT_U(u32x4_a4, false) }
+#undef LMI_FLAT_U
+#undef LMI_FLAT
+  LMI_HIP(hipGetLastError());
+  return LMI_OK;
+}
+
 static int launch_move_rows_tiled(Server *s, hipStream_t st, const MoveArgs &a, bool nt, bool aligned16) {
   const int cpr = (int)(a.row_bytes / 16), tail = (int)(a.row_bytes % 16) / 4;
   const int tile = tiled_tile_rows(s, a.row_bytes);
@@ -373,6 +493,9 @@ static int launch_move_rows(Server *s, hipStream_t st, const MoveArgs &a, bool n
     const bool exact = vec == 16 && (c16 == 8 || c16 == 16 || c16 == 32 || c16 == 64);
     const bool knobs = s->gather_vec != 0 || (s->gather_lpr != 0 && !a.host_link);  // measurement knobs of the lane-group mover
     const int flat = a.host_link ? s->miss_flat : s->gather_flat;  // 0: when no lane group fits; 1: always; 2: never
+    bool direct = !a.host_link && a.row_bytes >= 16;  // rows walked directly, source row = src_index[row]: the hits
+    for (int k = 0; k < a.g.n; ++k) direct = direct && !a.g.p[k].list && a.g.p[k].src_index && !a.g.p[k].dst_index;
+    if (direct && !knobs && (flat == 0 || flat == 3)) return launch_gather_flat(s, st, a, nt, vec == 16);
     if (a.row_bytes >= 16 && (flat == 1 || (flat == 0 && !exact && !knobs)))
       return launch_move_rows_tiled(s, st, a, nt, vec == 16);
   }
@@ -511,7 +634,8 @@ template <> struct RawVec<4> { typedef uint32_t type; };
 template <typename OUT, int EPL, int U>
 static __global__ __launch_bounds__(256) void gather_int8_tiled_kernel(MoveGroup g, const int8_t *q, const float *scale,
                                                                        int dim, int tile_rows,
-                                                                       unsigned long long *row_counter) {
+                                                                       unsigned long long *row_counter,
+                                                                       int32_t *rows_seen) {
   typedef typename RawVec<EPL>::type IN;
   constexpr int OUT_VECS = EPL * (int)sizeof(OUT) / 16;
   constexpr int TILE = 64;
@@ -523,8 +647,10 @@ static __global__ __launch_bounds__(256) void gather_int8_tiled_kernel(MoveGroup
   OUT *out = reinterpret_cast<OUT *>(g.p[row].dst);
   const int n = *g.p[row].n_ptr;
   const int first = g.p[row].first_ptr ? *g.p[row].first_ptr : 0;
-  if (row_counter && bx == 0 && threadIdx.x == 0 && n > first)
-    atomicAdd(row_counter, (unsigned long long)(n - first));
+  if (bx == 0 && threadIdx.x == 0) {
+    if (row_counter && n > first) atomicAdd(row_counter, (unsigned long long)(n - first));
+    if (rows_seen) rows_seen[row] = n - first;  // for the host to size the next grids by (hinted_rows)
+  }
   const int units = dim / EPL;
   const int dq = 256 / units, dr = 256 % units;
   const int r0 = (int)threadIdx.x / units, u0 = (int)threadIdx.x % units;
@@ -879,15 +1005,18 @@ static int launch_hits_int8(Server *s, const MoveGroup &g, hipStream_t st, int s
     if (half && epl == 4) epl = 8;  // fewer than 16 output bytes per lane are not offered
     // 768-element fp16 rows, share of HBM peak: 8 rows per tile 45 %, 16 51 %, 32 54 %, 64 52 %
     const int tile_rows = s->gather_tile_rows > 0 ? std::min(64, s->gather_tile_rows) : 32;
-    const int64_t want_f = ceil_div(n_max, tile_rows);
-    const int64_t cap_f = s->gather_blocks > 0 ? s->gather_blocks : auto_gather_blocks(s, want_f);
+    // sized by the rows the last launches held (hinted_rows): a block without a tile is not free
+    const int64_t want_f = ceil_div(hinted_rows(s, n_max), tile_rows);
+    const int64_t cap_f = s->gather_blocks > 0 ? s->gather_blocks
+                          : s->gather_adaptive ? (int64_t)s->n_cu * 64 : auto_gather_blocks(s, want_f);
     const int grid_f = g.n * (int)std::max<int64_t>(1, std::min<int64_t>(want_f, cap_f));
 #define LMI_INT8_FLAT(KERN)                                                                                   \
   if (e0)                                                                                                     \
     hipExtLaunchKernelGGL((KERN), dim3(grid_f), dim3(256), 0, st, e0, e1, 0, g, q, s->cache_scale, dim,        \
-                          tile_rows, rc);                                                                     \
+                          tile_rows, rc, s->rows_seen_dev);                                                   \
   else                                                                                                        \
-    hipLaunchKernelGGL((KERN), dim3(grid_f), dim3(256), 0, st, g, q, s->cache_scale, dim, tile_rows, rc)
+    hipLaunchKernelGGL((KERN), dim3(grid_f), dim3(256), 0, st, g, q, s->cache_scale, dim, tile_rows, rc,       \
+                       s->rows_seen_dev)
 #define LMI_INT8_FLAT_U(OUT_, EPL_)                                    \
   if (s->gather_unroll >= 4) {                                         \
     LMI_INT8_FLAT((gather_int8_tiled_kernel<OUT_, EPL_, 4>));           \

@@ -196,6 +196,9 @@ struct Server {
   volatile int32_t *fault_host = nullptr;
   int32_t *fault_dev = nullptr;  // the same words as the device addresses them
   bool fault_told[2] = {false, false};  // lmi_batch_wait has reported the condition once already
+  // row counts the gather kernels leave behind, one word per pipe of a launch, in the same pinned allocation
+  volatile int32_t *rows_seen_host = nullptr;
+  int32_t *rows_seen_dev = nullptr;
   // pipes
   std::vector<Pipe> pipes;
   hipStream_t side = nullptr;  // server-owned second stream for gathers that must not hold up the caller's stream
@@ -203,12 +206,14 @@ struct Server {
   int gather_lpr = 0;     // lanes per row (0 = auto)
   int gather_vec = 0;     // bytes per lane access (0 = widest that fits: 16)
   int gather_unroll = 0;  // rows (units) in flight per lane; 0 = the mover's own best: 1 for the lane-group mover
-                          // (a few percent ahead of 4), 2 for the tiled movers
+                          // (a few percent ahead of 4), 2 for the flat gather and the tiled movers
   int gather_tile_rows = 0;  // tiled movers: rows per tile; 0 = the mover's own rule: about 8 KB worth of rows,
                              // 2..64 (256 for rows under 128 bytes); the tiled int8 gather takes 32
   int gather_blocks = 0;  // blocks per pipe; 0 = auto (auto_gather_blocks)
   int gather_nt = 1;      // non-temporal output stores
-  int gather_flat = 0;    // 0: rows that a lane group does not fit exactly use the tiled mover; 1: every row; 2: none
+  int gather_adaptive = 1;   // gather grids sized by the row counts of recent launches instead of the worst case
+  int gather_flat = 0;    // HBM gather of hits: 0 / 3 the flat gather (gather_rows_flat_kernel); 1 the LDS-tiled
+                          // mover; 2 power-of-two lane groups, tiled only when no lane group fits the row
   int miss_flat = 0;      // the same choice for the host-link gather
   int int8_epl = 0;       // tiled int8 gather: elements per lane (0 = one 16-byte store per lane: 8 fp16 or 4 fp32)
   int64_t fuse_small_max = 32768;  // hops of at most this many nodes use the small tile of hop_tile_nodes
