@@ -388,6 +388,9 @@ def main():
     ap.add_argument("--group", type=int, default=8,
                     help="at most this many mini-batches are issued together with lmi_run_group (their sampling "
                          "kernels share launches)")
+    ap.add_argument("--group-sizes", default="",
+                    help="comma-separated sizes of the groups the timed region is issued in (must add up to --steps), "
+                         "instead of the fewest groups of at most --group, sized evenly")
     ap.add_argument("--seed", type=int, default=20260101)
     ap.add_argument("--cpu-seconds", type=float, default=15.0, help="CPU baseline budget (0 = skip)")
     ap.add_argument("--host-gb", type=float, default=0.0,
@@ -483,6 +486,11 @@ def main():
     def group_sizes(count):
         """`count` batches as the fewest groups of at most `group`, sized evenly (20 in groups of up to
         8: 7, 7, 6): the side stream's last, exposed, host-link gather is then no longer than the others."""
+        if args.group_sizes and count == args.steps:
+            sizes = [int(x) for x in args.group_sizes.split(",")]
+            if sum(sizes) != count or max(sizes) > min(group, lmi.MAX_GROUP) or min(sizes) < 1:
+                raise SystemExit("--group-sizes must add up to --steps, each 1..%d" % min(group, lmi.MAX_GROUP))
+            return sizes
         n_groups = -(-count // group)
         base, extra = divmod(count, n_groups) if n_groups else (0, 0)
         return [base + 1] * extra + [base] * (n_groups - extra)

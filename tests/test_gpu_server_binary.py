@@ -131,22 +131,20 @@ def test_sampling_server_stops_on_a_seed_outside_the_graph(tmp_path):
     assert "batches:" not in out.stdout       # the run did not report a throughput
 
 
-def test_server_run_reaches_the_rate_of_the_grouped_path(tmp_path, lmi):
-    """A products-sized dataset on disk (2.45 M nodes, 61.9 M edges, 100-d fp32 rows, batch 800, fan-out
-    [25,10], cache = 30 % of the rows) served by the `sampling_server` binary through Server::Run, which
-    issues groups of eight batches on sixteen buffer sets when nothing takes the batches one by one: its
-    own batches/s line against bench.py's products figure (the same graph, the same issue pattern through
-    the Python binding)."""
-    import json
-    import re
+@pytest.fixture(scope="module")
+def products_on_disk(tmp_path_factory, lmi):
+    """A products-sized dataset in the reference's on-disk format (2.45 M nodes, 61.9 M edges, 100-d
+    fp32 rows, batch 800, cache = 30 % of the rows, 8 epochs of 245 training steps), written from
+    bench.py's synthetic graph."""
     import sys
     sys.path.insert(0, ROOT)
     import bench
     if bench.mem_available_gb() < 16:
         pytest.skip("needs a few GB of host memory and of /tmp")
+    root = tmp_path_factory.mktemp("products")
     w = dict(bench.WORKLOADS["products"])
     inputs = bench.build_inputs(lmi, w, 20260101, 8.0)
-    data = tmp_path / "data"
+    data = root / "data"
     data.mkdir()
     try:
         n_nodes, n_edges, n_train = inputs["n_nodes"], inputs["n_edges"], inputs["n_train"]
@@ -158,15 +156,26 @@ def test_server_run_reaches_the_rate_of_the_grouped_path(tmp_path, lmi):
         bench.free_inputs(lmi, inputs)
     epochs = 8
     cache_bytes = int(n_nodes * 0.30) * w["dim"] * 4
-    (tmp_path / "meta_config").write_text("%s/ %d %d %d %d %d %d %d %d %d" % (
+    (root / "meta_config").write_text("%s/ %d %d %d %d %d %d %d %d %d" % (
         data, w["batch"], n_nodes, n_edges, w["dim"], n_train, 0, 0, cache_bytes, epochs))
-    out = subprocess.run([BIN, "1", "0", "0", "25,10"], cwd=str(tmp_path), timeout=300, capture_output=True, text=True)
+    return dict(root=root, steps=(n_train - 1) // w["batch"] * epochs, batch=w["batch"])
+
+
+def test_server_run_reaches_the_rate_of_the_grouped_path(products_on_disk):
+    """The products-sized dataset served by the `sampling_server` binary through Server::Run, which
+    issues groups of eight batches on sixteen buffer sets when nothing takes the batches one by one: its
+    own batches/s line against bench.py's products figure (the same graph, the same issue pattern through
+    the Python binding)."""
+    import json
+    import re
+    import sys
+    root, steps = products_on_disk["root"], products_on_disk["steps"]
+    out = subprocess.run([BIN, "1", "0", "0", "25,10"], cwd=str(root), timeout=300, capture_output=True, text=True)
     assert out.returncode == 0, out.stdout[-2000:] + out.stderr[-2000:]
-    steps = (n_train - 1) // w["batch"] * epochs
     m = re.search(r"batches: (\d+) .*\(([0-9.]+) batches/s\)", out.stdout)
     assert m and int(m.group(1)) == steps, out.stdout[-2000:]
     served = float(m.group(2))
-    one = subprocess.run([BIN, "1", "0", "0", "25,10"], cwd=str(tmp_path), timeout=300, capture_output=True, text=True,
+    one = subprocess.run([BIN, "1", "0", "0", "25,10"], cwd=str(root), timeout=300, capture_output=True, text=True,
                          env=dict(os.environ, LEGION_MI_GROUP="1"))
     assert one.returncode == 0, one.stdout[-2000:] + one.stderr[-2000:]
     one_by_one = float(re.search(r"\(([0-9.]+) batches/s\)", one.stdout).group(1))
@@ -179,3 +188,36 @@ def test_server_run_reaches_the_rate_of_the_grouped_path(tmp_path, lmi):
         served, one_by_one, line["value"]))
     assert served >= 0.85 * line["value"], (served, line["value"])
     assert served > one_by_one
+
+
+def test_handoff_rate_with_a_trainer_that_only_takes_the_batches(products_on_disk):
+    """The same dataset through the two-process hand-off (two buffer sets, two semaphores each, as the
+    reference deploys it) with a trainer that releases every batch at once: what the sampler side of the
+    hand-off sustains.  The runner posts batch i while batch i + 1 is already queued, so the rate stays
+    near that of the free-running one-batch-per-call loop."""
+    import re
+    import sys
+    import time
+    root, steps = products_on_disk["root"], products_on_disk["steps"]
+    env = dict(os.environ, LEGION_MI_HANDOFF="1", LEGION_MI_WAIT_SECONDS="120")
+    log_path = root / "handoff_server.log"
+    with open(log_path, "w") as log:
+        server = subprocess.Popen([BIN, "1", "0", "0", "25,10"], cwd=str(root), env=env, stdout=log, stderr=subprocess.STDOUT)
+    try:
+        deadline = time.time() + 200
+        while "System is ready for serving" not in log_path.read_text():
+            assert server.poll() is None, "the server ended early:\n" + log_path.read_text()[-3000:]
+            assert time.time() < deadline, "the server did not come up:\n" + log_path.read_text()[-3000:]
+            time.sleep(0.2)
+        out = subprocess.run([sys.executable, os.path.join(ROOT, "tests", "handoff_drain.py"), str(steps)], timeout=300,
+                             capture_output=True, text=True, cwd=str(root), env=env)
+        assert out.returncode == 0, out.stdout[-3000:] + out.stderr[-3000:] + log_path.read_text()[-2000:]
+        m = re.search(r"DRAIN_OK (\d+) batches, ([0-9.]+) batches/s", out.stdout)
+        assert m and int(m.group(1)) == steps, out.stdout
+        assert server.wait(timeout=120) == 0, log_path.read_text()[-3000:]
+        print("hand-off, trainer that only takes the batches: %s batches/s" % m.group(2))
+        assert float(m.group(2)) > 1000.0
+    finally:
+        if server.poll() is None:
+            server.kill()       # this test's own child, by its handle
+            server.wait()
