@@ -410,6 +410,10 @@ def main():
     ap.add_argument("--runner-steps", type=int, default=100, help="steps of the extra runner-issue leg (0 = skip)")
     ap.add_argument("--companion-steps", type=int, default=96,
                     help="steps of the extra leg on the same workload with uniform neighbours (0 = skip)")
+    ap.add_argument("--shape-study", action="store_true",
+                    help="after the run, sweep the row-streaming kernel of this workload's gather shape (scattered rows, "
+                         "computed places, no index) over rows per block visit, idle blocks in the grid and idle lanes "
+                         "that load anyway, and print one line per setting instead of the benchmark line")
     ap.add_argument("--gather-variants", action="store_true",
                     help="instead of the benchmark line, sweep the feature gather's access patterns on this "
                          "workload and print one line per variant")
@@ -639,6 +643,30 @@ def main():
         rows_gbs = moved / (ms * 1e-3) / 1e9
         ms = lmi.bench_row_stream(int(hit_rows), src_pitch, rd, wr, max(2, info["cache_rows"]), 20, True)
         rows_launch_gbs = moved / (ms * 1e-3) / 1e9
+
+    if args.shape_study:
+        src_pitch = w["dim"] if info["cache_kind"] == "int8" else rb
+        upr = src_pitch // rd
+        rows_n, table = int(hit_rows), max(2, info["cache_rows"])
+        moved = rows_n * upr * (rd + wr)
+        print("row-streaming kernel in the shape of the %s hit gather: %d rows of %d B from hashed places of a table of %d rows,"
+              " %d:%d bytes per lane and step, one launch at a time on an idle device, timed by the launch's own events;"
+              " the gather itself: %.1f us per launch, %.3f of the 8 TB/s peak" % (
+                  args.workload, rows_n, src_pitch, table, rd, wr, hit_ms * 1e3, achieved / HBM_PEAK_GBS))
+        auto_rpb = max(1, min(64, 32768 // max(1, (src_pitch if src_pitch % 16 else upr * wr))))
+        print("%-16s %-26s %-18s %10s %10s" % ("rows per visit", "grid", "idle lanes", "us", "of peak"))
+        for rpb in sorted({1, 2, 4, 8, 16, 32, 64, auto_rpb}):
+            tiles = -(-rows_n // rpb)
+            for label, grid in (("one block per visit", tiles), ("2x: half the blocks idle", 2 * tiles),
+                                ("4x: three in four idle", 4 * tiles), ("half: two visits a block", max(1, tiles // 2))):
+                for every in (False, True):
+                    if every and grid != tiles:
+                        continue
+                    ms = lmi.bench_row_stream_shape(rows_n, src_pitch, rd, wr, table, rpb, grid, every, 20, True)
+                    print("%-16d %-26s %-18s %10.1f %10.3f" % (rpb, label, "load anyway" if every else "issue nothing", ms * 1e3,
+                                                             moved / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS), flush=True)
+        srv.close()
+        return
 
     def mover(host_link):
         # the instantiation the library picks for this row size (launch_move_rows): a power-of-two lane

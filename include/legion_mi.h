@@ -331,6 +331,14 @@ int lmi_bench_stream(size_t units, int read_bytes, int write_bytes, int misalign
  * do not follow each other. */
 int lmi_bench_row_stream(int64_t rows, int64_t src_pitch, int read_bytes, int write_bytes, int64_t table_rows,
                          int repeats, int launch_by_launch, double *ms_per_launch);
+/* The same kernel with the launch shape in the caller's hands, for studying what a gather's own choices
+ * cost: rows_per_block (0 = about 32 KB of output per block visit), grid_blocks (0 = one block per
+ * visit; more = blocks that find nothing to do and leave, as a grid sized for the worst case of a
+ * batch holds; fewer = blocks that loop), every_lane_loads != 0 (lanes without a unit in a block's
+ * last pass issue their loads anyway and only skip the store). */
+int lmi_bench_row_stream_shape(int64_t rows, int64_t src_pitch, int read_bytes, int write_bytes, int64_t table_rows,
+                               int rows_per_block, int grid_blocks, int every_lane_loads, int repeats,
+                               int launch_by_launch, double *ms_per_launch);
 /* Streaming zero-copy read of `bytes` bytes of pinned host memory (from lmi_host_alloc) into
  * HBM, repeated; returns mean ms per pass (the measured host-link ceiling). */
 int lmi_bench_host_read(const void *host_ptr, size_t bytes, int repeats, double *ms_per_pass);

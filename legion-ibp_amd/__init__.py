@@ -34,7 +34,7 @@ ABI_SYMBOLS = [
     "lmi_cache_info_get", "lmi_cache_dump", "lmi_op_batch_generate", "lmi_op_random_sample",
     "lmi_op_cache_lookup", "lmi_op_io_submit", "lmi_op_io_complete", "lmi_run_once",
     "lmi_run_group", "lmi_run_once_static", "lmi_batch_wait", "lmi_server_status", "lmi_batch_view_get", "lmi_batch_counters", "lmi_steps_per_epoch", "lmi_profile_enable",
-    "lmi_profile_read", "lmi_tune", "lmi_bench_copy", "lmi_bench_copy_launch", "lmi_bench_stream", "lmi_bench_row_stream", "lmi_bench_host_read", "lmi_bench_random_read", "lmi_synth_graph", "lmi_synth_trainset",
+    "lmi_profile_read", "lmi_tune", "lmi_bench_copy", "lmi_bench_copy_launch", "lmi_bench_stream", "lmi_bench_row_stream", "lmi_bench_row_stream_shape", "lmi_bench_host_read", "lmi_bench_random_read", "lmi_synth_graph", "lmi_synth_trainset",
     "lmi_synth_features",
 ]
 
@@ -143,6 +143,8 @@ def lib():
         L.lmi_bench_stream.argtypes = [C.c_size_t, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.POINTER(C.c_double)]
         L.lmi_bench_row_stream.argtypes = [C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_int64, C.c_int, C.c_int,
                                            C.POINTER(C.c_double)]
+        L.lmi_bench_row_stream_shape.argtypes = [C.c_int64, C.c_int64, C.c_int, C.c_int, C.c_int64, C.c_int, C.c_int, C.c_int,
+                                                 C.c_int, C.c_int, C.POINTER(C.c_double)]
         L.lmi_bench_host_read.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.POINTER(C.c_double)]
         L.lmi_bench_random_read.argtypes = [C.c_void_p, C.c_size_t, C.c_int64, C.c_int, C.POINTER(C.c_double)]
         L.lmi_synth_graph.argtypes = [C.c_uint64, C.c_void_p, C.c_int32, C.c_int64, C.c_int32,
@@ -409,6 +411,16 @@ def bench_row_stream(rows, src_pitch, read_bytes, write_bytes, table_rows, repea
     ms = C.c_double()
     check(lib().lmi_bench_row_stream(int(rows), int(src_pitch), read_bytes, write_bytes, int(table_rows), repeats,
                                      int(launch_by_launch), C.byref(ms)))
+    return ms.value
+
+
+def bench_row_stream_shape(rows, src_pitch, read_bytes, write_bytes, table_rows, rows_per_block=0, grid_blocks=0,
+                           every_lane_loads=False, repeats=10, launch_by_launch=True):
+    """bench_row_stream with the rows per block visit, the grid and the treatment of idle lanes chosen by the caller."""
+    ms = C.c_double()
+    check(lib().lmi_bench_row_stream_shape(int(rows), int(src_pitch), read_bytes, write_bytes, int(table_rows),
+                                           int(rows_per_block), int(grid_blocks), int(every_lane_loads), repeats,
+                                           int(launch_by_launch), C.byref(ms)))
     return ms.value
 
 

@@ -242,7 +242,7 @@ static __global__ __launch_bounds__(256) void stream_kernel(const uint8_t *__res
 // source row is computed, not loaded, so nothing waits for an index.  A block takes rows_per_block
 // consecutive output rows at a time and its 256 threads walk their units in flat order, four in
 // flight per lane -- the access pattern of the tiled gathers, minus table lookups, LDS and barriers.
-template <int RB, int WB, bool A4>
+template <int RB, int WB, bool A4, bool EVERY>
 static __global__ __launch_bounds__(256) void row_stream_kernel(const uint8_t *__restrict__ src, uint8_t *__restrict__ dst,
                                                                 int64_t n_rows, int upr, int64_t src_pitch,
                                                                 int64_t dst_pitch, int log2_src_rows, int rows_per_block) {
@@ -272,7 +272,7 @@ static __global__ __launch_bounds__(256) void row_stream_kernel(const uint8_t *_
         const uint32_t src_row = h >> (32 - log2_src_rows);
         const int64_t sa = (int64_t)src_row * src_pitch + (int64_t)uu * RB;
         da[u] = (int64_t)out_row * dst_pitch + (int64_t)uu * WB;
-        if (on[u]) {
+        if (EVERY || on[u]) {  // EVERY: lanes without a unit load all the same (a row that exists), and only skip the store
           if (A4) r[u].o = __builtin_nontemporal_load(reinterpret_cast<const OUT *>(src + sa));
           else r[u].v = __builtin_nontemporal_load(reinterpret_cast<const IN *>(src + sa));
         }
@@ -1387,6 +1387,13 @@ int lmi_bench_stream(size_t units, int read_bytes, int write_bytes, int misalign
 
 int lmi_bench_row_stream(int64_t rows, int64_t src_pitch, int read_bytes, int write_bytes, int64_t table_rows,
                          int repeats, int launch_by_launch, double *ms_per_launch) {
+  return lmi_bench_row_stream_shape(rows, src_pitch, read_bytes, write_bytes, table_rows, 0, 0, 0, repeats,
+                                    launch_by_launch, ms_per_launch);
+}
+
+int lmi_bench_row_stream_shape(int64_t rows, int64_t src_pitch, int read_bytes, int write_bytes, int64_t table_rows,
+                               int rows_per_block, int grid_blocks, int every_lane_loads, int repeats,
+                               int launch_by_launch, double *ms_per_launch) {
   if (!ms_per_launch || repeats < 1 || rows < 1 || table_rows < 2) LMI_FAIL(LMI_ERR_ARG, "bad argument");
   const int shape = read_bytes * 100 + write_bytes;
   if (shape != 416 && shape != 816 && shape != 1616) LMI_FAIL(LMI_ERR_ARG, "read : write bytes per unit must be 4:16, 8:16 or 16:16");
@@ -1408,23 +1415,29 @@ int lmi_bench_row_stream(int64_t rows, int64_t src_pitch, int read_bytes, int wr
   LMI_TRY(m.events());
   const uint8_t *src = (const uint8_t *)m.a;
   int turn = 0;
-  // about 32 KB of output per block visit, at least one row
-  const int rpb = (int)std::max<int64_t>(1, std::min<int64_t>(64, 32768 / std::max<int64_t>(1, dst_pitch)));
-  const int grid = (int)std::max<int64_t>(1, std::min<int64_t>((rows + rpb - 1) / rpb, 16384));
+  // about 32 KB of output per block visit, at least one row, one block per visit -- unless the caller says otherwise
+  const int rpb = rows_per_block > 0 ? rows_per_block
+                                     : (int)std::max<int64_t>(1, std::min<int64_t>(64, 32768 / std::max<int64_t>(1, dst_pitch)));
+  const int grid = grid_blocks > 0 ? grid_blocks
+                                   : (int)std::max<int64_t>(1, std::min<int64_t>((rows + rpb - 1) / rpb, 1 << 20));
   auto launch = [&](hipEvent_t e0, hipEvent_t e1) {
     uint8_t *dst = (uint8_t *)m.b + dst_bytes * (size_t)(turn++ % copies);
-#define LMI_ROWS(RB_, WB_, A4_)                                                                                      \
+#define LMI_ROWS_E(RB_, WB_, A4_, EV_)                                                                                \
   if (e0)                                                                                                            \
-    hipExtLaunchKernelGGL((row_stream_kernel<RB_, WB_, A4_>), dim3(grid), dim3(256), 0, 0, e0, e1, 0, src, dst,       \
+    hipExtLaunchKernelGGL((row_stream_kernel<RB_, WB_, A4_, EV_>), dim3(grid), dim3(256), 0, 0, e0, e1, 0, src, dst,  \
                           rows, upr, src_pitch, dst_pitch, lg, rpb);                                                 \
   else                                                                                                               \
-    hipLaunchKernelGGL((row_stream_kernel<RB_, WB_, A4_>), dim3(grid), dim3(256), 0, 0, src, dst, rows, upr,          \
+    hipLaunchKernelGGL((row_stream_kernel<RB_, WB_, A4_, EV_>), dim3(grid), dim3(256), 0, 0, src, dst, rows, upr,     \
                        src_pitch, dst_pitch, lg, rpb)
-    if (shape == 416) { LMI_ROWS(4, 16, false); }
-    else if (shape == 816) { LMI_ROWS(8, 16, false); }
-    else if (a4) { LMI_ROWS(16, 16, true); }
-    else { LMI_ROWS(16, 16, false); }
+#define LMI_ROWS(RB_, WB_, A4_)                               \
+  if (every_lane_loads) { LMI_ROWS_E(RB_, WB_, A4_, true); }  \
+  else { LMI_ROWS_E(RB_, WB_, A4_, false); }
+    if (shape == 416) { LMI_ROWS(4, 16, false) }
+    else if (shape == 816) { LMI_ROWS(8, 16, false) }
+    else if (a4) { LMI_ROWS(16, 16, true) }
+    else { LMI_ROWS(16, 16, false) }
 #undef LMI_ROWS
+#undef LMI_ROWS_E
   };
   if (launch_by_launch) {
     double total = 0.0;
