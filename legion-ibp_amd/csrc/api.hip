@@ -1054,13 +1054,15 @@ int lmi_server_status(lmi_server *h, int clear) {
 // not fail the wait of every good batch after it.
 static int fault_status_once(Server *s) {
   if (!s->fault_host) return LMI_OK;
-  const bool scan = s->fault_host[kFaultScan] != 0 && !s->fault_told[kFaultScan];
-  const bool bad = s->fault_host[kFaultBadId] != 0 && !s->fault_told[kFaultBadId];
-  if (scan) s->fault_told[kFaultScan] = true;
-  if (bad) s->fault_told[kFaultBadId] = true;
-  if (scan) LMI_FAIL(LMI_ERR_HIP, "a device scan timed out waiting for an earlier tile: that batch is incomplete");
-  if (bad)
+  // one condition per call: when both are pending, the second is told by the next call
+  if (s->fault_host[kFaultScan] != 0 && !s->fault_told[kFaultScan]) {
+    s->fault_told[kFaultScan] = true;
+    LMI_FAIL(LMI_ERR_HIP, "a device scan timed out waiting for an earlier tile: that batch is incomplete");
+  }
+  if (s->fault_host[kFaultBadId] != 0 && !s->fault_told[kFaultBadId]) {
+    s->fault_told[kFaultBadId] = true;
     LMI_FAIL(LMI_ERR_BAD_ID, "a seed id outside [0, %lld) was seen on the device and skipped", (long long)s->n_nodes);
+  }
   return LMI_OK;
 }
 
@@ -1394,14 +1396,16 @@ int lmi_bench_row_stream(int64_t rows, int64_t src_pitch, int read_bytes, int wr
 int lmi_bench_row_stream_shape(int64_t rows, int64_t src_pitch, int read_bytes, int write_bytes, int64_t table_rows,
                                int rows_per_block, int grid_blocks, int every_lane_loads, int repeats,
                                int launch_by_launch, double *ms_per_launch) {
-  if (!ms_per_launch || repeats < 1 || rows < 1 || table_rows < 2) LMI_FAIL(LMI_ERR_ARG, "bad argument");
+  if (!ms_per_launch || repeats < 1 || rows < 1 || rows > INT32_MAX || table_rows < 2) LMI_FAIL(LMI_ERR_ARG, "bad argument");
+  if (rows_per_block < 0 || rows_per_block > 4096 || grid_blocks < 0 || grid_blocks > (1 << 22))
+    LMI_FAIL(LMI_ERR_ARG, "a block visit takes 1..4096 rows and a grid has at most 2^22 blocks (0 = chosen here)");
   const int shape = read_bytes * 100 + write_bytes;
   if (shape != 416 && shape != 816 && shape != 1616) LMI_FAIL(LMI_ERR_ARG, "read : write bytes per unit must be 4:16, 8:16 or 16:16");
   if (src_pitch < read_bytes || src_pitch % 4 != 0) LMI_FAIL(LMI_ERR_ARG, "rows are a multiple of 4 bytes and hold a unit");
   const bool a4 = src_pitch % 16 != 0;  // 16-byte accesses that may only assume 4-byte alignment
   if (a4 && shape != 1616) LMI_FAIL(LMI_ERR_ARG, "rows that are no multiple of 16 bytes go with 16:16");
   const int upr = (int)(src_pitch / read_bytes);  // whole units; a row's last few bytes are left out
-  if (upr < 1 || upr > (1 << 20)) LMI_FAIL(LMI_ERR_ARG, "row length out of range");
+  if (upr < 1 || upr > (1 << 16)) LMI_FAIL(LMI_ERR_ARG, "row length out of range");  // rows_per_block x upr stays an int
   int lg = 1;
   while ((int64_t(2) << lg) <= table_rows && lg < 31) ++lg;  // the table holds 2^lg rows, at most table_rows
   const int64_t dst_pitch = a4 ? src_pitch : (int64_t)upr * write_bytes;

@@ -236,7 +236,7 @@ static __global__ __launch_bounds__(256) void move_rows_tiled_kernel(
   }
 }
 
-// The HBM gather of cache hits for rows that no power-of-two lane group fits.  Output rows [first, n)
+// The HBM gather of cache hits, for fp32 / fp16 rows of every size from 16 bytes up.  Output rows [first, n)
 // directly, source row = src_index[row] (a cache slot; negative = a miss, skipped).  A block takes a
 // tile of consecutive rows and its 256 threads walk the tile's 16-byte units in flat order -- unit f is
 // piece f % upr of row f / upr -- U units per lane and pass: the U slots (lanes of one row read the
@@ -492,7 +492,9 @@ static int launch_move_rows(Server *s, hipStream_t st, const MoveArgs &a, bool n
     const int64_t c16 = a.row_bytes / 16;
     const bool exact = vec == 16 && (c16 == 8 || c16 == 16 || c16 == 32 || c16 == 64);
     const bool knobs = s->gather_vec != 0 || (s->gather_lpr != 0 && !a.host_link);  // measurement knobs of the lane-group mover
-    const int flat = a.host_link ? s->miss_flat : s->gather_flat;  // 0: when no lane group fits; 1: always; 2: never
+    // HBM gather (gather_flat): 0 or 3 the flat gather, 1 the LDS-tiled mover, 2 lane groups; host-link
+    // gather (miss_flat): the LDS-tiled mover 0 when no lane group fits, 1 always, 2 never
+    const int flat = a.host_link ? s->miss_flat : s->gather_flat;
     bool direct = !a.host_link && a.row_bytes >= 16;  // rows walked directly, source row = src_index[row]: the hits
     for (int k = 0; k < a.g.n; ++k) direct = direct && !a.g.p[k].list && a.g.p[k].src_index && !a.g.p[k].dst_index;
     if (direct && !knobs && (flat == 0 || flat == 3)) return launch_gather_flat(s, st, a, nt, vec == 16);

@@ -47,6 +47,14 @@ def test_bad_arguments_are_rejected_without_a_gpu(lmi):
     cfg.fanout[0] = 65
     assert lib.lmi_server_create(ctypes.byref(cfg), ctypes.byref(h)) == -1   # fanout > LMI_MAX_FANOUT
     assert lib.lmi_server_destroy(None) == 0
+    # the measurement kernels check their shapes before they touch a device
+    ms = ctypes.c_double()
+    assert lib.lmi_bench_stream(1 << 20, 12, 16, 0, 1, 0, ctypes.byref(ms)) == -1          # no 12:16 shape
+    assert lib.lmi_bench_stream(1 << 20, 8, 16, 4, 1, 0, ctypes.byref(ms)) == -1           # misaligned only as 16:16
+    assert lib.lmi_bench_row_stream_shape(1000, 512, 16, 16, 4096, 5000, 0, 0, 1, 1, ctypes.byref(ms)) == -1   # rows per visit
+    assert lib.lmi_bench_row_stream_shape(1000, 510, 16, 16, 4096, 0, 0, 0, 1, 1, ctypes.byref(ms)) == -1      # rows of 4 k bytes
+    assert lib.lmi_bench_row_stream_shape(1000, 404, 8, 16, 4096, 0, 0, 0, 1, 1, ctypes.byref(ms)) == -1       # 8:16 wants 16-byte rows
+    assert lib.lmi_server_pipes(None, 4) == -1
 
 
 def test_header_cites_the_reference_for_every_group():
