@@ -306,7 +306,8 @@ def cpu_baseline(lmi, srv, w, info, seed, budget_s, issue):
         ", ".join(str(n) for n in checked_sizes[:6]) + (", ..." if len(checked_sizes) > 6 else ""), pipes)
            if group > 1 else "lmi_run_once on %d pipes" % pipes)
     return dict(value=done / spent, unit="batches/s", cores=threads, kind="port",
-                sample="%d batches of the same workload (oracle sample_batch + gather, OpenMP over %d threads); "
+                sample="%d batches of the same workload (oracle sample_batch + gather, OpenMP over %d threads: picks and the "
+                       "row gather run in parallel, the dedup / relabel pass of a batch is one thread's loop); "
                        "GPU output of the same batches, issued as the timed region issues them (%s), %s" % (
                            done, threads, how, "bit-exact" if parity_ok else "MISMATCH"),
                 gather_rows_per_s=rows / spent, checked_batches=done, checked_group_sizes=checked_sizes), parity_ok
