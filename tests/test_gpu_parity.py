@@ -418,7 +418,11 @@ def test_a_bad_seed_stays_on_record_until_cleared(lmi, oracle):
 
 @pytest.mark.parametrize("table", [0, 1, 2])
 @pytest.mark.parametrize("dim,dtype", [(128, np.float32), (100, np.float32), (1433, np.float32), (768, np.float16),
-                                        (6, np.float16)])
+                                        (6, np.float16),      # 12-byte rows: under one 16-byte unit
+                                        (5, np.float32),      # 20 bytes: two units that overlap by 12
+                                        (17, np.float32),     # 68 bytes: four whole units and a 4-byte tail
+                                        (102, np.float32),    # 408 bytes: 8-byte aligned rows
+                                        (4, np.float32)])     # 16 bytes: one unit per row
 def test_static_cache_parity(lmi, oracle, table, dim, dtype):
     rng = np.random.default_rng(dim + table)
     n_nodes, batch, fanout = 4000, 96, [10, 5]
