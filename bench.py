@@ -41,7 +41,9 @@ WORKLOADS = {
     # name: nodes, mean degree, alpha, d_max, dim, dtype, batch, fanout, train, cache
     "paper100m": dict(nodes=111_059_956, mean_deg=14.548, alpha=2.0, d_max=100_000, dim=128, dtype="f32",
                       batch=8000, fanout=[25, 10], train=1_200_000, cache=("static", 38e9),
-                      tune={"miss_blocks": 40}),   # 5 blocks for each of a group's 8 batches
+                      # groups of 8: the seeds' and the first hop's misses leave over the host link while the second
+                      # hop is still sampled (two host-link gathers per group), 6 blocks for each of the 8 batches
+                      tune={"miss_blocks": 48, "split_lookup": 2}),
     "products": dict(nodes=2_449_029, mean_deg=25.27, alpha=2.1, d_max=17_000, dim=100, dtype="f32",
                      batch=800, fanout=[25, 10], train=196_615, cache=("static_frac", 0.30)),
     "paper100m-lru": dict(nodes=111_059_956, mean_deg=14.548, alpha=2.0, d_max=100_000, dim=128, dtype="f32",
@@ -449,10 +451,10 @@ def main():
         return
     tunes = {k: str(v) for k, v in w.get("tune", {}).items()}   # the workload's own settings, then --tune
     tunes.update(kv.split("=") for kv in args.tune)
-    # host-link gather grid (miss_blocks, library default 32), measured on paper100m-shaped in groups
-    # of 8 on 16 pipes (the grid is shared out evenly, so it counts in eights): 32 -> 8.1 k batches/s, 40 -> 8.5 k,
-    # 48 -> 8.1 k, 64 -> 7.4 k; the HBM gather
-    # stays at 68-69 % of peak throughout
+    # paper100m-shaped in groups of 8 on 16 pipes (the host-link grid is shared out evenly, so it counts in
+    # eights), 20-step run / 200-step run, batches/s: one lookup per group and 40 blocks 7.2 k / 8.4 k; split
+    # lookups and 40 blocks 7.6 k / 8.3 k; split lookups and 48 blocks 7.6 k / 8.4 k (the HBM gather 0.69, 0.69
+    # and 0.67 of peak: what more host-link reads beside it cost)
     for k, v in tunes.items():
         srv.tune(k, int(v))
     steps_per_epoch = -(-info["n_train"] // w["batch"])
@@ -574,14 +576,18 @@ def main():
     runner = None
     if args.issue != "runner" and args.runner_steps > 0:
         lmi.check(lmi.lib().lmi_device_sync())
+        if "miss_blocks" not in dict(kv.split("=") for kv in args.tune):
+            srv.tune("miss_blocks", 32)   # the runner of the host shim sets no knobs: the library's own host-link grid
         r0 = time.perf_counter()
         runner_steps(done, args.runner_steps)
         lmi.check(lmi.lib().lmi_device_sync())
         r1 = time.perf_counter()
         srv.status()
+        srv.tune("miss_blocks", int(tunes.get("miss_blocks", 32)))
         runner = dict(batches_s=round(args.runner_steps / (r1 - r0), 2), steps=args.runner_steps,
-                      what="one lmi_run_once per batch on 2 pipes; before batch i+1 is issued the host waits for batch "
-                           "i-1 to be complete (GPURunner::RunOnce with the hand-off on, without a trainer's own time)")
+                      what="one lmi_run_once per batch on 2 pipes, the library's default host-link grid; before batch i+1 "
+                           "is issued the host waits for batch i-1 to be complete (GPURunner::RunOnce with the hand-off "
+                           "on, without a trainer's own time)")
         done += args.runner_steps
     # untimed extra leg with every phase of every batch bracketed (level 1), for the per-phase breakdown only
     srv.tune("profile_every", 1)
@@ -749,6 +755,7 @@ def main():
                      achieved=round(miss_rows * rb / (miss_ms * 1e-3) / 1e9, 2) if miss_ms > 0 else 0.0,
                      peak=HOST_LINK_PEAK_GBS, unit="GB/s", rows_per_launch=round(miss_rows, 1),
                      batches_per_launch=round(miss_batches, 2),
+                     launches_per_group=round(prof.gather_miss_launches / max(prof.gather_hit_launches, 1), 2),
                      avg_launch_ms=round(miss_ms, 4))
     # the sampling kernels are bound by cold random reads: what the device sustains on the neighbour array
     rr_reads = 1 << 24

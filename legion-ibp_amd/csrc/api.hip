@@ -112,6 +112,7 @@ static void pipe_free(Pipe &p) {
   if (p.graph_exec) (void)hipGraphExecDestroy(p.graph_exec);
   if (p.graph) (void)hipGraphDestroy(p.graph);
   if (p.fork) (void)hipEventDestroy(p.fork);
+  if (p.fork_early) (void)hipEventDestroy(p.fork_early);
   if (p.join) (void)hipEventDestroy(p.join);
   if (p.handover) (void)hipEventDestroy(p.handover);
   p = Pipe{};
@@ -162,6 +163,7 @@ static int pipe_alloc(Server *s, Pipe &p) {
   LMI_TRY(dmalloc(&p.lru_next, s->max_nodes));
   LMI_TRY(dmalloc(&p.seed_stage, s->cfg.batch_size));
   LMI_HIP(hipEventCreateWithFlags(&p.fork, hipEventDisableTiming));
+  LMI_HIP(hipEventCreateWithFlags(&p.fork_early, hipEventDisableTiming));
   LMI_HIP(hipEventCreateWithFlags(&p.join, hipEventDisableTiming));
   LMI_HIP(hipEventCreateWithFlags(&p.handover, hipEventDisableTiming));
   return LMI_OK;
@@ -894,6 +896,7 @@ static int capture_batch_graph(Server *s, Pipe &p, hipStream_t st, const BatchPa
 static int run_group(Server *s, Pipe *const *pp, const BatchParams *bps, int n, hipStream_t st) {
   for (int k = 0; k < n; ++k) pipe_begin(*pp[k], st);
   prof_phase(s, st, &s->prof_open, PROF_SAMPLE);
+  bool split = false;
   if (s->use_graph && st != nullptr && n == 1) {  // the legacy default stream cannot be captured
     Pipe &p = *pp[0];
     LMI_TRY(lru_wait_ready(s, st));  // the lookup sits inside the graph: the whole replay waits
@@ -901,12 +904,23 @@ static int run_group(Server *s, Pipe *const *pp, const BatchParams *bps, int n, 
     LMI_TRY(graph_update_begin(s, p, bps[0]));
     LMI_HIP(hipGraphLaunch(p.graph_exec, st));
   } else {
+    // split_lookup: the seeds and the first hop's nodes are looked up as soon as they are known and their
+    // misses start over the host link while the later hops are still being sampled
+    split = s->split_lookup && s->cfg.hops >= 2 && s->feat_loc == LMI_LOC_HOST && s->split_miss == 1 &&
+            (s->cache_kind == LMI_CACHE_STATIC || s->cache_kind == LMI_CACHE_INT8) &&
+            (s->split_lookup == 1 || (s->split_lookup == 2 && n > 1));
     LMI_TRY(launch_batch_generate(s, pp, bps, n, st, false));
-    for (int k = 0; k < s->cfg.hops; ++k) LMI_TRY(launch_hop(s, pp, n, st, k, true, true));
+    for (int k = 0; k < s->cfg.hops; ++k) {
+      LMI_TRY(launch_hop(s, pp, n, st, k, true, true));
+      if (split && k == 0) {
+        LMI_TRY(launch_lookup(s, pp, n, st, 0, 1));
+        LMI_TRY(launch_misses_early(s, pp, n, st, 0, 1));
+      }
+    }
     LMI_TRY(lru_wait_ready(s, st));  // sampling may overlap the previous batch's insertion, the lookup may not
-    LMI_TRY(launch_lookup(s, pp, n, st, 0, s->cfg.hops));
+    LMI_TRY(launch_lookup(s, pp, n, st, split ? 2 : 0, s->cfg.hops));
   }
-  LMI_TRY(launch_gather_group(s, pp, n, st, 0, s->cfg.hops, s->cache_kind == LMI_CACHE_LRU ? 1 : 0));
+  LMI_TRY(launch_gather_group(s, pp, n, st, split ? 2 : 0, s->cfg.hops, s->cache_kind == LMI_CACHE_LRU ? 1 : 0, false, 0));
   prof_phase(s, st, &s->prof_open, -1);
   return LMI_OK;
 }
@@ -1188,6 +1202,8 @@ int lmi_tune(lmi_server *h, const char *key, int64_t value) {
   else if (!strcmp(key, "group_miss")) s->group_miss = (int)value;
   else if (!strcmp(key, "lru_early_miss")) s->lru_early_miss = (int)value;
   else if (!strcmp(key, "early_fork")) s->early_fork = (int)value;
+  else if (!strcmp(key, "split_lookup")) s->split_lookup = (int)value;
+  else if (!strcmp(key, "miss_blocks_early")) s->miss_blocks_early = (int)value;
   else if (!strcmp(key, "table_epochs")) {
     s->table_epochs = std::max<int64_t>(0, value);
     for (auto &p : s->pipes) p.table_dirty = true;

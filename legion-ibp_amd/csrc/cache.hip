@@ -1099,7 +1099,7 @@ static int launch_hits(Server *s, Pipe *const *pp, int n, hipStream_t st, int se
 // Gather of the rows on the segment's miss list from the feature table, on a
 // small grid when the table sits behind the host link (few bytes in flight fill it).
 // One launch for all n pipes; the small grid is then shared between them.
-static int launch_misses(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg, int seg_last) {
+static int launch_misses(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg, int seg_last, int blocks_override = 0) {
   MoveArgs m{};
   m.g.n = n;
   for (int k = 0; k < n; ++k) {
@@ -1113,7 +1113,7 @@ static int launch_misses(Server *s, Pipe *const *pp, int n, hipStream_t st, int 
   m.src_row_bytes = m.dst_row_bytes = m.row_bytes = s->row_bytes;
   m.n_max = s->node_cap[seg_last];
   if (s->feat_loc == LMI_LOC_HOST) {
-    const int blocks = s->miss_blocks > 0 ? s->miss_blocks : s->n_cu;
+    const int blocks = blocks_override > 0 ? blocks_override : s->miss_blocks > 0 ? s->miss_blocks : s->n_cu;
     m.max_blocks = std::max(1, (blocks + n - 1) / n);  // per pipe
     m.unroll = s->miss_unroll;
     m.host_link = 1;
@@ -1137,8 +1137,18 @@ static int launch_misses(Server *s, Pipe *const *pp, int n, hipStream_t st, int 
 //      is done.
 // With 1 and 2 the caller's stream does not wait here: the next call on this pipe,
 // or lmi_batch_wait, joins.  The LRU cache joins at once (its insert copies the rows).
+int launch_misses_early(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg, int seg_last) {
+  hipEvent_t fork = pp[0]->fork_early;
+  LMI_HIP(hipEventRecord(fork, st));
+  LMI_HIP(hipStreamWaitEvent(s->side, fork, 0));
+  if (n > 1 && s->group_miss) return launch_misses(s, pp, n, s->side, seg, seg_last, s->miss_blocks_early);
+  for (int k = 0; k < n; ++k) LMI_TRY(launch_misses(s, pp + k, 1, s->side, seg, seg_last, s->miss_blocks_early));
+  return LMI_OK;  // the join event that launch_gather_group records behind the batch's last misses covers these
+}
+
 int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg, int seg_last, int lru_lists,
-                        bool same_stream) {
+                        bool same_stream, int hit_seg_first) {
+  const int hit_seg = hit_seg_first >= 0 ? hit_seg_first : seg;  // the hits of segments whose misses went ahead
   const bool have_cache = s->cache_kind != LMI_CACHE_NONE;
   int mode = (s->feat_loc == LMI_LOC_HOST && have_cache && !same_stream) ? s->split_miss : 0;
   // The gather kernels carry their own profiling events (prof_kernel_events); a bracket
@@ -1180,7 +1190,7 @@ int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int s
       fork = pp[0]->fork;
       LMI_HIP(hipEventRecord(fork, st));
     }
-    LMI_TRY(launch_hits(s, pp, n, st, seg, seg_last));  // one launch for the group
+    LMI_TRY(launch_hits(s, pp, n, st, hit_seg, seg_last));  // one launch for the group
   }
   if (!fork) {  // one fork for the whole group
     fork = pp[0]->fork;

@@ -102,6 +102,7 @@ struct Pipe {
   int32_t *lru_fill = nullptr;                        // [max_nodes] slot granted to a miss
   int32_t *lru_next = nullptr;                        // [max_nodes] next row in the list of misses of the same LRU set
   hipEvent_t fork = nullptr, join = nullptr;
+  hipEvent_t fork_early = nullptr;  // releases the side stream for the first hops' misses while later hops are still sampled
   // The event that marks the end of this pipe's side-stream work: its own `join`, or that of the
   // first pipe of the group its misses were gathered with (one record and one wait per group: a
   // wait on another queue's event costs a stream about 10 us, fired or not).
@@ -182,6 +183,10 @@ struct Server {
   hipEvent_t side_idle = nullptr;  // recorded behind the last host-link gather issued on the side stream
   bool side_busy = false;
   int protect_hits = 0;            // 1: HBM gathers wait until earlier host-link gathers have drained
+  int miss_blocks_early = 0;       // grid of the host-link gather released by split_lookup (0 = miss_blocks)
+  int split_lookup = 0;            // 1 (always) or 2 (groups of more than one batch): the seeds and the first hop's
+                                   // nodes are looked up before the later hops are sampled and their misses start
+                                   // over the host link then (static / int8 cache, 2+ hops); 0: one lookup at the end
   int early_fork = 2;              // when the side stream is released ahead of the HBM gather instead of behind it:
                                    // 0 never, 1 always, 2 for groups of batches (their host-link gather then starts a
                                    // whole HBM gather earlier, which is what a short run or a first batch waits for)
@@ -287,7 +292,9 @@ int launch_gather_seg(Server *s, Pipe &p, hipStream_t st, int seg, int seg_last,
 // host-link gathers one after another on the side stream.
 // same_stream: hits then misses on `st` whatever the schedule knob says (nothing is left pending).
 int launch_gather_group(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg, int seg_last, int lru_lists,
-                        bool same_stream = false);
+                        bool same_stream = false, int hit_seg_first = -1);
+// the host-link gather of segments [seg, seg_last] released now, ahead of the batch's later hops (split_lookup)
+int launch_misses_early(Server *s, Pipe *const *pp, int n, hipStream_t st, int seg, int seg_last);
 int launch_lru_insert(Server *s, Pipe &p, hipStream_t st, int n_lists);
 int lru_wait_ready(Server *s, hipStream_t st);
 int lru_wait_copied(Server *s, hipStream_t st);  // orders `st` behind the last LRU insertion

@@ -202,9 +202,12 @@ def test_dedup_table_epochs_wrap(lmi, oracle, epochs):
 
 @pytest.mark.parametrize("cache", ["static", "int8", "none"])
 @pytest.mark.parametrize("group,fanout", [(2, [25, 10]), (3, [6, 4, 3]), (4, [64, 2]), (8, [5])])
-def test_groups_of_batches_share_their_launches(lmi, oracle, group, fanout, cache):
+@pytest.mark.parametrize("split_lookup", [0, 2])
+def test_groups_of_batches_share_their_launches(lmi, oracle, group, fanout, cache, split_lookup):
     """lmi_run_group: several mini-batches, each in its own pipe, go through the same kernel
-    launches; every one of them must come out as if it had been run alone."""
+    launches; every one of them must come out as if it had been run alone.  split_lookup: with two hops
+    or more and a cache, the seeds and the first hop's nodes are looked up, and their misses fetched,
+    before the later hops are sampled (no difference for one hop or without a cache)."""
     rng = np.random.default_rng(group * 10 + len(fanout))
     n_nodes, batch, dim = 5000, 150, 16
     indptr, indices = random_graph(rng, n_nodes, 15, hubs=5, hub_deg=600)
@@ -218,6 +221,7 @@ def test_groups_of_batches_share_their_launches(lmi, oracle, group, fanout, cach
             srv.tune("protect_hits", 1)   # HBM gathers held back until earlier host-link gathers have drained
         if group == 4:
             srv.tune("group_miss", 0)     # one host-link gather launch per batch instead of one per group
+        srv.tune("split_lookup", split_lookup)
         srv.load_graph(indptr, indices)
         srv.attach_features(feats)
         srv.load_idset(lmi.MODE_TRAIN, train)
@@ -1039,7 +1043,7 @@ def test_random_groups_sweep(lmi, oracle, case):
     try:
         for key, vals in (("group_miss", [0, 1]), ("protect_hits", [0, 1]), ("fuse_count", [0, 1]),
                           ("table_epochs", [0, 2, 1 << 30]), ("miss_blocks", [1, 8, 32]), ("split_miss", [0, 1, 2]),
-                          ("early_fork", [0, 1])):
+                          ("early_fork", [0, 1]), ("split_lookup", [0, 1, 2]), ("miss_blocks_early", [0, 1, 16])):
             srv.tune(key, int(rng.choice(vals)))
         srv.load_graph(indptr, indices)
         srv.attach_features(feats)
@@ -1077,14 +1081,16 @@ def test_random_groups_sweep(lmi, oracle, case):
 
 @pytest.mark.parametrize("early_fork", [0, 1, 2])
 @pytest.mark.parametrize("streams", [1, 2])
-def test_groups_that_reuse_pipes_wait_for_the_host_link_gather_before(lmi, oracle, streams, early_fork):
+@pytest.mark.parametrize("split_lookup", [0, 1])
+def test_groups_that_reuse_pipes_wait_for_the_host_link_gather_before(lmi, oracle, streams, early_fork, split_lookup):
     """Groups issued back to back on overlapping sets of pipes, nothing fetched in between: a pipe's
     next batch may only start once the side stream has finished the host-link gather of the one
     before (one event per group marks that, whichever pipes of it are reused first).  The host-link
     gather is slowed to one block and most rows miss, so a batch that started early would be
     overwritten by the rows of its predecessor.  With the side stream released ahead of the HBM gather
     (early_fork) that event does not cover the HBM gather: a pipe taken over by the other caller's
-    stream is ordered behind the stream that carried its batch."""
+    stream is ordered behind the stream that carried its batch.  With split lookups a batch has two host-link
+    gathers, the first released before its second hop is sampled; the one event still marks the end of both."""
     rng = np.random.default_rng(77 + streams)
     n_nodes, batch, dim, fanout, pipes = 40_000, 500, 128, [10, 5], 8
     indptr, indices = random_graph(rng, n_nodes, 12, hubs=4, hub_deg=2000)
@@ -1094,6 +1100,7 @@ def test_groups_that_reuse_pipes_wait_for_the_host_link_gather_before(lmi, oracl
     try:
         srv.tune("miss_blocks", 1)
         srv.tune("early_fork", early_fork)
+        srv.tune("split_lookup", split_lookup)
         srv.load_graph(indptr, indices)
         srv.attach_features(feats)
         srv.build_static_cache(n_nodes // 10, lmi.TABLE_RANK)

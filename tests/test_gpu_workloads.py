@@ -180,11 +180,13 @@ def test_paper100m_hot_set_at_full_size(lmi, oracle, paper100m_inputs):
 # (pipes, tuning, sizes of the groups issued back to back with nothing read in between): the last is what
 # bench.py issues for the driver's `--steps 20` -- 7, 7, 6 on 16 pipes, batch i in pipe i % 16, so the
 # third group takes over pipes of the first while the first group's host-link gather may still run
-GROUPED = [(8, {}, [4]), (16, {"miss_blocks": 40}, [8, 8]), (16, {"miss_blocks": 40}, [7, 7, 6]),
+GROUPED = [(8, {}, [4]), (16, {"miss_blocks": 40}, [8, 8]), (16, {"miss_blocks": 48, "split_lookup": 2}, [7, 7, 6]),
+           (16, {"miss_blocks": 48, "split_lookup": 2}, [8, 8, 8]),
            (16, {"miss_blocks": 40, "early_fork": 0}, [8, 8, 8])]
 
 
-@pytest.mark.parametrize("pipes,tune,sizes", GROUPED, ids=["4on8", "8+8on16", "7+7+6on16", "8+8+8on16-latefork"])
+@pytest.mark.parametrize("pipes,tune,sizes", GROUPED,
+                         ids=["4on8", "8+8on16", "7+7+6on16-split", "8+8+8on16-split", "8+8+8on16-latefork"])
 def test_paper100m_at_full_size_in_groups(lmi, oracle, paper100m_inputs, pipes, tune, sizes):
     """The benchmark's own configuration at its real size (111 M nodes, 38 GB cache), issued exactly as
     bench.py's timed region issues it -- lmi_run_group, the same group sizes, pipes and tuning, every
