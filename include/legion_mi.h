@@ -336,7 +336,7 @@ int lmi_bench_row_stream(int64_t rows, int64_t src_pitch, int read_bytes, int wr
  * visit; more = blocks that find nothing to do and leave, as a grid sized for the worst case of a
  * batch holds; fewer = blocks that loop), every_lane_loads != 0 (lanes without a unit in a block's
  * last pass issue their loads anyway and only skip the store).  Refused: more than 4096 rows per
- * visit, more than 2^22 blocks, rows of more than 2^16 units, more than 2^31 - 1 rows. */
+ * visit, more than 2^24 blocks, rows of more than 2^16 units, more than 2^31 - 1 rows. */
 int lmi_bench_row_stream_shape(int64_t rows, int64_t src_pitch, int read_bytes, int write_bytes, int64_t table_rows,
                                int rows_per_block, int grid_blocks, int every_lane_loads, int repeats,
                                int launch_by_launch, double *ms_per_launch);

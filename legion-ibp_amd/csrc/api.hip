@@ -1413,8 +1413,8 @@ int lmi_bench_row_stream_shape(int64_t rows, int64_t src_pitch, int read_bytes, 
                                int rows_per_block, int grid_blocks, int every_lane_loads, int repeats,
                                int launch_by_launch, double *ms_per_launch) {
   if (!ms_per_launch || repeats < 1 || rows < 1 || rows > INT32_MAX || table_rows < 2) LMI_FAIL(LMI_ERR_ARG, "bad argument");
-  if (rows_per_block < 0 || rows_per_block > 4096 || grid_blocks < 0 || grid_blocks > (1 << 22))
-    LMI_FAIL(LMI_ERR_ARG, "a block visit takes 1..4096 rows and a grid has at most 2^22 blocks (0 = chosen here)");
+  if (rows_per_block < 0 || rows_per_block > 4096 || grid_blocks < 0 || grid_blocks > (1 << 24))
+    LMI_FAIL(LMI_ERR_ARG, "a block visit takes 1..4096 rows and a grid has at most 2^24 blocks (0 = chosen here)");
   const int shape = read_bytes * 100 + write_bytes;
   if (shape != 416 && shape != 816 && shape != 1616) LMI_FAIL(LMI_ERR_ARG, "read : write bytes per unit must be 4:16, 8:16 or 16:16");
   if (src_pitch < read_bytes || src_pitch % 4 != 0) LMI_FAIL(LMI_ERR_ARG, "rows are a multiple of 4 bytes and hold a unit");
