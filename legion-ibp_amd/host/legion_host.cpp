@@ -361,6 +361,21 @@ class GPUServer : public Server {
     params_.in_memory = in_memory_mode != 0;
     params_.dyn_cache = dyn_cache;
     params_.fused = std::getenv("LEGION_MI_OPERATOR_TABLE") == nullptr;
+    // LEGION_MI_TUNE="key=value,key=value": the library's tuning keys (lmi_tune) for deployments that know
+    // their workload, e.g. "split_lookup=2,miss_blocks=48"; none changes a result
+    if (const char *tune = std::getenv("LEGION_MI_TUNE")) {
+      std::istringstream list(tune);
+      std::string item;
+      while (std::getline(list, item, ',')) {
+        const size_t eq = item.find('=');
+        if (item.empty()) continue;
+        if (eq == std::string::npos || eq == 0 || eq + 1 >= item.size()) {
+          std::fprintf(stderr, "LEGION_MI_TUNE: '%s' is not key=value\n", item.c_str());
+          std::exit(EXIT_FAILURE);
+        }
+        LMI_MUST(lmi_tune(h_, item.substr(0, eq).c_str(), std::atoll(item.c_str() + eq + 1)));
+      }
+    }
     runner_->Initialize(&params_);
     std::cout << "Storage Initialized\n";
   }

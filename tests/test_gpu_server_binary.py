@@ -57,7 +57,8 @@ def read_dump(path, dim, dtype=np.float32):
     (0, False, False, "f32", None), (0, False, False, "f32", 1), (0, False, False, "f32", 2),
     (0, True, False, "f32", None), (1, False, False, "f32", None), (1, True, False, "f32", None),
     (8, False, False, "f32", None), (0, True, True, "f32", None), (0, False, True, "f32", None),
-    (0, False, False, "f16", None), (1, False, False, "f16", None), (8, False, False, "f16", None)])   # fp16 `features` file
+    (0, False, False, "f16", None), (1, False, False, "f16", None), (8, False, False, "f16", None),   # fp16 `features` file
+    (0, False, False, "f32", "tuned"), (8, False, False, "f16", "tuned")])   # knobs through LEGION_MI_TUNE: split lookups
 def test_sampling_server_binary(tmp_path, oracle, dyn_cache, table_mode, presample, dtype, group):
     assert os.path.exists(BIN), "build the host shim first (make -C legion-ibp_amd)"
     rng = np.random.default_rng(dyn_cache * 2 + table_mode)
@@ -72,7 +73,9 @@ def test_sampling_server_binary(tmp_path, oracle, dyn_cache, table_mode, presamp
     dump = tmp_path / "dump"
     dump.mkdir()
     env = dict(os.environ, LEGION_MI_DUMP=str(dump), LEGION_MI_DUMP_BATCHES="9")
-    if group:
+    if group == "tuned":
+        env["LEGION_MI_TUNE"] = "split_lookup=2,miss_blocks=16,miss_blocks_early=8"
+    elif group:
         env["LEGION_MI_GROUP"] = str(group)
     if dtype == "f16":
         env["LEGION_MI_FEAT_DTYPE"] = "f16"
