@@ -189,7 +189,7 @@ def test_server_run_reaches_the_rate_of_the_grouped_path(products_on_disk):
     line = json.loads(ref.stdout.strip().splitlines()[-1])
     print("Server::Run %.0f batches/s (one batch per RunOnce: %.0f); bench.py --workload products %.0f batches/s" % (
         served, one_by_one, line["value"]))
-    assert served >= 0.85 * line["value"], (served, line["value"])
+    assert served >= 0.90 * line["value"], (served, line["value"])   # 0.96 measured, box after box
     assert served > one_by_one
 
 
